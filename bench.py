@@ -1,0 +1,208 @@
+#!/usr/bin/env python3
+"""Benchmark of the N-input reduce on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one call of mi_ccl_comp_reduce_n over one batch of synthetic input that is already resident in
+HBM.  Default workload: the Llama-3-8B-sized gradient share, 8 input buffers of 1,003,782,144 bf16 elements
+(N(0, 1e-3) cast to bf16), fp32 accumulation in input order, one round-to-nearest-even narrowing
+(ccl_comp_batch_reduce keep-precision semantics under CCL_BF16=avx512bf).  Prints ONE JSON line.
+
+Algorithmic bytes of a launch = (N + 1) x count x sizeof(element): N reads and one write.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0      # MI355X published HBM3E peak
+
+WORKLOADS = {
+    # name: (dtype name, n inputs, elements per buffer, in_place, lp keep precision, value std / range)
+    "c5_bf16": dict(dtype="bfloat16", n=8, count=1_003_782_144, keep=True, sets=1,
+                    desc="8-input bf16 sum, 1,003,782,144 elements per buffer (Llama-3-8B gradient share / 8), "
+                         "fp32 accumulate in input order, RNE once"),
+    "c5_fp32": dict(dtype="float32", n=4, count=1_003_782_144, keep=False, sets=1,
+                    desc="4-input fp32 sum, 1,003,782,144 elements per buffer"),
+    "c2_bf16": dict(dtype="bfloat16", n=8, count=33_554_432, keep=True, sets=6,
+                    desc="8-input bf16 sum, 33,554,432 elements per buffer (64 MiB), rotating over 6 buffer sets"),
+    "c1_fp32": dict(dtype="float32", n=2, count=16_777_216, keep=False, sets=8, in_place=True,
+                    desc="2-input in-place fp32 sum, 16,777,216 elements per buffer (64 MiB), rotating over 8 buffer sets"),
+}
+
+# HBM traffic per launch of the default workload measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (see profiles/); None until measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def make_buffers(torch, w, seed):
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    count, n = w["count"], w["n"]
+    bufs = []
+    for _ in range(n):
+        if w["dtype"] == "bfloat16":
+            t = torch.empty(count, dtype=torch.bfloat16, device="cuda")
+            t.normal_(0.0, 1e-3 if count > 100_000_000 else 1.0, generator=g)   # fp32 normal, RNE cast to bf16
+        else:
+            t = torch.empty(count, dtype=torch.float32, device="cuda")
+            if w["n"] == 2:
+                t.uniform_(-1.0, 1.0, generator=g)
+            else:
+                t.normal_(0.0, 1e-3, generator=g)
+        bufs.append(t)
+    return bufs
+
+
+def cpu_baseline(torch, comp, w, bufs, sample_elems):
+    """The oracle timed on the host cores over the first sample_elems elements of the same buffers."""
+    import numpy as np
+    import oracle_lib as O
+    dt = O.BFLOAT16 if w["dtype"] == "bfloat16" else O.FLOAT32
+    np_t = np.uint16 if dt == O.BFLOAT16 else np.float32
+    esz = 2 if dt == O.BFLOAT16 else 4
+    s = min(sample_elems, w["count"])
+    s -= s % 16
+    host = []
+    for b in bufs:
+        v = b[:s].view(torch.int16) if dt == O.BFLOAT16 else b[:s]
+        host.append(v.cpu().numpy().view(np_t))
+    algo_bytes = (w["n"] + 1) * s * esz
+    # (i) one thread, the reference's own pass structure: slices of one buffer, widen to tmp / fp32 add into
+    # acc / narrow (ccl_comp_batch_reduce keep-precision), or the pairwise chain for plain types
+    buf = np.concatenate(host)
+    offs = np.arange(w["n"], dtype=np.uint64) * np.uint64(s)
+    tmp = np.empty(s, np.float32)
+    acc = np.empty(s, np.float32)
+    L = O.lib()
+    t0 = time.perf_counter()
+    rc = L.orc_comp_batch_reduce(buf.ctypes.data, offs.ctypes.data, w["n"], s, buf.ctypes.data, dt, O.SUM,
+                                 1 if w["keep"] else 0, tmp.ctypes.data, acc.ctypes.data, O.BF16_AVX512BF,
+                                 O.FP16_AVX512F)
+    t1 = time.perf_counter()
+    assert rc == 0
+    one = algo_bytes / (t1 - t0) / 1e9
+    ref_out = buf[:s].copy()
+    del buf, tmp, acc
+    # (ii) W threads on disjoint count/W partitions (what CCL_WORKER_COUNT=W does), fused single pass
+    W = min(16, os.cpu_count() or 1)
+    t0 = time.perf_counter()
+    out = O.reduce_n(host, dt, O.SUM, keep=1 if w["keep"] else 0, quirk_tail=1, threads=W)
+    t1 = time.perf_counter()
+    multi = algo_bytes / (t1 - t0) / 1e9
+    assert (out.view(np.uint8) == ref_out.view(np.uint8)).all(), "oracle forms disagree"
+    return dict(value=round(one, 3), unit="GB/s", cores=1, kind="port",
+                sample=f"first {s} elements of each of the {w['n']} buffers of the same workload "
+                       f"({algo_bytes / 1e9:.2f} GB algorithmic), reference pass structure "
+                       f"(ccl_comp_batch_reduce: widen / fp32 add / narrow), 1 thread = CCL_WORKER_COUNT=1; "
+                       f"{W}-thread partitioned single-pass port: {multi:.2f} GB/s",
+                multi_thread=dict(value=round(multi, 3), cores=W)), out, s
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c5_bf16", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-sample", type=int, default=1 << 28, help="elements per buffer for the CPU baseline")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--set", action="append", default=[], metavar="NAME=VALUE", help="launch knob (mi_ccl_set_param)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the reduce is elementwise and runs on one GPU's share of the data; "
+                 "--gpus must be 1")
+
+    import torch
+    import oneccl_amd.comp as comp
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    comp.lib()      # raises when the HIP library is missing
+    for kv in args.set:
+        k, v = kv.split("=")
+        comp.set_param(k, int(v))
+
+    w = WORKLOADS[args.workload]
+    dt = comp.BFLOAT16 if w["dtype"] == "bfloat16" else comp.FLOAT32
+    esz = 2 if dt == comp.BFLOAT16 else 4
+    lp = comp.LP_KEEP_PRECISION if w["keep"] else comp.LP_PAIRWISE
+    n, count = w["n"], w["count"]
+    sets = [make_buffers(torch, w, 1234 + i) for i in range(w["sets"])]
+    outs = [s[0] if w.get("in_place") else torch.empty_like(s[0]) for s in sets]
+    algo_bytes = (n + 1) * count * esz
+    stream = torch.cuda.current_stream()
+
+    def step(i):
+        s = sets[i % len(sets)]
+        comp.comp_reduce_n(dt, comp.SUM, s, outs[i % len(sets)], count, lp_mode=lp, stream=stream)
+
+    # parity outside the timed region: GPU result of set 0 against the oracle on a sample
+    base = None
+    if not args.no_cpu_baseline:
+        snapshot = [b.clone() for b in sets[0]] if w.get("in_place") else sets[0]
+        base, want, s_elems = cpu_baseline(torch, comp, w, snapshot, args.cpu_sample)
+        step(0)
+        torch.cuda.synchronize()
+        import numpy as np
+        got = outs[0][:s_elems]
+        got = (got.view(torch.int16) if dt == comp.BFLOAT16 else got).cpu().numpy()
+        same = (got.view(np.uint8) == want.view(np.uint8)).all()
+        if not same:
+            sys.exit("GPU result differs from the oracle on the CPU-baseline sample")
+        if w.get("in_place"):
+            for b, c in zip(sets[0], snapshot):
+                b.copy_(c)
+        del snapshot
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record(stream)
+    for i in range(args.steps):
+        step(i)
+    ev1.record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+
+    ms_per_step = (t1 - t0) / args.steps * 1e3
+    kernel_ms = ev0.elapsed_time(ev1) / args.steps
+    value = algo_bytes / (ms_per_step * 1e-3) / 1e9
+    achieved = algo_bytes / (kernel_ms * 1e-3) / 1e9
+    out = {
+        "metric": "N-way reduce GB/s (bf16 sum, 8 inputs x 2 GiB)" if args.workload == "c5_bf16"
+                  else f"N-way reduce GB/s ({args.workload})",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if dt == comp.BFLOAT16 else "f32",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "description": w["desc"], "inputs": n, "elements_per_buffer": count,
+                   "bytes_per_buffer": count * esz, "algorithmic_bytes_per_step": algo_bytes,
+                   "lp_mode": "fp32 accumulate, RNE once" if w["keep"] else "native",
+                   "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+                   "parity": "bit-exact vs oracle on the CPU-baseline sample" if base else "not checked in this run"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel_ms": round(kernel_ms, 4)},
+        "cpu_baseline": base,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

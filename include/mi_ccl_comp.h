@@ -1,0 +1,172 @@
+/*
+ * mi_ccl_comp.h -- C ABI of the MI355X reduction engine (libmi_ccl_comp.so).
+ *
+ * Drop-in boundary for oneCCL's data-parallel reduction path.  oneCCL has no public plugin ABI for
+ * reductions; its boundary is the internal operator surface of src/comp/comp.hpp:23-51 plus the
+ * device-kernel launch sites under src/sched/entry/ze/.  Every entry point below names the reference
+ * interface it replaces.
+ *
+ * Conventions
+ *   - All buffer arguments are DEVICE pointers (HIP device memory); the library never dereferences
+ *     them on the host, never allocates or frees device memory in a reduce/copy/convert call, and keeps
+ *     no pointer after the call returns (fusion plans own one small device table, allocated at plan
+ *     creation).  Pointers must be aligned to the element size.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls are asynchronous:
+ *     they enqueue kernels on `stream` and return.
+ *   - dtype / op use the numbering of ccl::datatype / ccl::reduction
+ *     (include/oneapi/ccl/types.hpp:41-69).
+ *   - Return value: a ccl::status number (src/internal_types.hpp:29-37): 0 success, 1 out_of_resource,
+ *     2 invalid_arguments, 3 runtime_error.  Nothing here throws or terminates the process; count == 0
+ *     succeeds without touching any pointer (comp.cpp:132-134, :61-63).
+ *   - Results are bit-identical to the reference CPU reduction on the same inputs (integers wrap;
+ *     one IEEE operation per pair in input order, no FMA; min/max return the same operand as the
+ *     reference on ties and NaNs).  The payload and sign of a NaN produced by sum/prod are unspecified.
+ */
+#ifndef MI_CCL_COMP_H
+#define MI_CCL_COMP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ccl::datatype, include/oneapi/ccl/types.hpp:52-69 */
+enum mi_ccl_datatype {
+    MI_CCL_INT8 = 0, MI_CCL_UINT8, MI_CCL_INT16, MI_CCL_UINT16, MI_CCL_INT32, MI_CCL_UINT32,
+    MI_CCL_INT64, MI_CCL_UINT64, MI_CCL_FLOAT16 = 8, MI_CCL_FLOAT32, MI_CCL_FLOAT64, MI_CCL_BFLOAT16 = 11,
+    MI_CCL_DATATYPE_LAST
+};
+
+/* ccl::reduction, include/oneapi/ccl/types.hpp:41-47 (custom is handled above this ABI, on the host) */
+enum mi_ccl_reduction { MI_CCL_SUM = 0, MI_CCL_PROD, MI_CCL_MIN, MI_CCL_MAX, MI_CCL_CUSTOM };
+
+/* ccl::status, src/internal_types.hpp:29-37 */
+enum mi_ccl_status {
+    MI_CCL_SUCCESS = 0, MI_CCL_OUT_OF_RESOURCE = 1, MI_CCL_INVALID_ARGUMENTS = 2, MI_CCL_RUNTIME_ERROR = 3
+};
+
+/* ccl_bf16_impl_type, src/comp/bf16/bf16_utils.hpp:26 -- which of the reference's three bf16
+ * implementations the results must equal (the reference picks one through CCL_BF16, env.cpp:711-713):
+ *   scalar   narrow by truncation, min/max with std:: semantics (ties/NaN return `in`)
+ *   avx512f  narrow by truncation, min/max return `inout` on ties/NaN
+ *   avx512bf narrow with round-to-nearest-even, fp32 denormals to zero, NaN quieted (VCVTNEPS2BF16);
+ *            min/max as avx512f */
+enum mi_ccl_bf16_impl { MI_CCL_BF16_SCALAR = 0, MI_CCL_BF16_AVX512F = 1, MI_CCL_BF16_AVX512BF = 2 };
+
+/* How 16-bit floating types are carried through an N-input reduce (flags, OR them):
+ *   MI_CCL_LP_PAIRWISE        round to the 16-bit type after every pair: a chain of ccl_comp_reduce calls
+ *                             (comp.cpp:236-245; the only mode the reference has for float16)
+ *   MI_CCL_LP_KEEP_PRECISION  bfloat16 only: widen, accumulate in fp32 in input order, narrow once
+ *                             (ccl_comp_batch_reduce with bf16_keep_precision_mode = 1, comp.cpp:214-234)
+ *   MI_CCL_LP_TAIL_QUIRK      with KEEP_PRECISION under avx512f/avx512bf: narrow the last count % 16 elements
+ *                             by truncation, as ccl_convert_fp32_to_bf16_arrays does (bf16.cpp:134-148) */
+enum mi_ccl_lp_mode { MI_CCL_LP_PAIRWISE = 0, MI_CCL_LP_KEEP_PRECISION = 1, MI_CCL_LP_TAIL_QUIRK = 2 };
+
+/* ---- tables ------------------------------------------------------------------------------------ */
+
+/* Element size in bytes, 0 for an unknown dtype.  Replaces ccl_datatype::size(), datatype.cpp:79-91. */
+size_t mi_ccl_datatype_size(int dtype);
+/* "int8" ... "bfloat16", "" for an unknown dtype.  Replaces the name table of datatype.cpp:94-106. */
+const char* mi_ccl_datatype_name(int dtype);
+/* "sum", "prod", "min", "max", "custom", "unknown".  Replaces ccl_reduction_to_str, comp.cpp:251-260. */
+const char* mi_ccl_reduction_to_str(int op);
+/* Text for a status code. */
+const char* mi_ccl_status_str(int status);
+/* Name the reference gives the matching device kernel: "<kernel>_<dtype-name>_<op>"
+ * (ze_primitives.cpp:152-161); written into buf (NUL terminated), returns the status. */
+int mi_ccl_kernel_name(const char* kernel, int dtype, int op, char* buf, size_t buf_len);
+
+/* ---- pairwise, in place ------------------------------------------------------------------------- */
+
+/* inout[i] = inout[i] OP in[i] for i < count.  Replaces ccl_comp_reduce / ccl_comp_reduce_regular
+ * (src/comp/comp.cpp:76-200) and reduce_local_inplace_kernel (src/kernels/kernels.cl:236-246,
+ * launched from ze_reduce_local_entry.cpp:40-58).  in and inout must be identical or disjoint. */
+int mi_ccl_comp_reduce(int dtype, int op, const void* in, size_t count, void* inout, int bf16_impl,
+                       void* stream);
+
+/* Replaces ccl_bf16_reduce (src/comp/bf16/bf16.cpp:87-110) and ccl_fp16_reduce
+ * (src/comp/fp16/fp16.cpp:41-53; results of the f16c / avx512f implementations). */
+int mi_ccl_bf16_reduce(const void* in, size_t count, void* inout, int op, int bf16_impl, void* stream);
+int mi_ccl_fp16_reduce(const void* in, size_t count, void* inout, int op, void* stream);
+
+/* ---- N inputs ----------------------------------------------------------------------------------- */
+
+/* dst[i] = (((srcs[0][i] OP srcs[1][i]) OP srcs[2][i]) ... OP srcs[n-1][i]): own buffer first, peers in
+ * argument order, one pass over memory.  srcs is a HOST array of n device pointers (1 <= n <= 64).
+ * dst may equal any srcs[j].  Replaces reduce_monolithic_kernel_{1..7}, local_reduce_kernel_{1..7},
+ * reduce_single_local_inplace_kernel and reduce_local_outofplace_kernel (src/kernels/kernels.cl:179-421;
+ * launch sites ze_a2a_reduce_scatter_entry.cpp:48-136, ze_a2a_pipeline_reduce_scatter_entry.cpp:195-228)
+ * and, with slice pointers, ccl_comp_batch_reduce (src/comp/comp.cpp:202-249). */
+int mi_ccl_comp_reduce_n(int dtype, int op, const void* const* srcs, int n, void* dst, size_t count,
+                         int lp_mode, int bf16_impl, void* stream);
+
+/* Slice form of the same: slice i starts at in_buf + offsets[i] elements (offsets: HOST array); inout is
+ * slice 0 and receives the result.  Replaces ccl_comp_batch_reduce (src/comp/comp.cpp:202-249); the tmp and
+ * acc scratch arrays of the reference are not needed.  keep_precision != 0 requires dtype bfloat16 and
+ * reproduces the reference bit for bit, including the truncated tail (MI_CCL_LP_TAIL_QUIRK). */
+int mi_ccl_comp_batch_reduce(const void* in_buf, const size_t* offsets, size_t n_offsets, size_t count,
+                             void* inout, int dtype, int op, int bf16_keep_precision_mode, int bf16_impl,
+                             void* stream);
+
+/* ---- copies and converters ---------------------------------------------------------------------- */
+
+/* out[0..bytes) = in[0..bytes).  Replaces ccl_comp_copy (src/comp/comp.cpp:60-74) and the copy_entry body
+ * (src/sched/entry/copy/copy_entry.cpp:201-207).  use_nontemporal selects streaming stores, as
+ * ccl::memcpy_nontemporal does (src/common/utils/memcpy.cpp:49-). */
+int mi_ccl_comp_copy(const void* in, void* out, size_t bytes, int use_nontemporal, void* stream);
+
+/* Replace ccl_convert_fp32_to_bf16_arrays / ccl_convert_bf16_to_fp32_arrays (bf16.cpp:130-169), tail
+ * truncation included. */
+int mi_ccl_convert_fp32_to_bf16_arrays(const void* fp32_buf, void* bf16_buf, size_t count, int bf16_impl,
+                                       void* stream);
+int mi_ccl_convert_bf16_to_fp32_arrays(const void* bf16_buf, void* fp32_buf, size_t count, void* stream);
+
+/* ---- fusion buffer ------------------------------------------------------------------------------ */
+
+/* Byte offset of each of k tensors in a fusion buffer: running offset in queue order, every start
+ * rounded up to `align` bytes (align = 1 is the reference's tight layout, fusion.cpp:283-316).  Host
+ * arithmetic only.  *total_bytes = end of the last tensor. */
+int mi_ccl_fusion_offsets(const size_t* counts, size_t k, size_t dtype_size, size_t align,
+                          size_t* byte_offsets, size_t* total_bytes);
+
+typedef struct mi_ccl_fusion_plan mi_ccl_fusion_plan;
+
+/* A plan fixes (counts, dtype, alignment) of one fused group -- what ccl_fusion_manager::build_sched
+ * derives from its exec_queue (fusion.cpp:145-376) and caches with the fused sched (:206-237).  Creating a
+ * plan allocates its device-side work table once; destroy frees it. */
+int mi_ccl_fusion_plan_create(const size_t* counts, size_t k, int dtype, size_t align,
+                              mi_ccl_fusion_plan** plan);
+int mi_ccl_fusion_plan_destroy(mi_ccl_fusion_plan* plan);
+size_t mi_ccl_fusion_plan_bytes(const mi_ccl_fusion_plan* plan);            /* fused buffer size */
+size_t mi_ccl_fusion_plan_offset(const mi_ccl_fusion_plan* plan, size_t i); /* byte offset of tensor i */
+
+/* tensors: HOST array of k device pointers.  pack copies every tensor to its offset in fusion_buf in one
+ * launch (replaces the pack copy_entry list, fusion.cpp:283-316); unpack copies them back (replaces
+ * fusion.cpp:323-362).  Padding bytes between tensors are not written by pack. */
+int mi_ccl_fusion_pack(mi_ccl_fusion_plan* plan, const void* const* tensors, void* fusion_buf, void* stream);
+int mi_ccl_fusion_unpack(mi_ccl_fusion_plan* plan, const void* fusion_buf, void* const* tensors,
+                         void* stream);
+
+/* The whole pack -> N-input reduce -> unpack sequence in one pass over memory:
+ * out_tensors[t][i] = own_tensors[t][i] OP peers[0][off_t + i] OP ... OP peers[n_peers-1][off_t + i],
+ * where every peer is a fusion buffer with this plan's layout.  Same bits as the three-step sequence. */
+int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* own_tensors,
+                         const void* const* peers, int n_peers, void* const* out_tensors, int lp_mode,
+                         int bf16_impl, void* stream);
+
+/* ---- launch tuning ------------------------------------------------------------------------------- */
+
+/* Launch-shape knobs, the counterpart of CCL_KERNEL_GROUP_SIZE / CCL_KERNEL_MEM_ALIGN
+ * (src/common/env/env.cpp:251-253).  Names: "waves_per_cu" (resident blocks per CU the grid is sized
+ * for), "max_blocks" (cap on the grid; 0 = no cap), "xcd_chunked" (0/1: give each of the 8 XCDs one
+ * contiguous share of the buffer), "variant" (kernel variant selector, 0 = default).
+ * Returns invalid_arguments for an unknown name or out-of-range value. */
+int mi_ccl_set_param(const char* name, long value);
+long mi_ccl_get_param(const char* name);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_CCL_COMP_H */

@@ -1,0 +1,275 @@
+// Fusion plans and the extern "C" fusion entry points of libmi_ccl_comp.so.
+#include <hip/hip_runtime.h>
+
+#include <new>
+#include <vector>
+
+#include "../../include/mi_ccl_comp.h"
+#include "fusion_kernels.hpp"
+
+namespace mi {
+
+Tuning current_tuning();
+
+#define MI_DECLARE_FUSION(TR) extern template hipError_t launch_fusion_reduce<TR>(const FusionLaunchArgs&)
+MI_DECLARE_FUSION(I8Traits);
+MI_DECLARE_FUSION(U8Traits);
+MI_DECLARE_FUSION(I16Traits);
+MI_DECLARE_FUSION(U16Traits);
+MI_DECLARE_FUSION(I32Traits);
+MI_DECLARE_FUSION(U32Traits);
+MI_DECLARE_FUSION(I64Traits);
+MI_DECLARE_FUSION(U64Traits);
+MI_DECLARE_FUSION(F32Traits);
+MI_DECLARE_FUSION(F64Traits);
+MI_DECLARE_FUSION(Fp16PairwiseTraits);
+typedef Bf16PairwiseTraits<false, false> Bf16PairScalar;
+typedef Bf16PairwiseTraits<false, true> Bf16PairAvx512f;
+typedef Bf16PairwiseTraits<true, true> Bf16PairAvx512bf;
+MI_DECLARE_FUSION(Bf16PairScalar);
+MI_DECLARE_FUSION(Bf16PairAvx512f);
+MI_DECLARE_FUSION(Bf16PairAvx512bf);
+MI_DECLARE_FUSION(Bf16KeepTraits<false>);
+MI_DECLARE_FUSION(Bf16KeepTraits<true>);
+
+static int fusion_status_of(hipError_t e) {
+    if (e == hipSuccess)
+        return MI_CCL_SUCCESS;
+    if (e == hipErrorOutOfMemory)
+        return MI_CCL_OUT_OF_RESOURCE;
+    if (e == hipErrorInvalidValue)
+        return MI_CCL_INVALID_ARGUMENTS;
+    return MI_CCL_RUNTIME_ERROR;
+}
+
+static size_t fusion_dtype_size(int dtype) {
+    static const size_t sz[MI_CCL_DATATYPE_LAST] = { 1, 1, 2, 2, 4, 4, 8, 8, 2, 4, 8, 2 };
+    return (dtype >= 0 && dtype < MI_CCL_DATATYPE_LAST) ? sz[dtype] : 0;
+}
+
+// to_fusion != 0: tensors -> fusion buffer (pack); else fusion buffer -> tensors (unpack)
+__global__ void __launch_bounds__(kBlock)
+fusion_copy_kernel(FusionPtrs tensors, unsigned char* fusion_buf, const uint64_t* off, const uint64_t* bytes,
+                   const FusionItem* items, uint32_t nitems, uint32_t t0, int to_fusion) {
+    for (uint32_t it = blockIdx.x; it < nitems; it += gridDim.x) {
+        const FusionItem w = items[it];
+        const uint64_t lo = (uint64_t)w.c * kFusionChunk;
+        const uint64_t left = bytes[w.t] - lo;
+        const uint32_t n = left < kFusionChunk ? (uint32_t)left : kFusionChunk;
+        unsigned char* tp = (unsigned char*)tensors.p[w.t - t0] + lo;
+        unsigned char* fp = fusion_buf + off[w.t] + lo;
+        if (to_fusion)
+            copy_span(tp, fp, n);
+        else
+            copy_span(fp, tp, n);
+    }
+}
+
+}  // namespace mi
+
+using namespace mi;
+
+struct mi_ccl_fusion_plan {
+    size_t k = 0;
+    int dtype = 0;
+    size_t esz = 0;
+    size_t align = 1;
+    size_t total_bytes = 0;
+    std::vector<size_t> counts;
+    std::vector<size_t> offsets;           // bytes
+    std::vector<uint64_t> item_begin;      // k + 1
+    void* d_table = nullptr;               // [off: k x u64][bytes: k x u64][items]
+    const uint64_t* d_off = nullptr;
+    const uint64_t* d_bytes = nullptr;
+    const FusionItem* d_items = nullptr;
+};
+
+extern "C" {
+
+int mi_ccl_fusion_offsets(const size_t* counts, size_t k, size_t dtype_size, size_t align, size_t* byte_offsets,
+                          size_t* total_bytes) {
+    if (dtype_size == 0 || align == 0 || (align & (align - 1)) != 0 || (k && (!counts || !byte_offsets)))
+        return MI_CCL_INVALID_ARGUMENTS;
+    size_t end = 0;
+    for (size_t i = 0; i < k; i++) {
+        size_t off = (end + align - 1) & ~(align - 1);
+        byte_offsets[i] = off;
+        end = off + counts[i] * dtype_size;
+    }
+    if (total_bytes)
+        *total_bytes = end;
+    return MI_CCL_SUCCESS;
+}
+
+int mi_ccl_fusion_plan_create(const size_t* counts, size_t k, int dtype, size_t align, mi_ccl_fusion_plan** plan) {
+    if (!plan)
+        return MI_CCL_INVALID_ARGUMENTS;
+    *plan = nullptr;
+    const size_t esz = fusion_dtype_size(dtype);
+    if (esz == 0 || k == 0 || !counts || align == 0 || (align & (align - 1)) != 0)
+        return MI_CCL_INVALID_ARGUMENTS;
+    mi_ccl_fusion_plan* p = new (std::nothrow) mi_ccl_fusion_plan;
+    if (!p)
+        return MI_CCL_OUT_OF_RESOURCE;
+    p->k = k;
+    p->dtype = dtype;
+    p->esz = esz;
+    p->align = align;
+    p->counts.assign(counts, counts + k);
+    p->offsets.resize(k);
+    mi_ccl_fusion_offsets(counts, k, esz, align, p->offsets.data(), &p->total_bytes);
+    p->item_begin.resize(k + 1);
+    std::vector<FusionItem> items;
+    for (size_t t = 0; t < k; t++) {
+        p->item_begin[t] = items.size();
+        const uint64_t bytes = (uint64_t)counts[t] * esz;
+        const uint64_t chunks = (bytes + kFusionChunk - 1) / kFusionChunk;
+        if (chunks > 0xffffffffull || t > 0xffffffffull || items.size() + chunks > 0x7fffffffull) {
+            delete p;
+            return MI_CCL_INVALID_ARGUMENTS;
+        }
+        for (uint64_t c = 0; c < chunks; c++) items.push_back(FusionItem{ (uint32_t)t, (uint32_t)c });
+    }
+    p->item_begin[k] = items.size();
+    std::vector<uint64_t> host(2 * k);
+    for (size_t t = 0; t < k; t++) {
+        host[t] = p->offsets[t];
+        host[k + t] = (uint64_t)counts[t] * esz;
+    }
+    const size_t table_bytes = 2 * k * sizeof(uint64_t) + (items.size() ? items.size() : 1) * sizeof(FusionItem);
+    hipError_t e = hipMalloc(&p->d_table, table_bytes);
+    if (e != hipSuccess) {
+        delete p;
+        return fusion_status_of(e);
+    }
+    e = hipMemcpy(p->d_table, host.data(), 2 * k * sizeof(uint64_t), hipMemcpyHostToDevice);
+    if (e == hipSuccess && !items.empty())
+        e = hipMemcpy((char*)p->d_table + 2 * k * sizeof(uint64_t), items.data(), items.size() * sizeof(FusionItem),
+                      hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(p->d_table);
+        delete p;
+        return fusion_status_of(e);
+    }
+    p->d_off = (const uint64_t*)p->d_table;
+    p->d_bytes = p->d_off + k;
+    p->d_items = (const FusionItem*)(p->d_bytes + k);
+    *plan = p;
+    return MI_CCL_SUCCESS;
+}
+
+int mi_ccl_fusion_plan_destroy(mi_ccl_fusion_plan* plan) {
+    if (!plan)
+        return MI_CCL_SUCCESS;
+    hipError_t e = plan->d_table ? hipFree(plan->d_table) : hipSuccess;
+    delete plan;
+    return fusion_status_of(e);
+}
+
+size_t mi_ccl_fusion_plan_bytes(const mi_ccl_fusion_plan* plan) {
+    return plan ? plan->total_bytes : 0;
+}
+
+size_t mi_ccl_fusion_plan_offset(const mi_ccl_fusion_plan* plan, size_t i) {
+    return (plan && i < plan->k) ? plan->offsets[i] : (size_t)-1;
+}
+
+static int fusion_copy(mi_ccl_fusion_plan* plan, const void* const* tensors, void* fusion_buf, void* stream,
+                       int to_fusion) {
+    if (!plan || !tensors || (!fusion_buf && plan->total_bytes))
+        return MI_CCL_INVALID_ARGUMENTS;
+    for (size_t t = 0; t < plan->k; t++)
+        if (!tensors[t] && plan->counts[t])
+            return MI_CCL_INVALID_ARGUMENTS;
+    Tuning tune = current_tuning();
+    for (size_t t0 = 0; t0 < plan->k; t0 += kFusionGroup) {
+        const size_t t1 = (t0 + kFusionGroup < plan->k) ? t0 + kFusionGroup : plan->k;
+        const uint64_t i0 = plan->item_begin[t0], i1 = plan->item_begin[t1];
+        if (i1 == i0)
+            continue;
+        FusionPtrs ptrs;
+        for (size_t t = t0; t < t1; t++) ptrs.p[t - t0] = tensors[t];
+        int grid = grid_for(i1 - i0, tune);
+        hipLaunchKernelGGL(fusion_copy_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ptrs,
+                           (unsigned char*)fusion_buf, plan->d_off, plan->d_bytes, plan->d_items + i0,
+                           (uint32_t)(i1 - i0), (uint32_t)t0, to_fusion);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess)
+            return fusion_status_of(e);
+    }
+    return MI_CCL_SUCCESS;
+}
+
+int mi_ccl_fusion_pack(mi_ccl_fusion_plan* plan, const void* const* tensors, void* fusion_buf, void* stream) {
+    return fusion_copy(plan, tensors, fusion_buf, stream, 1);
+}
+
+int mi_ccl_fusion_unpack(mi_ccl_fusion_plan* plan, const void* fusion_buf, void* const* tensors, void* stream) {
+    return fusion_copy(plan, (const void* const*)tensors, (void*)fusion_buf, stream, 0);
+}
+
+int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* own_tensors, const void* const* peers,
+                         int n_peers, void* const* out_tensors, int lp_mode, int bf16_impl, void* stream) {
+    if (!plan || !own_tensors || !out_tensors || n_peers < 0 || n_peers > kFusionMaxPeers || (n_peers && !peers))
+        return MI_CCL_INVALID_ARGUMENTS;
+    if (op < MI_CCL_SUM || op > MI_CCL_MAX || bf16_impl < MI_CCL_BF16_SCALAR || bf16_impl > MI_CCL_BF16_AVX512BF)
+        return MI_CCL_INVALID_ARGUMENTS;
+    const bool keep = (lp_mode & MI_CCL_LP_KEEP_PRECISION) != 0;
+    // the truncated tail of the array converter belongs to the end of the *fused* buffer; this entry point
+    // narrows every element the same way
+    if ((lp_mode & ~MI_CCL_LP_KEEP_PRECISION) != 0 || (keep && plan->dtype != MI_CCL_BFLOAT16))
+        return MI_CCL_INVALID_ARGUMENTS;
+    for (size_t t = 0; t < plan->k; t++) {
+        if (plan->counts[t] == 0)
+            continue;
+        if (!own_tensors[t] || !out_tensors[t] || ((uintptr_t)own_tensors[t] % plan->esz) ||
+            ((uintptr_t)out_tensors[t] % plan->esz))
+            return MI_CCL_INVALID_ARGUMENTS;
+    }
+    for (int j = 0; j < n_peers; j++)
+        if (!peers[j] || ((uintptr_t)peers[j] % plan->esz))
+            return MI_CCL_INVALID_ARGUMENTS;
+
+    FusionLaunchArgs a;
+    a.own = own_tensors;
+    a.out = out_tensors;
+    a.peers = peers;
+    a.n_peers = n_peers;
+    a.op = op;
+    a.k = plan->k;
+    a.d_off = plan->d_off;
+    a.d_bytes = plan->d_bytes;
+    a.d_items = plan->d_items;
+    a.item_begin = plan->item_begin.data();
+    a.stream = (hipStream_t)stream;
+    a.tune = current_tuning();
+    hipError_t e;
+    switch (plan->dtype) {
+        case MI_CCL_INT8: e = launch_fusion_reduce<I8Traits>(a); break;
+        case MI_CCL_UINT8: e = launch_fusion_reduce<U8Traits>(a); break;
+        case MI_CCL_INT16: e = launch_fusion_reduce<I16Traits>(a); break;
+        case MI_CCL_UINT16: e = launch_fusion_reduce<U16Traits>(a); break;
+        case MI_CCL_INT32: e = launch_fusion_reduce<I32Traits>(a); break;
+        case MI_CCL_UINT32: e = launch_fusion_reduce<U32Traits>(a); break;
+        case MI_CCL_INT64: e = launch_fusion_reduce<I64Traits>(a); break;
+        case MI_CCL_UINT64: e = launch_fusion_reduce<U64Traits>(a); break;
+        case MI_CCL_FLOAT16: e = launch_fusion_reduce<Fp16PairwiseTraits>(a); break;
+        case MI_CCL_FLOAT32: e = launch_fusion_reduce<F32Traits>(a); break;
+        case MI_CCL_FLOAT64: e = launch_fusion_reduce<F64Traits>(a); break;
+        case MI_CCL_BFLOAT16:
+            if (keep)
+                e = (bf16_impl == MI_CCL_BF16_AVX512BF) ? launch_fusion_reduce<Bf16KeepTraits<true>>(a)
+                                                        : launch_fusion_reduce<Bf16KeepTraits<false>>(a);
+            else if (bf16_impl == MI_CCL_BF16_SCALAR)
+                e = launch_fusion_reduce<Bf16PairScalar>(a);
+            else if (bf16_impl == MI_CCL_BF16_AVX512F)
+                e = launch_fusion_reduce<Bf16PairAvx512f>(a);
+            else
+                e = launch_fusion_reduce<Bf16PairAvx512bf>(a);
+            break;
+        default: e = hipErrorInvalidValue; break;
+    }
+    return fusion_status_of(e);
+}
+
+} /* extern "C" */

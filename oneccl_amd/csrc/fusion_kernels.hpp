@@ -1,0 +1,201 @@
+// Fusion-buffer kernels: pack / unpack of many tensors in one launch and the fused
+// (tensors + peer fusion buffers -> tensors) reduce.  Layout follows oneCCL's fusion manager
+// (src/fusion/fusion.cpp:283-362): tensor t lives at fusion_buf + off[t]; off is a running byte offset,
+// optionally rounded up to an alignment.
+//
+// Work is cut into items of kFusionChunk bytes of one tensor; a block takes items grid-stride.  The item
+// list and the per-tensor offset/size tables live in device memory owned by the plan; the tensor pointers
+// of a call travel as kernel arguments, kFusionGroup tensors per launch.
+#pragma once
+
+#include "reduce_kernels.hpp"
+
+namespace mi {
+
+constexpr int kFusionGroup = 192;                 // tensors per launch (pointer tables must fit the kernarg segment)
+constexpr int kFusionMaxPeers = 16;
+constexpr uint32_t kFusionChunk = 16384;          // bytes of one tensor per work item = kBlock lanes x 16 B x 4
+
+struct FusionItem {
+    uint32_t t;     // tensor index
+    uint32_t c;     // chunk index inside the tensor
+};
+struct FusionPtrs {
+    const void* p[kFusionGroup];
+};
+struct PeerPtrs {
+    const void* p[kFusionMaxPeers];
+};
+
+struct FusionLaunchArgs {
+    const void* const* own;       // host arrays of k device pointers
+    void* const* out;
+    const void* const* peers;     // n_peers fusion buffers
+    int n_peers;
+    int op;
+    size_t k;
+    const uint64_t* d_off;        // device tables of the plan
+    const uint64_t* d_bytes;
+    const FusionItem* d_items;
+    const uint64_t* item_begin;   // host: first item of tensor t, k + 1 entries
+    hipStream_t stream;
+    Tuning tune;
+};
+
+// Copy n <= kFusionChunk bytes with one block.
+__device__ __forceinline__ void copy_span(const unsigned char* src, unsigned char* dst, uint32_t n) {
+    const uint32_t tid = threadIdx.x;
+    const uint32_t d = (uint32_t)((uintptr_t)src ^ (uintptr_t)dst);
+    if ((d & 15u) == 0) {
+        uint32_t head = (uint32_t)(-(intptr_t)src) & 15u;
+        if (head > n) head = n;
+        const uint32_t nvec = (n - head) >> 4, tail = n - head - (nvec << 4);
+        const u32x4* s = (const u32x4*)(src + head);
+        u32x4* o = (u32x4*)(dst + head);
+        u32x4 x[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (tid + u * kBlock < nvec) x[u] = ld_stream(s + tid + u * kBlock);
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (tid + u * kBlock < nvec) st_stream(o + tid + u * kBlock, x[u]);
+        if (tid < head + tail) {
+            uint32_t i = (tid < head) ? tid : head + (nvec << 4) + (tid - head);
+            dst[i] = src[i];
+        }
+        return;
+    }
+    // source and destination disagree modulo 16: move the widest unit both can be aligned to
+    const uint32_t unit = (d & 1u) ? 1u : (d & 2u) ? 2u : (d & 4u) ? 4u : 8u;
+    uint32_t head = (uint32_t)(-(intptr_t)src) & (unit - 1u);
+    if (head > n) head = n;
+    const uint32_t nu = (n - head) / unit, tail = n - head - nu * unit;
+    if (unit == 8) {
+        const uint64_t* s = (const uint64_t*)(src + head);
+        uint64_t* o = (uint64_t*)(dst + head);
+        for (uint32_t i = tid; i < nu; i += kBlock) o[i] = s[i];
+    }
+    else if (unit == 4) {
+        const uint32_t* s = (const uint32_t*)(src + head);
+        uint32_t* o = (uint32_t*)(dst + head);
+        for (uint32_t i = tid; i < nu; i += kBlock) o[i] = s[i];
+    }
+    else if (unit == 2) {
+        const uint16_t* s = (const uint16_t*)(src + head);
+        uint16_t* o = (uint16_t*)(dst + head);
+        for (uint32_t i = tid; i < nu; i += kBlock) o[i] = s[i];
+    }
+    else {
+        for (uint32_t i = tid; i < nu; i += kBlock) dst[head + i] = src[head + i];
+    }
+    if (tid < head + tail) {
+        uint32_t i = (tid < head) ? tid : head + nu * unit + (tid - head);
+        dst[i] = src[i];
+    }
+}
+
+// out_t[i] = own_t[i] OP peer_0[off_t + i] OP ... : one pass, same arithmetic as reduce_vec_rt_kernel
+template <class TR, int OP>
+__global__ void __launch_bounds__(kBlock)
+fusion_reduce_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers, const uint64_t* off,
+                     const uint64_t* bytes, const FusionItem* items, uint32_t nitems, uint32_t t0) {
+    typedef typename TR::elem_t E;
+    constexpr uint32_t ES = sizeof(E);
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t it = blockIdx.x; it < nitems; it += gridDim.x) {
+        const FusionItem w = items[it];
+        const uint64_t lo = (uint64_t)w.c * kFusionChunk;
+        const uint64_t left = bytes[w.t] - lo;
+        const uint32_t nb = left < kFusionChunk ? (uint32_t)left : kFusionChunk;
+        const unsigned char* a = (const unsigned char*)own.p[w.t - t0] + lo;
+        unsigned char* o = (unsigned char*)out.p[w.t - t0] + lo;
+        const uint64_t poff = off[w.t] + lo;
+        // all streams congruent modulo 16?
+        uint32_t mis = (uint32_t)(uintptr_t)a & 15u;
+        bool same = (((uint32_t)(uintptr_t)o & 15u) == mis);
+        for (int j = 0; j < n_peers; j++)
+            same = same && ((((uint32_t)(uintptr_t)peers.p[j] + (uint32_t)poff) & 15u) == mis);
+        const uint32_t nelem = nb / ES;
+        if (same) {
+            uint32_t head = mis ? (16u - mis) / ES : 0;
+            if (head > nelem) head = nelem;
+            const uint32_t nvec = (nelem - head) / TR::VEC, tail = nelem - head - nvec * TR::VEC;
+            Accs<TR> acc[4];
+            const u32x4* s0 = (const u32x4*)(a + head * ES);
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint32_t i = tid + u * kBlock;
+                acc[u] = vec_init<TR>((i < nvec) ? ld_stream(s0 + i) : u32x4{ 0, 0, 0, 0 });
+            }
+            for (int j = 0; j < n_peers; j++) {
+                const u32x4* sj = (const u32x4*)((const unsigned char*)peers.p[j] + poff + head * ES);
+                u32x4 x[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const uint32_t i = tid + u * kBlock;
+                    x[u] = (i < nvec) ? ld_stream(sj + i) : u32x4{ 0, 0, 0, 0 };
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) vec_step<TR, OP>(x[u], acc[u]);
+            }
+            u32x4* d = (u32x4*)(o + head * ES);
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint32_t i = tid + u * kBlock;
+                if (i < nvec) st_stream(d + i, vec_finish<TR>(acc[u]));
+            }
+            if (tid < head + tail) {
+                const uint32_t i = (tid < head) ? tid : head + nvec * TR::VEC + (tid - head);
+                typename TR::acc_t r = TR::init(((const E*)a)[i]);
+                for (int j = 0; j < n_peers; j++)
+                    r = TR::template step<OP>(((const E*)((const unsigned char*)peers.p[j] + poff))[i], r);
+                ((E*)o)[i] = TR::finish(r);
+            }
+        }
+        else {
+            for (uint32_t i = tid; i < nelem; i += kBlock) {
+                typename TR::acc_t r = TR::init(((const E*)a)[i]);
+                for (int j = 0; j < n_peers; j++)
+                    r = TR::template step<OP>(((const E*)((const unsigned char*)peers.p[j] + poff))[i], r);
+                ((E*)o)[i] = TR::finish(r);
+            }
+        }
+    }
+}
+
+template <class TR, int OP>
+inline hipError_t launch_fusion_op(const FusionLaunchArgs& a) {
+    PeerPtrs pp;
+    for (int j = 0; j < kFusionMaxPeers; j++) pp.p[j] = (j < a.n_peers) ? a.peers[j] : nullptr;
+    for (size_t t0 = 0; t0 < a.k; t0 += kFusionGroup) {
+        const size_t t1 = (t0 + kFusionGroup < a.k) ? t0 + kFusionGroup : a.k;
+        const uint64_t i0 = a.item_begin[t0], i1 = a.item_begin[t1];
+        if (i1 == i0)
+            continue;
+        FusionPtrs own, out;
+        for (size_t t = t0; t < t1; t++) {
+            own.p[t - t0] = a.own[t];
+            out.p[t - t0] = a.out[t];
+        }
+        int grid = grid_for(i1 - i0, a.tune);
+        hipLaunchKernelGGL((fusion_reduce_kernel<TR, OP>), dim3(grid), dim3(kBlock), 0, a.stream, own, out, pp,
+                           a.n_peers, a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess)
+            return e;
+    }
+    return hipSuccess;
+}
+
+template <class TR>
+hipError_t launch_fusion_reduce(const FusionLaunchArgs& a) {
+    switch (a.op) {
+        case OP_SUM: return launch_fusion_op<TR, OP_SUM>(a);
+        case OP_PROD: return launch_fusion_op<TR, OP_PROD>(a);
+        case OP_MIN: return launch_fusion_op<TR, OP_MIN>(a);
+        case OP_MAX: return launch_fusion_op<TR, OP_MAX>(a);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace mi

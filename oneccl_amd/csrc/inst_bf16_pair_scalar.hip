@@ -1,0 +1,7 @@
+// Kernels of one element-traits class: Bf16PairwiseTraits<false, false>
+#include "fusion_kernels.hpp"
+
+namespace mi {
+template hipError_t launch_reduce<Bf16PairwiseTraits<false, false>>(const LaunchArgs&);
+template hipError_t launch_fusion_reduce<Bf16PairwiseTraits<false, false>>(const FusionLaunchArgs&);
+}  // namespace mi

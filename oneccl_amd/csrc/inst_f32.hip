@@ -1,0 +1,11 @@
+// Kernels of one element-traits class: F32Traits
+#include "fusion_kernels.hpp"
+
+namespace mi {
+template <>
+struct HasUnrollVariants<F32Traits> {
+    static constexpr bool value = true;
+};
+template hipError_t launch_reduce<F32Traits>(const LaunchArgs&);
+template hipError_t launch_fusion_reduce<F32Traits>(const FusionLaunchArgs&);
+}  // namespace mi

@@ -1,0 +1,7 @@
+// Kernels of one element-traits class: I8Traits
+#include "fusion_kernels.hpp"
+
+namespace mi {
+template hipError_t launch_reduce<I8Traits>(const LaunchArgs&);
+template hipError_t launch_fusion_reduce<I8Traits>(const FusionLaunchArgs&);
+}  // namespace mi

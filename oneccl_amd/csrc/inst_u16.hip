@@ -1,0 +1,7 @@
+// Kernels of one element-traits class: U16Traits
+#include "fusion_kernels.hpp"
+
+namespace mi {
+template hipError_t launch_reduce<U16Traits>(const LaunchArgs&);
+template hipError_t launch_fusion_reduce<U16Traits>(const FusionLaunchArgs&);
+}  // namespace mi

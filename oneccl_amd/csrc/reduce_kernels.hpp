@@ -1,0 +1,477 @@
+// N-input elementwise reduce kernels for gfx950 (MI355X), templated on an element-traits class.
+//
+// Every kernel is a pure HBM stream: each lane issues one 128-bit load per input per unrolled step (a
+// wave reads 1 KiB contiguous per input per instruction), folds the inputs in argument order in registers
+// and writes one 128-bit nontemporal store.  There is no cross-lane traffic, no LDS and no MFMA.
+//
+// Arithmetic follows the oneCCL CPU reduction: acc = src0; acc = step(in = src_j, inout = acc), j = 1..N-1
+// (src/comp/comp.cpp:31-58 for the step, src/kernels/kernels.cl:279-282 for the order).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace mi {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kBlock = 256;     // 4 wavefronts of 64 lanes
+constexpr int kMaxFixedN = 8;   // inputs unrolled at compile time
+constexpr int kMaxSrcs = 64;    // inputs of the run-time-N kernels
+
+enum { OP_SUM = 0, OP_PROD = 1, OP_MIN = 2, OP_MAX = 3 };
+
+struct SrcTable {               // by-value kernel argument
+    const void* p[kMaxSrcs];
+};
+template <int N>
+struct SrcFixed {
+    const void* p[N];
+};
+
+struct Tuning {
+    int waves_per_cu;   // resident 256-thread blocks per CU the grid is sized for
+    int max_blocks;     // 0 = no cap
+    int xcd_chunked;    // 1: each XCD streams one contiguous eighth of the buffer
+    int variant;        // kernel variant selector (unroll depth), 0 = default
+    int num_cus;
+};
+
+struct LaunchArgs {
+    const void* const* srcs;    // host array of n device pointers
+    int n;
+    void* dst;
+    size_t count;               // elements
+    int op;
+    hipStream_t stream;
+    Tuning tune;
+};
+
+// ---------------------------------------------------------------------------------------------------
+// bit helpers
+
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// fp32 -> bf16 exactly as VCVTNEPS2BF16 (src/comp/bf16/bf16_intrisics.hpp:73-75): round to nearest even,
+// fp32 denormals read as zero, NaN quieted keeping its top payload bits, overflow rounds to Inf.
+__device__ __forceinline__ uint32_t bf16_narrow_rne(uint32_t u) {
+    uint32_t e = u & 0x7f800000u;
+    uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    uint32_t nan = (u >> 16) | 0x40u;
+    r = (e == 0x7f800000u && (u & 0x007fffffu) != 0) ? nan : r;
+    r = (e == 0) ? ((u >> 16) & 0x8000u) : r;
+    return r & 0xffffu;
+}
+// fp32 -> bf16 by dropping the low half (src/comp/bf16/bf16.cpp:50-54, bf16_intrisics.hpp:67-70)
+__device__ __forceinline__ uint32_t bf16_narrow_trunc(uint32_t u) { return u >> 16; }
+
+// compare on the float value, select on the bits: the returned operand's bits are never touched
+template <int OP, bool VEC_SEM>
+__device__ __forceinline__ uint32_t f32_minmax_bits(uint32_t in, uint32_t io) {
+    float a = as_f32(in), b = as_f32(io);
+    if (VEC_SEM)   // _mm512_min_ps(in, inout): second source on ties/NaN (bf16_intrisics.cpp:28-34)
+        return (OP == OP_MIN) ? ((a < b) ? in : io) : ((a > b) ? in : io);
+    // std::min(in, inout) / std::max(in, inout): first argument on ties/NaN (comp.cpp:46-55)
+    return (OP == OP_MIN) ? ((b < a) ? io : in) : ((a < b) ? io : in);
+}
+
+template <int OP, bool VEC_SEM>
+__device__ __forceinline__ uint32_t f32_step_bits(uint32_t in, uint32_t io) {
+    if (OP == OP_SUM) return as_u32(as_f32(io) + as_f32(in));
+    if (OP == OP_PROD) return as_u32(as_f32(io) * as_f32(in));
+    return f32_minmax_bits<OP, VEC_SEM>(in, io);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// element traits: elem_t (storage), acc_t (what is carried between steps), init / step / finish
+
+// Integers and fp32/fp64 (CCL_REDUCE, comp.cpp:31-58).  Integer sum/prod are done on the unsigned type of
+// the same width (two's-complement wrap).  min/max: ties and unordered operands return `in`.
+template <class T, class U>
+struct PlainTraits {
+    typedef T elem_t;
+    typedef T acc_t;
+    static constexpr int VEC = 16 / sizeof(T);
+    static __device__ __forceinline__ acc_t init(elem_t x) { return x; }
+    template <int OP>
+    static __device__ __forceinline__ acc_t step(elem_t in, acc_t io) {
+        if (OP == OP_SUM) return (T)((U)io + (U)in);
+        if (OP == OP_PROD) return (T)((U)io * (U)in);
+        if (OP == OP_MIN) return (io < in) ? io : in;
+        return (in < io) ? io : in;
+    }
+    static __device__ __forceinline__ elem_t finish(acc_t a) { return a; }
+};
+
+// float and double go through their bit patterns for min/max so that no floating-point instruction can
+// canonicalise the operand that is returned.
+struct F32Traits {
+    typedef uint32_t elem_t;
+    typedef uint32_t acc_t;
+    static constexpr int VEC = 4;
+    static __device__ __forceinline__ acc_t init(elem_t x) { return x; }
+    template <int OP>
+    static __device__ __forceinline__ acc_t step(elem_t in, acc_t io) { return f32_step_bits<OP, false>(in, io); }
+    static __device__ __forceinline__ elem_t finish(acc_t a) { return a; }
+};
+
+struct F64Traits {
+    typedef uint64_t elem_t;
+    typedef uint64_t acc_t;
+    static constexpr int VEC = 2;
+    static __device__ __forceinline__ acc_t init(elem_t x) { return x; }
+    template <int OP>
+    static __device__ __forceinline__ acc_t step(elem_t in, acc_t io) {
+        double a = __builtin_bit_cast(double, in), b = __builtin_bit_cast(double, io);
+        if (OP == OP_SUM) return __builtin_bit_cast(uint64_t, b + a);
+        if (OP == OP_PROD) return __builtin_bit_cast(uint64_t, b * a);
+        if (OP == OP_MIN) return (b < a) ? io : in;
+        return (a < b) ? io : in;
+    }
+    static __device__ __forceinline__ elem_t finish(acc_t a) { return a; }
+};
+
+// bfloat16, rounded to bf16 after every pair (ccl_bf16_reduce, src/comp/bf16/bf16.cpp:63-110,
+// bf16_intrisics.hpp:80-114).  RNE: avx512bf narrowing, else truncation.  VEC_SEM: vector min/max operand
+// order (avx512f / avx512bf) instead of std:: (scalar).  The carried value is the raw bf16 pattern, so a
+// single input passes through unchanged, as a chain of zero pairwise calls does.
+template <bool RNE, bool VEC_SEM>
+struct Bf16PairwiseTraits {
+    typedef uint16_t elem_t;
+    typedef uint32_t acc_t;     // bf16 bits in the low half
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ acc_t init(elem_t x) { return x; }
+    template <int OP>
+    static __device__ __forceinline__ acc_t step(elem_t in, acc_t io) {
+        uint32_t r = f32_step_bits<OP, VEC_SEM>((uint32_t)in << 16, io << 16);
+        return RNE ? bf16_narrow_rne(r) : bf16_narrow_trunc(r);
+    }
+    static __device__ __forceinline__ elem_t finish(acc_t a) { return (elem_t)a; }
+};
+
+// bfloat16, widened once, accumulated in fp32 with the plain fp32 step (std:: min/max), narrowed once
+// (ccl_comp_batch_reduce with bf16_keep_precision_mode, src/comp/comp.cpp:214-234).
+template <bool RNE>
+struct Bf16KeepTraits {
+    typedef uint16_t elem_t;
+    typedef uint32_t acc_t;     // fp32 bits
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ acc_t init(elem_t x) { return (uint32_t)x << 16; }
+    template <int OP>
+    static __device__ __forceinline__ acc_t step(elem_t in, acc_t io) {
+        return f32_step_bits<OP, false>((uint32_t)in << 16, io);
+    }
+    static __device__ __forceinline__ elem_t finish(acc_t a) {
+        return (elem_t)(RNE ? bf16_narrow_rne(a) : bf16_narrow_trunc(a));
+    }
+};
+
+// float16, rounded after every pair through fp32 (ccl_fp16_reduce f16c / avx512f implementations,
+// src/comp/fp16/fp16_intrisics.hpp:95-148): VCVTPH2PS both, one fp32 op, VCVTPS2PH round-to-nearest-even,
+// fp16 subnormals kept.  min/max return `inout` on ties/NaN and quiet a NaN they return (the x86 widening
+// conversion quiets it).
+struct Fp16PairwiseTraits {
+    typedef uint16_t elem_t;
+    typedef uint32_t acc_t;     // fp16 bits in the low half
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ acc_t init(elem_t x) { return x; }
+    static __device__ __forceinline__ float widen(uint32_t h) {
+        return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+    }
+    template <int OP>
+    static __device__ __forceinline__ acc_t step(elem_t in, acc_t io) {
+        float a = widen(in), b = widen(io);
+        if (OP == OP_SUM || OP == OP_PROD) {
+            float r = (OP == OP_SUM) ? (b + a) : (b * a);
+            return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)r);
+        }
+        uint32_t r = (OP == OP_MIN) ? ((a < b) ? (uint32_t)in : io) : ((a > b) ? (uint32_t)in : io);
+        bool nan = (r & 0x7c00u) == 0x7c00u && (r & 0x03ffu) != 0;
+        return nan ? (r | 0x0200u) : r;
+    }
+    static __device__ __forceinline__ elem_t finish(acc_t a) { return (elem_t)a; }
+};
+
+typedef PlainTraits<int8_t, uint8_t> I8Traits;
+typedef PlainTraits<uint8_t, uint8_t> U8Traits;
+typedef PlainTraits<int16_t, uint16_t> I16Traits;
+typedef PlainTraits<uint16_t, uint16_t> U16Traits;
+typedef PlainTraits<int32_t, uint32_t> I32Traits;
+typedef PlainTraits<uint32_t, uint32_t> U32Traits;
+typedef PlainTraits<int64_t, uint64_t> I64Traits;
+typedef PlainTraits<uint64_t, uint64_t> U64Traits;
+
+// ---------------------------------------------------------------------------------------------------
+// 128-bit vector <-> VEC elements
+
+template <class TR>
+struct Lanes {
+    typename TR::elem_t v[TR::VEC];
+};
+template <class TR>
+struct Accs {
+    typename TR::acc_t v[TR::VEC];
+};
+
+template <class TR>
+__device__ __forceinline__ Accs<TR> vec_init(u32x4 x) {
+    Lanes<TR> l = __builtin_bit_cast(Lanes<TR>, x);
+    Accs<TR> a;
+#pragma unroll
+    for (int k = 0; k < TR::VEC; k++) a.v[k] = TR::init(l.v[k]);
+    return a;
+}
+template <class TR, int OP>
+__device__ __forceinline__ void vec_step(u32x4 x, Accs<TR>& a) {
+    Lanes<TR> l = __builtin_bit_cast(Lanes<TR>, x);
+#pragma unroll
+    for (int k = 0; k < TR::VEC; k++) a.v[k] = TR::template step<OP>(l.v[k], a.v[k]);
+}
+template <class TR>
+__device__ __forceinline__ u32x4 vec_finish(const Accs<TR>& a) {
+    Lanes<TR> l;
+#pragma unroll
+    for (int k = 0; k < TR::VEC; k++) l.v[k] = TR::finish(a.v[k]);
+    return __builtin_bit_cast(u32x4, l);
+}
+
+__device__ __forceinline__ u32x4 ld_stream(const u32x4* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void st_stream(u32x4* p, u32x4 v) { __builtin_nontemporal_store(v, p); }
+
+// The count % VEC elements after the last full vector and the elements before the first aligned one:
+// at most 2*(VEC-1) <= 30 elements, one per lane of the first wave of block 0.
+template <class TR, int OP, class SRC>
+__device__ __forceinline__ void reduce_edges(const SRC& src, int n, void* dst, uint32_t head, uint64_t nvec,
+                                             uint32_t tail) {
+    typedef typename TR::elem_t E;
+    uint32_t t = threadIdx.x;
+    if (t < head + tail) {
+        uint64_t i = (t < head) ? t : (uint64_t)head + nvec * TR::VEC + (t - head);
+        typename TR::acc_t a = TR::init(((const E*)src.p[0])[i]);
+        for (int j = 1; j < n; j++) a = TR::template step<OP>(((const E*)src.p[j])[i], a);
+        ((E*)dst)[i] = TR::finish(a);
+    }
+}
+
+// tile index sequence of one block: plain grid stride, or per-XCD contiguous shares (blocks are handed to
+// the 8 XCDs round-robin, so blockIdx & 7 names the XCD a block runs on)
+struct TileIter {
+    uint64_t tile, end, stride;
+    __device__ __forceinline__ TileIter(uint64_t ntiles, int xcd_chunked) {
+        if (xcd_chunked && (gridDim.x & 7u) == 0) {
+            uint64_t per_xcd = (ntiles + 7) >> 3;
+            uint64_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+            tile = xcd * per_xcd + slot;
+            end = (xcd + 1) * per_xcd < ntiles ? (xcd + 1) * per_xcd : ntiles;
+            stride = gridDim.x >> 3;
+        }
+        else {
+            tile = blockIdx.x;
+            end = ntiles;
+            stride = gridDim.x;
+        }
+    }
+};
+
+// Fixed N (1..8): all N*UNROLL loads of a tile are issued before the first use.
+template <class TR, int OP, int N, int UNROLL>
+__global__ void __launch_bounds__(kBlock)
+reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint32_t tail, int xcd_chunked) {
+    typedef typename TR::elem_t E;
+    constexpr uint64_t kTile = (uint64_t)kBlock * UNROLL;
+    const u32x4* s[N];
+#pragma unroll
+    for (int j = 0; j < N; j++) s[j] = (const u32x4*)((const E*)src.p[j] + head);
+    u32x4* d = (u32x4*)((E*)dst + head);
+    const uint64_t ntiles = (nvec + kTile - 1) / kTile;
+
+    for (TileIter it(ntiles, xcd_chunked); it.tile < it.end; it.tile += it.stride) {
+        const uint64_t base = it.tile * kTile + threadIdx.x;
+        if (base + (uint64_t)(UNROLL - 1) * kBlock < nvec) {
+            u32x4 x[N][UNROLL];
+#pragma unroll
+            for (int j = 0; j < N; j++)
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++) x[j][u] = ld_stream(s[j] + base + (uint64_t)u * kBlock);
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                Accs<TR> a = vec_init<TR>(x[0][u]);
+#pragma unroll
+                for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j][u], a);
+                st_stream(d + base + (uint64_t)u * kBlock, vec_finish<TR>(a));
+            }
+        }
+        else {
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const uint64_t i = base + (uint64_t)u * kBlock;
+                if (i < nvec) {
+                    u32x4 x[N];
+#pragma unroll
+                    for (int j = 0; j < N; j++) x[j] = ld_stream(s[j] + i);
+                    Accs<TR> a = vec_init<TR>(x[0]);
+#pragma unroll
+                    for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j], a);
+                    st_stream(d + i, vec_finish<TR>(a));
+                }
+            }
+        }
+    }
+    if (blockIdx.x == 0 && (head | tail)) reduce_edges<TR, OP>(src, N, dst, head, nvec, tail);
+}
+
+// Run-time N (9..64): inputs are folded in one after the other, UNROLL vectors of each in flight.
+template <class TR, int OP, int UNROLL>
+__global__ void __launch_bounds__(kBlock)
+reduce_vec_rt_kernel(SrcTable src, int n, void* dst, uint32_t head, uint64_t nvec, uint32_t tail,
+                     int xcd_chunked) {
+    typedef typename TR::elem_t E;
+    constexpr uint64_t kTile = (uint64_t)kBlock * UNROLL;
+    u32x4* d = (u32x4*)((E*)dst + head);
+    const uint64_t ntiles = (nvec + kTile - 1) / kTile;
+    for (TileIter it(ntiles, xcd_chunked); it.tile < it.end; it.tile += it.stride) {
+        const uint64_t base = it.tile * kTile + threadIdx.x;
+        Accs<TR> a[UNROLL];
+        const u32x4* s0 = (const u32x4*)((const E*)src.p[0] + head);
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            const uint64_t i = base + (uint64_t)u * kBlock;
+            u32x4 x = (i < nvec) ? ld_stream(s0 + i) : u32x4{ 0, 0, 0, 0 };
+            a[u] = vec_init<TR>(x);
+        }
+        for (int j = 1; j < n; j++) {
+            const u32x4* sj = (const u32x4*)((const E*)src.p[j] + head);
+            u32x4 x[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const uint64_t i = base + (uint64_t)u * kBlock;
+                x[u] = (i < nvec) ? ld_stream(sj + i) : u32x4{ 0, 0, 0, 0 };
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) vec_step<TR, OP>(x[u], a[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            const uint64_t i = base + (uint64_t)u * kBlock;
+            if (i < nvec) st_stream(d + i, vec_finish<TR>(a[u]));
+        }
+    }
+    if (blockIdx.x == 0 && (head | tail)) reduce_edges<TR, OP>(src, n, dst, head, nvec, tail);
+}
+
+// One element per lane, any alignment of the buffers relative to each other.
+template <class TR, int OP>
+__global__ void __launch_bounds__(kBlock)
+reduce_elem_kernel(SrcTable src, int n, void* dst, uint64_t count) {
+    typedef typename TR::elem_t E;
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < count; i += stride) {
+        typename TR::acc_t a = TR::init(((const E*)src.p[0])[i]);
+        for (int j = 1; j < n; j++) a = TR::template step<OP>(((const E*)src.p[j])[i], a);
+        ((E*)dst)[i] = TR::finish(a);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// host-side launch
+
+inline int grid_for(uint64_t ntiles, const Tuning& t) {
+    uint64_t g = (uint64_t)t.num_cus * (uint64_t)(t.waves_per_cu > 0 ? t.waves_per_cu : 8);
+    if (t.max_blocks > 0 && g > (uint64_t)t.max_blocks) g = (uint64_t)t.max_blocks;
+    if (t.xcd_chunked) g = (g + 7) & ~7ull;
+    if (g > ntiles) g = ntiles;
+    if (t.xcd_chunked && g >= 8) g &= ~7ull;
+    return g ? (int)g : 1;
+}
+
+template <class TR, int OP, int N, int UNROLL>
+inline hipError_t launch_fixed(const LaunchArgs& a, uint32_t head, uint64_t nvec, uint32_t tail) {
+    SrcFixed<N> s;
+    for (int j = 0; j < N; j++) s.p[j] = a.srcs[j];
+    const uint64_t tile = (uint64_t)kBlock * UNROLL;
+    int grid = grid_for((nvec + tile - 1) / tile, a.tune);
+    hipLaunchKernelGGL((reduce_vec_kernel<TR, OP, N, UNROLL>), dim3(grid), dim3(kBlock), 0, a.stream, s, a.dst,
+                       head, nvec, tail, a.tune.xcd_chunked);
+    return hipGetLastError();
+}
+
+// Traits classes whose unroll depth can be switched at run time (Tuning::variant = 1, 2 or 4); for the
+// others only the default depth is compiled.
+template <class TR>
+struct HasUnrollVariants {
+    static constexpr bool value = false;
+};
+
+template <class TR, int OP, int N>
+inline hipError_t launch_fixed_unroll(const LaunchArgs& a, uint32_t head, uint64_t nvec, uint32_t tail) {
+    // loads in flight per lane = N * UNROLL
+    constexpr int kDefault = (N <= 4) ? 4 : 2;
+    if constexpr (HasUnrollVariants<TR>::value) {
+        switch (a.tune.variant) {
+            case 1: return launch_fixed<TR, OP, N, 1>(a, head, nvec, tail);
+            case 2: return launch_fixed<TR, OP, N, 2>(a, head, nvec, tail);
+            case 4: return launch_fixed<TR, OP, N, 4>(a, head, nvec, tail);
+            default: break;
+        }
+    }
+    return launch_fixed<TR, OP, N, kDefault>(a, head, nvec, tail);
+}
+
+template <class TR, int OP>
+inline hipError_t launch_op(const LaunchArgs& a) {
+    typedef typename TR::elem_t E;
+    constexpr uint32_t VEC = TR::VEC;
+    // common misalignment of all buffers to 16 bytes, in elements; mixed misalignment -> element kernel
+    const uintptr_t mis = (uintptr_t)a.dst & 15u;
+    bool same = true;
+    for (int j = 0; j < a.n; j++) same = same && (((uintptr_t)a.srcs[j] & 15u) == mis);
+    if (!same || (mis % sizeof(E)) != 0) {
+        SrcTable s;
+        for (int j = 0; j < a.n; j++) s.p[j] = a.srcs[j];
+        uint64_t blocks = (a.count + kBlock - 1) / kBlock;
+        int grid = grid_for(blocks, a.tune);
+        hipLaunchKernelGGL((reduce_elem_kernel<TR, OP>), dim3(grid), dim3(kBlock), 0, a.stream, s, a.n, a.dst,
+                           (uint64_t)a.count);
+        return hipGetLastError();
+    }
+    uint64_t head = mis ? (16u - mis) / sizeof(E) : 0;
+    if (head > a.count) head = a.count;
+    const uint64_t nvec = (a.count - head) / VEC;
+    const uint32_t tail = (uint32_t)(a.count - head - nvec * VEC);
+    switch (a.n) {
+        case 1: return launch_fixed_unroll<TR, OP, 1>(a, (uint32_t)head, nvec, tail);
+        case 2: return launch_fixed_unroll<TR, OP, 2>(a, (uint32_t)head, nvec, tail);
+        case 3: return launch_fixed_unroll<TR, OP, 3>(a, (uint32_t)head, nvec, tail);
+        case 4: return launch_fixed_unroll<TR, OP, 4>(a, (uint32_t)head, nvec, tail);
+        case 5: return launch_fixed_unroll<TR, OP, 5>(a, (uint32_t)head, nvec, tail);
+        case 6: return launch_fixed_unroll<TR, OP, 6>(a, (uint32_t)head, nvec, tail);
+        case 7: return launch_fixed_unroll<TR, OP, 7>(a, (uint32_t)head, nvec, tail);
+        case 8: return launch_fixed_unroll<TR, OP, 8>(a, (uint32_t)head, nvec, tail);
+        default: {
+            SrcTable s;
+            for (int j = 0; j < a.n; j++) s.p[j] = a.srcs[j];
+            constexpr int UNROLL = 4;
+            const uint64_t tile = (uint64_t)kBlock * UNROLL;
+            int grid = grid_for((nvec + tile - 1) / tile, a.tune);
+            hipLaunchKernelGGL((reduce_vec_rt_kernel<TR, OP, UNROLL>), dim3(grid), dim3(kBlock), 0, a.stream, s,
+                               a.n, a.dst, (uint32_t)head, nvec, tail, a.tune.xcd_chunked);
+            return hipGetLastError();
+        }
+    }
+}
+
+// One instantiation of this per traits class lives in its own translation unit.
+template <class TR>
+hipError_t launch_reduce(const LaunchArgs& a) {
+    switch (a.op) {
+        case OP_SUM: return launch_op<TR, OP_SUM>(a);
+        case OP_PROD: return launch_op<TR, OP_PROD>(a);
+        case OP_MIN: return launch_op<TR, OP_MIN>(a);
+        case OP_MAX: return launch_op<TR, OP_MAX>(a);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace mi

@@ -1,0 +1,134 @@
+"""GPU parity of the fusion-buffer path: pack / N-input reduce / unpack and the fused single-pass form,
+against the oracle's pack -> reduce -> unpack (layout of src/fusion/fusion.cpp:283-362)."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from gpu_util import assert_same, make_inputs, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def comp():
+    import torch
+    assert torch.cuda.is_available()
+    import oneccl_amd.comp as c
+    c.lib()
+    return c
+
+
+def log_uniform_counts(rng, k, lo, hi):
+    return [int(round(np.exp(rng.uniform(np.log(lo), np.log(hi))))) for _ in range(k)]
+
+
+def test_fusion_offsets_match_oracle(comp):
+    rng = np.random.default_rng(0)
+    counts = log_uniform_counts(rng, 300, 1, 100000)
+    for align in (1, 2, 16, 256):
+        for esz in (1, 2, 4, 8):
+            offs, total = comp.fusion_offsets(counts, esz, align)
+            o2, t2 = O.fusion_offsets(counts, esz, align)
+            assert offs == [int(x) for x in o2] and total == t2
+    assert comp.lib().mi_ccl_fusion_offsets(None, 0, 2, 3, None, None) == comp.INVALID_ARGUMENTS
+
+
+@pytest.mark.parametrize("align", [1, 256])
+@pytest.mark.parametrize("dtype", [O.BFLOAT16, O.FLOAT32, O.INT8])
+def test_pack_reduce_unpack_and_fused(comp, align, dtype):
+    import torch
+    rng = np.random.default_rng(42 + align + dtype)
+    k = 230                       # more than one launch group of tensors
+    counts = log_uniform_counts(rng, k, 1, 40000)
+    counts[5] = 0 if align == 256 else 1
+    np_t = O.NP_STORAGE[dtype]
+    esz = O.DTYPE_SIZE[dtype]
+    n_peers = 3
+    tensors = [make_inputs(rng, dtype, c, O.SUM, 1)[0] if c else np.zeros(0, np_t) for c in counts]
+    plan = comp.FusionPlan(counts, dtype, align)
+    offs, total = O.fusion_offsets(counts, esz, align)
+    assert plan.nbytes == total and [plan.offset(i) for i in range(k)] == [int(x) for x in offs]
+    nelem = (total + esz - 1) // esz
+    peers = [make_inputs(rng, dtype, nelem, O.SUM, 1)[0] for _ in range(n_peers)]
+    lp = comp.LP_KEEP_PRECISION if dtype == O.BFLOAT16 else comp.LP_PAIRWISE
+    keep = 1 if dtype == O.BFLOAT16 else 0
+
+    # oracle: pack -> N-input reduce over the fused buffer -> unpack
+    fb = O.fusion_pack(tensors, offs, nelem * esz, esz)
+    fused = O.reduce_n([fb.view(np_t)] + peers, dtype, O.SUM, keep=keep)
+    want = O.fusion_unpack(fused.view(np.uint8), counts, offs, np_t)
+
+    # GPU, three steps.  Some tensors sit at odd element offsets inside a larger allocation.
+    holders, d_t = [], []
+    for i, t in enumerate(tensors):
+        sh = (i % 3) if align == 1 else 0
+        h = to_dev(np.concatenate([np.zeros(sh, np_t), t, np.zeros(8, np_t)]))
+        holders.append(h)
+        d_t.append(h.data_ptr() + sh * esz)
+    d_fb = to_dev(np.full(nelem, 0, np_t))
+    plan.pack(d_t, d_fb)
+    torch.cuda.synchronize()
+    got_fb = to_host(d_fb, np_t).view(np.uint8)
+    for i, c in enumerate(counts):      # payload bytes only; padding is not written
+        o = int(offs[i])
+        assert (got_fb[o:o + c * esz] == fb[o:o + c * esz]).all(), f"pack tensor {i}"
+    d_peers = [to_dev(p) for p in peers]
+    comp.comp_reduce_n(dtype, O.SUM, [d_fb] + d_peers, d_fb, nelem, lp_mode=lp)
+    outs = [to_dev(np.zeros(c + 4, np_t)) for c in counts]
+    plan.unpack(d_fb, outs)
+    torch.cuda.synchronize()
+    for i, c in enumerate(counts):
+        g = to_host(outs[i], np_t)
+        assert_same(g[:c], want[i], dtype, f"3-step tensor {i}")
+        assert (g[c:] == 0).all(), "unpack wrote past the tensor"
+
+    # GPU, fused single pass, out of place and in place
+    outs2 = [to_dev(np.zeros(c + 4, np_t)) for c in counts]
+    plan.reduce(O.SUM, d_t, d_peers, outs2, lp_mode=lp)
+    torch.cuda.synchronize()
+    for i, c in enumerate(counts):
+        g = to_host(outs2[i], np_t)
+        assert_same(g[:c], want[i], dtype, f"fused tensor {i}")
+        assert (g[c:] == 0).all()
+    plan.reduce(O.SUM, d_t, d_peers, d_t, lp_mode=lp)
+    torch.cuda.synchronize()
+    for i, c in enumerate(counts):
+        sh = (i % 3) if align == 1 else 0
+        g = to_host(holders[i], np_t)
+        assert_same(g[sh:sh + c], want[i], dtype, f"fused in-place tensor {i}")
+        assert (g[:sh] == 0).all() and (g[sh + c:] == 0).all()
+    plan.close()
+
+
+def test_fusion_config_bf16_256_tensors(comp):
+    """The benchmark's fusion configuration at reduced element counts: 256 bf16 gradient tensors, counts
+    log-uniform, N(0, 0.02) values, 256-byte aligned offsets, 8-input sum against 7 peer fusion buffers."""
+    import torch
+    rng = np.random.default_rng(2024)
+    counts = log_uniform_counts(rng, 256, 2048, 65536)
+    tensors = [O.bf16_from_f32((rng.standard_normal(c) * 0.02).astype(np.float32)) for c in counts]
+    plan = comp.FusionPlan(counts, O.BFLOAT16, 256)
+    offs, total = O.fusion_offsets(counts, 2, 256)
+    nelem = total // 2
+    peers = [O.bf16_from_f32((rng.standard_normal(nelem) * 0.02).astype(np.float32)) for _ in range(7)]
+    fb = O.fusion_pack(tensors, offs, total, 2)
+    fused = O.reduce_n([fb.view(np.uint16)] + peers, O.BFLOAT16, O.SUM, keep=1, threads=8)
+    want = O.fusion_unpack(fused.view(np.uint8), counts, offs, np.uint16)
+    d_t = [to_dev(t) for t in tensors]
+    d_peers = [to_dev(p) for p in peers]
+    outs = [torch.empty_like(t) for t in d_t]
+    plan.reduce(O.SUM, d_t, d_peers, outs, lp_mode=comp.LP_KEEP_PRECISION)
+    torch.cuda.synchronize()
+    for i in range(256):
+        assert (to_host(outs[i], np.uint16) == want[i]).all(), i
+    # per-tensor invariant: fused result == unfused 8-input reduce of the tensor with the peer slices
+    i = 17
+    lo = int(offs[i]) // 2
+    single = torch.empty_like(d_t[i])
+    comp.comp_reduce_n(O.BFLOAT16, O.SUM, [d_t[i]] + [p.data_ptr() + lo * 2 for p in d_peers], single, counts[i],
+                       lp_mode=comp.LP_KEEP_PRECISION)
+    torch.cuda.synchronize()
+    assert (to_host(single, np.uint16) == want[i]).all()
+    with pytest.raises(comp.CclError):
+        plan.reduce(O.SUM, d_t, d_peers, outs, lp_mode=comp.LP_KEEP_PRECISION | comp.LP_TAIL_QUIRK)
+    plan.close()

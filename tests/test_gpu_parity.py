@@ -1,0 +1,304 @@
+"""GPU parity: the HIP path, called through the C ABI (ctypes binding oneccl_amd.comp), against the CPU oracle
+and against the golden vectors made by the reference's own code.  Bit-exact for every type; two NaNs of a
+floating type compare equal whatever their payload (the reference itself does not pin it for sum/prod)."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from gpu_util import assert_same, make_inputs, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def comp():
+    import torch
+    assert torch.cuda.is_available(), "needs a GPU"
+    import oneccl_amd.comp as c
+    c.lib()     # raises if the HIP library is missing: no fallback
+    return c
+
+
+def lp_variants(dtype):
+    """(lp_mode, bf16_impl, oracle keep, oracle quirk) combinations that exist for a dtype."""
+    if dtype == O.BFLOAT16:
+        return [(0, 0, 0, 0), (0, 1, 0, 0), (0, 2, 0, 0), (1, 2, 1, 0), (1, 1, 1, 0), (3, 2, 1, 1), (3, 0, 1, 1)]
+    return [(0, 2, 0, 0)]
+
+
+COUNTS = [1, 7, 15, 16, 17, 33, 1000, 4099, 70001]
+
+
+@pytest.mark.parametrize("dtype", range(12))
+@pytest.mark.parametrize("op", range(4))
+def test_reduce_n_all_dtypes_ops(comp, dtype, op):
+    import torch
+    rng = np.random.default_rng(1000 + dtype * 4 + op)
+    for n in (1, 2, 3, 4, 5, 8, 9, 13):
+        for count in COUNTS:
+            if n > 8 and count not in (17, 4099, 70001):
+                continue
+            kinds = ["config", "bits"] if dtype in (O.FLOAT16, O.BFLOAT16) else ["config"]
+            for kind in kinds:
+                srcs = make_inputs(rng, dtype, count, op, n, kind)
+                d = [to_dev(s) for s in srcs]
+                for lp, impl, keep, quirk in lp_variants(dtype):
+                    out = torch.empty_like(d[0])
+                    comp.comp_reduce_n(dtype, op, d, out, count, lp_mode=lp, bf16_impl=impl)
+                    torch.cuda.synchronize()
+                    want = O.reduce_n(srcs, dtype, op, keep=keep, quirk_tail=quirk, bf16_impl=impl)
+                    assert_same(to_host(out, O.NP_STORAGE[dtype]), want, dtype,
+                                f"dtype={O.DTYPE_NAMES[dtype]} op={O.OP_NAMES[op]} n={n} count={count} "
+                                f"kind={kind} lp={lp} impl={impl}")
+
+
+@pytest.mark.parametrize("fam,dtype", [("bf16", O.BFLOAT16), ("fp16", O.FLOAT16)])
+def test_pairwise_against_reference_made_golden_vectors(comp, golden, fam, dtype):
+    """GPU result vs what the reference's ccl_bf16_reduce_impl_* / ccl_fp16_reduce_impl_* produced."""
+    import torch
+    impls = (1, 2) if fam == "bf16" else (3,)
+    checked = 0
+    for key in golden.files:
+        if not key.startswith(fam + "_") or not key.endswith("_in") or key.startswith("cvt"):
+            continue
+        stem = key[:-3]
+        if "specials" in stem:
+            continue
+        op = O.OP_NAMES.index(stem.split("_")[1])
+        a, b = golden[stem + "_in"], golden[stem + "_inout"]
+        for impl in impls:
+            da, db = to_dev(a), to_dev(b)
+            comp.comp_reduce(dtype, op, da, a.size, db, bf16_impl=impl)
+            torch.cuda.synchronize()
+            assert_same(to_host(db, np.uint16), golden[stem + f"_impl{impl}"], dtype, f"{stem} impl{impl}")
+            checked += 1
+    assert checked >= 4 * 11 * 2
+
+
+@pytest.mark.parametrize("fam,dtype", [("bf16", O.BFLOAT16), ("fp16", O.FLOAT16)])
+def test_special_value_pairs_against_golden(comp, golden, fam, dtype):
+    """Every pair of special values (zeros, denormals, infinities, quiet and signalling NaNs, extremes).
+    min/max must return the reference's operand bit for bit, NaN payloads included."""
+    import torch
+    impls = (1, 2) if fam == "bf16" else (3,)
+    a, b = golden[f"{fam}_specials_in"], golden[f"{fam}_specials_inout"]
+    for op in range(4):
+        for impl in impls:
+            da, db = to_dev(a), to_dev(b)
+            comp.comp_reduce(dtype, op, da, a.size, db, bf16_impl=impl)
+            torch.cuda.synchronize()
+            got = to_host(db, np.uint16)
+            want = golden[f"{fam}_specials_{O.OP_NAMES[op]}_impl{impl}"]
+            if op in (O.MIN, O.MAX):
+                assert (got == want).all(), (fam, op, impl, np.flatnonzero(got != want)[:8])
+            else:
+                assert_same(got, want, dtype, f"{fam} specials op={op} impl={impl}")
+    if fam == "bf16":   # scalar impl has no golden (not vector code): oracle, pinned by the recorded probes
+        for op in range(4):
+            da, db = to_dev(a), to_dev(b)
+            comp.comp_reduce(dtype, op, da, a.size, db, bf16_impl=0)
+            torch.cuda.synchronize()
+            want = O.comp_reduce(a, b, dtype, op, bf16_impl=0)
+            got = to_host(db, np.uint16)
+            if op in (O.MIN, O.MAX):
+                assert (got == want).all()
+            else:
+                assert_same(got, want, dtype)
+
+
+def test_recorded_probe_values_on_gpu(comp, probes):
+    """The known answers recorded from the real reference library, reproduced by the GPU path."""
+    import torch
+    hx = lambda s: np.uint16(int(s, 16))
+    p = probes["bf16_pairwise_sum"]
+    a = np.array([hx(x) for x in p["in"]], np.uint16)
+    for name, impl in (("scalar", 0), ("avx512f", 1), ("avx512bf", 2)):
+        db = to_dev(np.full(a.size, hx(p["inout"]), np.uint16))
+        comp.bf16_reduce(to_dev(a), a.size, db, O.SUM, bf16_impl=impl)
+        torch.cuda.synchronize()
+        assert [f"{v:04x}" for v in to_host(db, np.uint16)] == p[name]
+    p = probes["batch_reduce_bf16"]
+    cnt = p["count"]
+    buf = np.concatenate([np.full(cnt, hx(s), np.uint16) for s in p["slices"]])
+    offs = [i * cnt for i in range(4)]
+    d = to_dev(buf)
+    comp.comp_batch_reduce(d, offs, cnt, d, O.BFLOAT16, O.SUM, 1, bf16_impl=2)
+    torch.cuda.synchronize()
+    r = to_host(d, np.uint16)[:cnt]
+    assert all(f"{v:04x}" == p["keep_precision_1_body"] for v in r[:16]) and f"{r[16]:04x}" == p["keep_precision_1_tail"]
+    d = to_dev(buf)
+    comp.comp_batch_reduce(d, offs, cnt, d, O.BFLOAT16, O.SUM, 0, bf16_impl=2)
+    torch.cuda.synchronize()
+    assert all(f"{v:04x}" == p["keep_precision_0"] for v in to_host(d, np.uint16)[:cnt])
+    p = probes["fp16_pairwise_sum"]
+    a = np.array([hx(x) for x in p["in"]], np.uint16)
+    db = to_dev(np.array([hx(x) for x in p["inout"]], np.uint16))
+    comp.fp16_reduce(to_dev(a), a.size, db, O.SUM)
+    torch.cuda.synchronize()
+    assert [f"{v:04x}" for v in to_host(db, np.uint16)] == p["avx512f"]
+    for c in probes["int_wrap"]["cases"]:
+        dt = O.DTYPE_NAMES.index(c["dtype"])
+        np_t = O.NP_STORAGE[dt]
+        db = to_dev(np.array([c["inout"]] * 5, np_t))
+        comp.comp_reduce(dt, O.SUM, to_dev(np.array([c["in"]] * 5, np_t)), 5, db)
+        torch.cuda.synchronize()
+        assert (to_host(db, np_t) == np_t(c["out"])).all()
+    vals = {"nan": np.nan, "1": 1.0, "-0": -0.0, "+0": 0.0}
+    for dt, np_t in ((O.FLOAT32, np.float32), (O.FLOAT64, np.float64)):
+        for c in probes["fp_minmax_plain"]["cases"]:
+            db = to_dev(np.full(67, vals[c["inout"]], np_t))
+            comp.comp_reduce(dt, O.OP_NAMES.index(c["op"]), to_dev(np.full(67, vals[c["in"]], np_t)), 67, db)
+            torch.cuda.synchronize()
+            got = to_host(db, np_t)
+            w = np_t(vals[c["out"]])
+            assert (np.isnan(got).all() if np.isnan(w) else ((got == w).all() and (np.signbit(got) == np.signbit(w)).all())), c
+
+
+@pytest.mark.parametrize("dtype", [O.INT8, O.INT16, O.FLOAT32, O.FLOAT64, O.BFLOAT16, O.FLOAT16])
+def test_misaligned_and_inplace(comp, dtype):
+    """Buffers that share a misalignment modulo 16 bytes (head/tail lanes), buffers that do not (element
+    kernel), in-place output, output aliasing a later input."""
+    import torch
+    rng = np.random.default_rng(77 + dtype)
+    esz = O.DTYPE_SIZE[dtype]
+    np_t = O.NP_STORAGE[dtype]
+    count, n, pad = 5003, 4, 32
+    for op in (O.SUM, O.MAX):
+        srcs = make_inputs(rng, dtype, count, op, n)
+        want = O.reduce_n(srcs, dtype, op)
+        for shifts in ([3, 3, 3, 3, 3], [1, 1, 1, 1, 1], [0, 1, 2, 3, 5], [0, 0, 0, 0, 1]):
+            # payload j starts shifts[j] elements past a 16-byte boundary (pad elements are a multiple of 16 B)
+            big = []
+            for s_, sh in zip(srcs, shifts):
+                h = np.zeros(count + 2 * pad, np_t)
+                h[pad + sh:pad + sh + count] = s_
+                big.append(to_dev(h))
+            outbig = to_dev(np.zeros(count + 2 * pad, np_t))
+            ptrs = [b_.data_ptr() + (pad + sh) * esz for b_, sh in zip(big, shifts)]
+            lo = pad + shifts[4]
+            comp.comp_reduce_n(dtype, op, ptrs, outbig.data_ptr() + lo * esz, count)
+            torch.cuda.synchronize()
+            o = to_host(outbig, np_t)
+            assert_same(o[lo:lo + count], want, dtype, f"shifts={shifts}")
+            assert (o[:lo] == 0).all() and (o[lo + count:] == 0).all(), "wrote outside the destination"
+        d = [to_dev(s) for s in srcs]
+        comp.comp_reduce_n(dtype, op, d, d[0], count)          # in place on the own buffer
+        torch.cuda.synchronize()
+        assert_same(to_host(d[0], np_t), want, dtype, "in place")
+        d = [to_dev(s) for s in srcs]
+        comp.comp_reduce_n(dtype, op, d, d[2], count)          # output aliases a later input
+        torch.cuda.synchronize()
+        assert_same(to_host(d[2], np_t), want, dtype, "alias")
+
+
+def test_batch_reduce_slices_keep_precision_tail(comp):
+    import torch
+    rng = np.random.default_rng(5)
+    for count in (1, 15, 16, 17, 31, 100, 1000, 4112 + 9):
+        for n in (1, 2, 4, 8):
+            for op in range(4):
+                slices = make_inputs(rng, O.BFLOAT16, count, op, n)
+                gap = 24
+                buf = np.zeros(n * (count + gap), np.uint16)
+                offs = [i * (count + gap) for i in range(n)]
+                for s, o in zip(slices, offs):
+                    buf[o:o + count] = s
+                for keep in (0, 1):
+                    for impl in (0, 1, 2):
+                        d = to_dev(buf)
+                        comp.comp_batch_reduce(d, offs, count, d, O.BFLOAT16, op, keep, bf16_impl=impl)
+                        torch.cuda.synchronize()
+                        want = O.batch_reduce(buf, offs, count, O.BFLOAT16, op, keep, bf16_impl=impl)
+                        assert_same(to_host(d, np.uint16), want, O.BFLOAT16, f"count={count} n={n} op={op} keep={keep} impl={impl}")
+
+
+def test_copy_and_converters(comp):
+    import torch
+    rng = np.random.default_rng(9)
+    for nbytes in (1, 15, 16, 17, 4096, 100003, 1 << 20):
+        for sa, sb in ((0, 0), (3, 3), (1, 2), (8, 0)):
+            src = rng.integers(0, 256, nbytes + 64, dtype=np.uint8)
+            for nt in (False, True):
+                ds, dd = to_dev(src), to_dev(np.zeros(nbytes + 64, np.uint8))
+                comp.comp_copy(ds.data_ptr() + sa, dd.data_ptr() + sb, nbytes, use_nontemporal=nt)
+                torch.cuda.synchronize()
+                got = to_host(dd, np.uint8)
+                assert (got[sb:sb + nbytes] == src[sa:sa + nbytes]).all()
+                assert (got[:sb] == 0).all() and (got[sb + nbytes:] == 0).all()
+    L = O.lib()
+    for count in (1, 5, 16, 22, 1000, 65536 + 7):
+        f32 = rng.integers(0, 2**32, count, dtype=np.uint32)
+        f32[:min(count, 6)] = np.array([1, 0x007FFFFF, 0x7FC00000, 0x7F800001, 0x7F7FFFFF, 0x3F808000], np.uint32)[:min(count, 6)]
+        if count >= 22:
+            f32[16:22] = f32[:6]
+        for impl in (0, 1, 2):
+            want = np.empty(count, np.uint16)
+            L.orc_convert_fp32_to_bf16_arrays(f32.ctypes.data, want.ctypes.data, count, impl)
+            d = to_dev(np.zeros(count, np.uint16))
+            comp.convert_fp32_to_bf16_arrays(to_dev(f32), d, count, bf16_impl=impl)
+            torch.cuda.synchronize()
+            assert (to_host(d, np.uint16) == want).all(), (count, impl)
+        h = rng.integers(0, 65536, count, dtype=np.uint16)
+        d = to_dev(np.zeros(count, np.uint32))
+        comp.convert_bf16_to_fp32_arrays(to_dev(h), d, count)
+        torch.cuda.synchronize()
+        assert (to_host(d, np.uint32) == (h.astype(np.uint32) << 16)).all()
+
+
+def test_bf16_narrowing_exhaustive_on_gpu(comp):
+    """All 2^32 fp32 patterns through the GPU's round-to-nearest-even narrowing vs the oracle (itself
+    exhaustively equal to VCVTNEPS2BF16)."""
+    import torch
+    L = O.lib()
+    chunk = 1 << 26
+    d_out = torch.empty(chunk, dtype=torch.int16, device="cuda")
+    want = np.empty(chunk, np.uint16)
+    for c in range(0, 1 << 32, chunk):
+        x = torch.arange(c, c + chunk, dtype=torch.int64, device="cuda")
+        src = torch.where(x >= 2**31, x - 2**32, x).to(torch.int32)      # the fp32 bit pattern as int32
+        comp.convert_fp32_to_bf16_arrays(src, d_out, chunk, bf16_impl=2)
+        torch.cuda.synchronize()
+        host = np.arange(c, c + chunk, dtype=np.uint64).astype(np.uint32)
+        L.orc_convert_fp32_to_bf16_arrays(host.ctypes.data, want.ctypes.data, chunk, 2)
+        got = to_host(d_out, np.uint16)
+        assert (got == want).all(), hex(c + int(np.flatnonzero(got != want)[0]))
+
+
+@pytest.mark.parametrize("dtype,impl", [(O.FLOAT16, 3), (O.BFLOAT16, 2)])
+def test_all_pairs_of_16bit_values_sum_and_prod(comp, dtype, impl):
+    """Every (in, inout) pair of 16-bit patterns -- 2^32 pairs -- through the pairwise GPU kernel."""
+    import torch
+    allv = np.arange(65536, dtype=np.uint16)
+    rows = 512
+    a = np.tile(allv, rows)
+    da = to_dev(a)
+    for op in (O.SUM, O.PROD):
+        for r0 in range(0, 65536, rows):
+            b = np.repeat(allv[r0:r0 + rows], 65536)
+            db = to_dev(b)
+            comp.comp_reduce(dtype, op, da, a.size, db, bf16_impl=impl)
+            torch.cuda.synchronize()
+            want = O.reduce_n([b, a], dtype, op, bf16_impl=impl, fp16_impl=3, threads=16)
+            assert_same(to_host(db, np.uint16), want, dtype, f"op={op} rows from {r0}")
+
+
+def test_arguments_and_errors(comp):
+    import torch
+    L = comp.lib()
+    assert comp.datatype_size(O.BFLOAT16) == 2 and comp.datatype_size(99) == 0
+    assert [comp.datatype_name(i) for i in range(12)] == O.DTYPE_NAMES
+    assert [comp.reduction_to_str(i) for i in range(6)] == ["sum", "prod", "min", "max", "custom", "unknown"]
+    assert comp.kernel_name("reduce_monolithic_kernel_7", O.BFLOAT16, O.SUM) == "reduce_monolithic_kernel_7_bfloat16_sum"
+    # count 0 succeeds without touching pointers (comp.cpp:132-134), even with a bad dtype
+    assert L.mi_ccl_comp_reduce(99, 0, None, 0, None, 2, None) == 0
+    x = torch.zeros(64, dtype=torch.int32, device="cuda")
+    assert L.mi_ccl_comp_reduce(99, 0, x.data_ptr(), 4, x.data_ptr(), 2, None) == comp.INVALID_ARGUMENTS
+    assert L.mi_ccl_comp_reduce(O.INT32, 4, x.data_ptr(), 4, x.data_ptr(), 2, None) == comp.INVALID_ARGUMENTS  # custom
+    assert L.mi_ccl_comp_reduce(O.INT32, 0, None, 4, x.data_ptr(), 2, None) == comp.INVALID_ARGUMENTS
+    assert L.mi_ccl_comp_reduce(O.INT32, 0, x.data_ptr() + 2, 4, x.data_ptr(), 2, None) == comp.INVALID_ARGUMENTS
+    with pytest.raises(comp.CclError):
+        comp.comp_reduce_n(O.FLOAT32, O.SUM, [x], x, 4, lp_mode=comp.LP_KEEP_PRECISION)   # keep needs bfloat16
+    with pytest.raises(comp.CclError):
+        comp.comp_reduce_n(O.INT32, O.SUM, [x] * 65, x, 4)
+    torch.cuda.synchronize()
+    assert (x == 0).all()
