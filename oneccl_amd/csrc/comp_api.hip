@@ -41,7 +41,28 @@ static std::atomic<int> g_waves_per_cu{ 8 };
 static std::atomic<int> g_max_blocks{ 0 };
 static std::atomic<int> g_xcd_chunked{ 0 };
 static std::atomic<int> g_variant{ 0 };
+static std::atomic<long> g_phased_min_bytes{ 1L << 30 };
 static std::atomic<int> g_num_cus[64];
+
+// Barrier words of the phased kernel: one copy per device (each GPU holds its own instance of a
+// __device__ variable at its own address), looked up once per device.
+static __device__ PhaseSync g_phase_sync;
+static std::atomic<PhaseSync*> g_phase_sync_ptr[64];
+
+static PhaseSync* phase_sync() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        return nullptr;
+    PhaseSync* p = g_phase_sync_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        void* sym = nullptr;
+        if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_phase_sync)) != hipSuccess)
+            return nullptr;
+        p = (PhaseSync*)sym;
+        g_phase_sync_ptr[dev].store(p, std::memory_order_release);
+    }
+    return p;
+}
 
 static int num_cus() {
     int dev = 0;
@@ -63,6 +84,8 @@ Tuning current_tuning() {
     t.xcd_chunked = g_xcd_chunked.load(std::memory_order_relaxed);
     t.variant = g_variant.load(std::memory_order_relaxed);
     t.num_cus = num_cus();
+    t.phased_min_bytes = g_phased_min_bytes.load(std::memory_order_relaxed);
+    t.sync = phase_sync();
     return t;
 }
 
@@ -398,8 +421,12 @@ int mi_ccl_set_param(const char* name, long value) {
         g_xcd_chunked.store((int)value);
         return MI_CCL_SUCCESS;
     }
-    if (!strcmp(name, "variant") && value >= 0 && value <= 16) {
+    if (!strcmp(name, "variant") && (value == 0 || value == 1 || value == 2 || value == 4 || value == 8)) {
         g_variant.store((int)value);
+        return MI_CCL_SUCCESS;
+    }
+    if (!strcmp(name, "phased_min_bytes") && value >= 0) {
+        g_phased_min_bytes.store(value);
         return MI_CCL_SUCCESS;
     }
     return MI_CCL_INVALID_ARGUMENTS;
@@ -416,6 +443,8 @@ long mi_ccl_get_param(const char* name) {
         return g_xcd_chunked.load();
     if (!strcmp(name, "variant"))
         return g_variant.load();
+    if (!strcmp(name, "phased_min_bytes"))
+        return g_phased_min_bytes.load();
     if (!strcmp(name, "num_cus"))
         return num_cus();
     return -1;

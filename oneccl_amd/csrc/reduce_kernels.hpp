@@ -34,8 +34,10 @@ struct Tuning {
     int waves_per_cu;   // resident 256-thread blocks per CU the grid is sized for
     int max_blocks;     // 0 = no cap
     int xcd_chunked;    // 1: each XCD streams one contiguous eighth of the buffer
-    int variant;        // kernel variant selector (unroll depth), 0 = default
+    int variant;        // 0 = automatic; 1, 2, 4 = streaming kernel with that unroll depth; 8 = phased kernel
     int num_cus;
+    long phased_min_bytes;   // automatic choice: phased kernel when (N + 1) * bytes per buffer reaches this
+    struct PhaseSync* sync;  // device-resident barrier words of the current device (may be null)
 };
 
 struct LaunchArgs {
@@ -322,6 +324,100 @@ reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint
     if (blockIdx.x == 0 && (head | tail)) reduce_edges<TR, OP>(src, N, dst, head, nvec, tail);
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Phased kernel for large buffers.
+//
+// HBM on this part loses about a quarter of its bandwidth when reads and writes are interleaved (an
+// 8-read + 1-write stream sustains ~5.5 TB/s where reads alone reach ~7.1 TB/s and writes alone ~6 TB/s).
+// This kernel keeps the two apart in time, chip-wide: one 1024-lane block per CU reduces kPhaseU vectors per
+// lane into LDS (read phase: HBM sees only reads), all blocks meet at a barrier, then every block streams
+// its LDS contents out (write phase: HBM sees only writes), and they meet again.
+//
+// The barrier carries no data between blocks -- it only aligns them in time -- so a block that waits too
+// long simply goes on (and stops waiting for the rest of the launch): the result is the same whether the
+// barrier holds or not, and no wave can spin forever.
+
+constexpr int kPhaseBlock = 1024;                 // 16 wavefronts, one block per CU
+constexpr int kPhaseU = 9;                        // vectors per lane per phase: 9 x 16 B x 1024 lanes = 144 KiB of LDS
+constexpr int kPhaseGroups = 16;                  // arrival counters (same-address atomics serialise)
+constexpr long long kPhaseSpinTicks = 20000;      // 100 MHz ticks: 200 us
+
+struct __attribute__((aligned(256))) PhaseWord {
+    unsigned v;
+    unsigned pad[63];
+};
+struct PhaseSync {
+    PhaseWord grp[kPhaseGroups];    // arrivals per group of blocks
+    PhaseWord top;                  // groups that are complete
+    PhaseWord rel;                  // barrier generation, bumped by the last arriver
+};
+
+#define MI_ALOAD(p) __hip_atomic_load((p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define MI_AADD(p, x) __hip_atomic_fetch_add((p), (x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+
+// Every block calls this the same number of times per launch, so the counters stay multiples of their
+// group sizes from launch to launch.  gen is the generation this block waits for.
+__device__ __forceinline__ void phase_barrier(PhaseSync* ps, unsigned gen, bool& give_up) {
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned per = gridDim.x / kPhaseGroups;
+        const unsigned old = MI_AADD(&ps->grp[blockIdx.x % kPhaseGroups].v, 1u);
+        if ((old + 1u) % per == 0u) {
+            const unsigned o2 = MI_AADD(&ps->top.v, 1u);
+            if ((o2 + 1u) % kPhaseGroups == 0u) MI_AADD(&ps->rel.v, 1u);
+        }
+        if (!give_up) {
+            const long long t0 = wall_clock64();
+            while ((int)(MI_ALOAD(&ps->rel.v) - gen) < 0) {
+                __builtin_amdgcn_s_sleep(1);
+                if (wall_clock64() - t0 > kPhaseSpinTicks) {
+                    give_up = true;
+                    break;
+                }
+            }
+        }
+    }
+    __syncthreads();
+}
+
+template <class TR, int OP, int N>
+__global__ void __launch_bounds__(kPhaseBlock)
+reduce_phased_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint32_t tail, PhaseSync* ps) {
+    typedef typename TR::elem_t E;
+    __shared__ u32x4 stage[kPhaseU * kPhaseBlock];
+    const u32x4* s[N];
+#pragma unroll
+    for (int j = 0; j < N; j++) s[j] = (const u32x4*)((const E*)src.p[j] + head);
+    u32x4* d = (u32x4*)((E*)dst + head);
+    const uint64_t gthreads = (uint64_t)gridDim.x * kPhaseBlock;
+    const uint64_t gtid = (uint64_t)blockIdx.x * kPhaseBlock + threadIdx.x;
+    const uint64_t per_phase = gthreads * kPhaseU;
+    bool give_up = false;
+    unsigned gen = 0;
+    if (threadIdx.x == 0) gen = MI_ALOAD(&ps->rel.v);     // read before this block's first arrival
+    for (uint64_t p0 = 0; p0 < nvec; p0 += per_phase) {
+        for (int u = 0; u < kPhaseU; u++) {
+            const uint64_t i = p0 + (uint64_t)u * gthreads + gtid;
+            if (i < nvec) {
+                u32x4 x[N];
+#pragma unroll
+                for (int j = 0; j < N; j++) x[j] = ld_stream(s[j] + i);
+                Accs<TR> a = vec_init<TR>(x[0]);
+#pragma unroll
+                for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j], a);
+                stage[u * kPhaseBlock + threadIdx.x] = vec_finish<TR>(a);
+            }
+        }
+        phase_barrier(ps, ++gen, give_up);      // all reads of this phase are done
+        for (int u = 0; u < kPhaseU; u++) {
+            const uint64_t i = p0 + (uint64_t)u * gthreads + gtid;
+            if (i < nvec) st_stream(d + i, stage[u * kPhaseBlock + threadIdx.x]);
+        }
+        phase_barrier(ps, ++gen, give_up);      // all writes of this phase are issued
+    }
+    if (blockIdx.x == 0 && (head | tail)) reduce_edges<TR, OP>(src, N, dst, head, nvec, tail);
+}
+
 // Run-time N (9..64): inputs are folded in one after the other, UNROLL vectors of each in flight.
 template <class TR, int OP, int UNROLL>
 __global__ void __launch_bounds__(kBlock)
@@ -405,9 +501,26 @@ struct HasUnrollVariants {
 };
 
 template <class TR, int OP, int N>
+inline hipError_t launch_phased(const LaunchArgs& a, uint32_t head, uint64_t nvec, uint32_t tail) {
+    SrcFixed<N> s;
+    for (int j = 0; j < N; j++) s.p[j] = a.srcs[j];
+    // one block per CU, a multiple of the arrival groups; all blocks must be resident together
+    int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
+    hipLaunchKernelGGL((reduce_phased_kernel<TR, OP, N>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.dst, head,
+                       nvec, tail, a.tune.sync);
+    return hipGetLastError();
+}
+
+template <class TR, int OP, int N>
 inline hipError_t launch_fixed_unroll(const LaunchArgs& a, uint32_t head, uint64_t nvec, uint32_t tail) {
     // loads in flight per lane = N * UNROLL
     constexpr int kDefault = (N <= 4) ? 4 : 2;
+    if constexpr (N >= 2) {
+        const bool can = a.tune.sync != nullptr && a.tune.num_cus >= kPhaseGroups;
+        const bool big = (long)((uint64_t)(N + 1) * nvec * 16u >> 1) >= (a.tune.phased_min_bytes >> 1);
+        if (can && (a.tune.variant == 8 || (a.tune.variant == 0 && big)))
+            return launch_phased<TR, OP, N>(a, head, nvec, tail);
+    }
     if constexpr (HasUnrollVariants<TR>::value) {
         switch (a.tune.variant) {
             case 1: return launch_fixed<TR, OP, N, 1>(a, head, nvec, tail);

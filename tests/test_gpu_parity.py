@@ -302,3 +302,33 @@ def test_arguments_and_errors(comp):
         comp.comp_reduce_n(O.INT32, O.SUM, [x] * 65, x, 4)
     torch.cuda.synchronize()
     assert (x == 0).all()
+
+
+@pytest.mark.parametrize("dtype,op,n", [(O.BFLOAT16, O.SUM, 8), (O.FLOAT32, O.SUM, 4), (O.INT8, O.SUM, 4),
+                                        (O.FLOAT16, O.SUM, 4), (O.INT64, O.MAX, 4), (O.FLOAT64, O.PROD, 2),
+                                        (O.FLOAT32, O.MIN, 3)])
+def test_phased_kernel_parity(comp, dtype, op, n):
+    """The large-buffer kernel (read phase into LDS / write phase, blocks aligned by a timing-only barrier)
+    forced on at sizes from a few elements to several phases, aligned and with head/tail lanes."""
+    import torch
+    rng = np.random.default_rng(300 + dtype)
+    esz = O.DTYPE_SIZE[dtype]
+    per_phase = comp.get_param("num_cus") * 1024 * 9 * (16 // esz)      # elements one phase covers
+    comp.set_param("variant", 8)
+    try:
+        for count, shift in ((5, 0), (1000, 1), (per_phase // 3 + 7, 0), (2 * per_phase + 12345, 3)):
+            if count * esz * (n + 1) > 6 << 30:
+                count = (6 << 30) // (esz * (n + 1))
+            srcs = make_inputs(rng, dtype, count + shift, op, n)
+            d = [to_dev(s) for s in srcs]
+            out = torch.zeros_like(d[0])
+            ptrs = [t.data_ptr() + shift * esz for t in d]
+            comp.comp_reduce_n(dtype, op, ptrs, out.data_ptr() + shift * esz, count,
+                               lp_mode=comp.LP_KEEP_PRECISION if dtype == O.BFLOAT16 else 0)
+            torch.cuda.synchronize()
+            want = O.reduce_n([s[shift:] for s in srcs], dtype, op, keep=1 if dtype == O.BFLOAT16 else 0, threads=16)
+            got = to_host(out, O.NP_STORAGE[dtype])
+            assert_same(got[shift:], want, dtype, f"phased count={count} shift={shift}")
+            assert (got[:shift] == 0).all()
+    finally:
+        comp.set_param("variant", 0)
