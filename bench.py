@@ -34,6 +34,9 @@ WORKLOADS = {
                     desc="8-input bf16 sum, 33,554,432 elements per buffer (64 MiB), rotating over 6 buffer sets"),
     "c1_fp32": dict(dtype="float32", n=2, count=16_777_216, keep=False, sets=8, in_place=True,
                     desc="2-input in-place fp32 sum, 16,777,216 elements per buffer (64 MiB), rotating over 8 buffer sets"),
+    # calibration for the rocprofv3 FETCH_SIZE / WRITE_SIZE counters: a plain copy of known size
+    "copy_ref": dict(dtype="bfloat16", n=1, count=1_003_782_144, keep=False, sets=1, copy=True,
+                     desc="mi_ccl_comp_copy of 2,007,564,288 bytes (counter calibration: reads and writes that many bytes)"),
 }
 
 # HBM traffic per launch of the default workload measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
@@ -140,11 +143,14 @@ def main():
 
     def step(i):
         s = sets[i % len(sets)]
-        comp.comp_reduce_n(dt, comp.SUM, s, outs[i % len(sets)], count, lp_mode=lp, stream=stream)
+        if w.get("copy"):
+            comp.comp_copy(s[0], outs[i % len(sets)], count * esz, use_nontemporal=True, stream=stream)
+        else:
+            comp.comp_reduce_n(dt, comp.SUM, s, outs[i % len(sets)], count, lp_mode=lp, stream=stream)
 
     # parity outside the timed region: GPU result of set 0 against the oracle on a sample
     base = None
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not w.get("copy"):
         snapshot = [b.clone() for b in sets[0]] if w.get("in_place") else sets[0]
         base, want, s_elems = cpu_baseline(torch, comp, w, snapshot, args.cpu_sample)
         step(0)

@@ -338,7 +338,7 @@ reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint
 // barrier holds or not, and no wave can spin forever.
 
 constexpr int kPhaseBlock = 1024;                 // 16 wavefronts, one block per CU
-constexpr int kPhaseU = 9;                        // vectors per lane per phase: 9 x 16 B x 1024 lanes = 144 KiB of LDS
+constexpr int kPhaseU = 10;                       // vectors per lane per phase: 10 x 16 B x 1024 lanes = 160 KiB, all of a CU's LDS
 constexpr int kPhaseGroups = 16;                  // arrival counters (same-address atomics serialise)
 constexpr long long kPhaseSpinTicks = 20000;      // 100 MHz ticks: 200 us
 
