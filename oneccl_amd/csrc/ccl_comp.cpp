@@ -1,0 +1,199 @@
+// C++ operator surface over the C ABI (see ccl_comp.hpp).
+#include "ccl_comp.hpp"
+
+#include <hip/hip_runtime.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "../../include/mi_ccl_comp.h"
+
+namespace {
+
+[[noreturn]] void fail(const std::string& what) {
+    throw ccl::exception(what);
+}
+
+ccl::status to_status(int rc, const char* what) {
+    if (rc == MI_CCL_SUCCESS)
+        return ccl::status::success;
+    fail(std::string(what) + ": " + mi_ccl_status_str(rc));
+}
+
+void* stream_of(ccl_sched* sched) {
+    return sched ? sched->stream : nullptr;
+}
+
+void check_hip(hipError_t e, const char* what) {
+    if (e != hipSuccess)
+        fail(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+ccl::env_data parse_env() {
+    ccl::env_data e;
+    if (const char* v = getenv("CCL_BF16")) {      // env.cpp:711-713
+        if (!strcmp(v, "scalar"))
+            e.bf16_impl_type = ccl_bf16_scalar;
+        else if (!strcmp(v, "avx512f"))
+            e.bf16_impl_type = ccl_bf16_avx512f;
+        else if (!strcmp(v, "avx512bf"))
+            e.bf16_impl_type = ccl_bf16_avx512bf;
+        else
+            fail(std::string("unexpected CCL_BF16 value: ") + v);
+    }
+    if (const char* v = getenv("CCL_FP16")) {      // env.cpp:715-720; f16c and avx512f give the same bits
+        if (!strcmp(v, "f16c"))
+            e.fp16_impl_type = ccl_fp16_f16c;
+        else if (!strcmp(v, "avx512f"))
+            e.fp16_impl_type = ccl_fp16_avx512f;
+        else
+            fail(std::string("unsupported FP16 impl type: ") + v);
+    }
+    return e;
+}
+
+// ccl::reduction::custom: the callback is host code, so both buffers are staged to the host and the result is
+// copied back, blocking, exactly as the reference does for device USM buffers (comp.cpp:163-194).
+void custom_on_host(ccl_sched* sched, const void* in_buf, size_t in_count, void* inout_buf, size_t* out_count,
+                    const ccl_datatype& dtype, ccl::reduction_fn fn, const ccl::fn_context* context) {
+    hipStream_t s = (hipStream_t)stream_of(sched);
+    const size_t bytes = in_count * dtype.size();
+    std::vector<unsigned char> h_in(bytes), h_io(bytes);
+    check_hip(hipMemcpyAsync(h_in.data(), in_buf, bytes, hipMemcpyDeviceToHost, s), "custom reduction: copy in");
+    check_hip(hipMemcpyAsync(h_io.data(), inout_buf, bytes, hipMemcpyDeviceToHost, s), "custom reduction: copy in");
+    check_hip(hipStreamSynchronize(s), "custom reduction: sync");
+    fn(h_in.data(), in_count, h_io.data(), out_count, dtype.idx(), context);
+    check_hip(hipMemcpyAsync(inout_buf, h_io.data(), bytes, hipMemcpyHostToDevice, s), "custom reduction: copy out");
+    check_hip(hipStreamSynchronize(s), "custom reduction: sync");
+}
+
+}  // namespace
+
+ccl::env_data& ccl::global_data::env() {
+    static ccl::env_data e = parse_env();
+    return e;
+}
+
+size_t ccl_datatype::size() const {
+    if (m_size == 0)
+        fail("non-positive datatype size 0");      // datatype.hpp:46-49
+    return m_size;
+}
+
+ccl_datatype_storage::ccl_datatype_storage() {
+    for (int i = 0; i < 12; i++) {
+        table[i] = ccl_datatype((ccl::datatype)i, mi_ccl_datatype_size(i));
+        names[i] = mi_ccl_datatype_name(i);
+    }
+}
+
+const ccl_datatype_storage& ccl_datatype_storage::instance() {
+    static ccl_datatype_storage s;
+    return s;
+}
+
+const ccl_datatype& ccl_datatype_storage::get(ccl::datatype idx) const {
+    int i = (int)idx;
+    if (i < 0 || i >= 12)
+        fail("unexpected datatype " + std::to_string(i));
+    return table[i];
+}
+
+const std::string& ccl_datatype_storage::name(const ccl_datatype& dtype) const {
+    return names[(int)get(dtype.idx()).idx()];
+}
+
+const char* ccl_reduction_to_str(ccl::reduction type) {
+    return mi_ccl_reduction_to_str((int)type);
+}
+
+ccl::status ccl_comp_copy(const void* in_buf, void* out_buf, size_t bytes, bool use_nontemporal, ccl_sched* sched) {
+    return to_status(mi_ccl_comp_copy(in_buf, out_buf, bytes, use_nontemporal ? 1 : 0, stream_of(sched)),
+                     "ccl_comp_copy");
+}
+
+ccl::status ccl_comp_reduce(ccl_sched* sched, const void* in_buf, size_t in_count, void* inout_buf,
+                            size_t* out_count, const ccl_datatype& dtype, ccl::reduction reduction,
+                            ccl::reduction_fn reduction_fn, const ccl::fn_context* context) {
+    if (!in_count)
+        return ccl::status::success;                                   // comp.cpp:132-134
+    if (reduction == ccl::reduction::custom) {
+        if (!reduction_fn)
+            fail("custom reduction requires user callback");          // comp.cpp:85
+        custom_on_host(sched, in_buf, in_count, inout_buf, out_count, dtype, reduction_fn, context);
+        return ccl::status::success;
+    }
+    // only the 16-bit paths report a count (bf16.cpp:94-96, fp16.cpp:48-50)
+    if (out_count && (dtype.idx() == ccl::datatype::bfloat16 || dtype.idx() == ccl::datatype::float16))
+        *out_count = in_count;
+    return to_status(mi_ccl_comp_reduce((int)dtype.idx(), (int)reduction, in_buf, in_count, inout_buf,
+                                        (int)ccl::global_data::env().bf16_impl_type, stream_of(sched)),
+                     "ccl_comp_reduce");
+}
+
+ccl::status ccl_comp_batch_reduce(const void* in_buf, const std::vector<size_t>& offsets, size_t in_count,
+                                  void* inout_buf, size_t* out_count, const ccl_datatype& dtype,
+                                  ccl::reduction reduction, ccl::reduction_fn reduction_fn,
+                                  const ccl::fn_context* context, int bf16_keep_precision_mode, float* tmp,
+                                  float* acc, ccl_sched* sched) {
+    (void)tmp;
+    (void)acc;
+    if (reduction == ccl::reduction::custom) {                         // chain of pairwise calls, comp.cpp:236-245
+        for (size_t i = 1; i < offsets.size(); i++)
+            ccl_comp_reduce(sched, (const char*)in_buf + dtype.size() * offsets[i], in_count, inout_buf, out_count,
+                            dtype, reduction, reduction_fn, context);
+        return ccl::status::success;
+    }
+    if (offsets.empty() || !in_count)
+        return ccl::status::success;
+    if (out_count && !bf16_keep_precision_mode && offsets.size() > 1 &&
+        (dtype.idx() == ccl::datatype::bfloat16 || dtype.idx() == ccl::datatype::float16))
+        *out_count = in_count;
+    return to_status(mi_ccl_comp_batch_reduce(in_buf, offsets.data(), offsets.size(), in_count, inout_buf,
+                                              (int)dtype.idx(), (int)reduction, bf16_keep_precision_mode,
+                                              (int)ccl::global_data::env().bf16_impl_type, stream_of(sched)),
+                     "ccl_comp_batch_reduce");
+}
+
+void ccl_bf16_reduce(const void* in_buf, size_t in_cnt, void* inout_buf, size_t* out_cnt, ccl::reduction reduction_op,
+                     ccl_sched* sched) {
+    if (out_cnt)
+        *out_cnt = in_cnt;                                             // bf16.cpp:94-96
+    to_status(mi_ccl_bf16_reduce(in_buf, in_cnt, inout_buf, (int)reduction_op,
+                                 (int)ccl::global_data::env().bf16_impl_type, stream_of(sched)),
+              "ccl_bf16_reduce");
+}
+
+void ccl_fp16_reduce(const void* in_buf, size_t in_cnt, void* inout_buf, size_t* out_cnt, ccl::reduction reduction_op,
+                     ccl_sched* sched) {
+    if (out_cnt)
+        *out_cnt = in_cnt;                                             // fp16.cpp:48-50
+    to_status(mi_ccl_fp16_reduce(in_buf, in_cnt, inout_buf, (int)reduction_op, stream_of(sched)), "ccl_fp16_reduce");
+}
+
+void ccl_convert_fp32_to_bf16_arrays(void* fp32_buf, void* bf16_buf, size_t count, ccl_sched* sched) {
+    to_status(mi_ccl_convert_fp32_to_bf16_arrays(fp32_buf, bf16_buf, count,
+                                                 (int)ccl::global_data::env().bf16_impl_type, stream_of(sched)),
+              "ccl_convert_fp32_to_bf16_arrays");
+}
+
+void ccl_convert_bf16_to_fp32_arrays(void* bf16_buf, float* fp32_buf, size_t count, ccl_sched* sched) {
+    to_status(mi_ccl_convert_bf16_to_fp32_arrays(bf16_buf, fp32_buf, count, stream_of(sched)),
+              "ccl_convert_bf16_to_fp32_arrays");
+}
+
+ccl::status ccl_comp_reduce_n(ccl_sched* sched, const void* own_buf, const std::vector<const void*>& peer_bufs,
+                              size_t count, void* out_buf, const ccl_datatype& dtype, ccl::reduction reduction,
+                              int bf16_keep_precision_mode) {
+    if (!count)
+        return ccl::status::success;
+    if (reduction == ccl::reduction::custom)
+        fail("custom reduction is not available for the N-input device reduce");
+    std::vector<const void*> srcs;
+    srcs.reserve(peer_bufs.size() + 1);
+    srcs.push_back(own_buf);
+    srcs.insert(srcs.end(), peer_bufs.begin(), peer_bufs.end());
+    int lp = bf16_keep_precision_mode ? MI_CCL_LP_KEEP_PRECISION : MI_CCL_LP_PAIRWISE;
+    return to_status(mi_ccl_comp_reduce_n((int)dtype.idx(), (int)reduction, srcs.data(), (int)srcs.size(), out_buf,
+                                          count, lp, (int)ccl::global_data::env().bf16_impl_type, stream_of(sched)),
+                     "ccl_comp_reduce_n");
+}

@@ -1,0 +1,154 @@
+// C++ operator surface of the MI355X reduction engine: the functions oneCCL's scheduler entries call
+// (src/comp/comp.hpp:23-51, src/comp/bf16/bf16.hpp:26-38, src/comp/fp16/fp16.hpp:21-25), with the same
+// names, argument order and meaning, running on device buffers through the C ABI of mi_ccl_comp.h.
+//
+// Differences a caller sees, all of them at the edges:
+//   * buffers are HIP device pointers; the work is enqueued on the HIP stream carried by ccl_sched
+//     (the reference's sched argument is only used to reach the stream, src/comp/comp.cpp:137-141);
+//     a null sched means the default stream.  Calls return once enqueued.
+//   * functions that have no sched argument in the reference (batch reduce, copy, the bf16/fp16 entry
+//     points, the array converters) take it as a trailing, defaulted argument.
+//   * an unknown dtype or reduction throws ccl::exception where the reference calls CCL_FATAL
+//     (std::terminate, src/comp/comp.cpp:56,113).
+//   * ccl::reduction::custom runs the user's host callback on host copies of the two buffers, as the
+//     reference does for device buffers (src/comp/comp.cpp:163-194).
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include <exception>
+#include <string>
+#include <vector>
+
+namespace ccl {
+
+// include/oneapi/ccl/types.hpp:41-69
+enum class reduction : int { sum = 0, prod, min, max, custom };
+enum class datatype : int {
+    int8 = 0, uint8, int16, uint16, int32, uint32, int64, uint64, float16, float32, float64, bfloat16,
+    last_predefined = bfloat16
+};
+
+// src/internal_types.hpp:29-37
+enum status : int { success = 0, out_of_resource, invalid_arguments, runtime_error, blocked_due_to_resize, last_value };
+
+// include/oneapi/ccl/types.hpp:116-124
+typedef struct {
+    const char* match_id;
+    const size_t offset;
+} fn_context;
+typedef void (*reduction_fn)(const void* in_buf, size_t in_count, void* inout_buf, size_t* out_count,
+                             ccl::datatype dtype, const ccl::fn_context* context);
+
+// include/oneapi/ccl/lp_types.hpp:27-67: 16-bit floats travel as raw bit patterns
+struct float16 {
+    constexpr float16() : data(0) {}
+    constexpr float16(uint16_t v) : data(v) {}
+    uint16_t get_data() const { return data; }
+    friend bool operator==(const float16& a, const float16& b) { return a.data == b.data; }
+    friend bool operator!=(const float16& a, const float16& b) { return a.data != b.data; }
+
+private:
+    uint16_t data;
+} __attribute__((packed));
+struct bfloat16 {
+    constexpr bfloat16() : data(0) {}
+    constexpr bfloat16(uint16_t v) : data(v) {}
+    uint16_t get_data() const { return data; }
+    friend bool operator==(const bfloat16& a, const bfloat16& b) { return a.data == b.data; }
+    friend bool operator!=(const bfloat16& a, const bfloat16& b) { return a.data != b.data; }
+
+private:
+    uint16_t data;
+} __attribute__((packed));
+
+// include/oneapi/ccl/exception.hpp:27-51
+class exception : public std::exception {
+    std::string msg;
+
+public:
+    exception(const std::string& info = "") : msg("oneCCL: " + info) {}
+    const char* what() const noexcept override { return msg.c_str(); }
+};
+
+}  // namespace ccl
+
+// src/comp/bf16/bf16_utils.hpp:26, src/comp/fp16/fp16_utils.hpp:26-32
+typedef enum { ccl_bf16_scalar = 0, ccl_bf16_avx512f, ccl_bf16_avx512bf } ccl_bf16_impl_type;
+typedef enum {
+    ccl_fp16_no_compiler_support = 0, ccl_fp16_no_hardware_support, ccl_fp16_f16c, ccl_fp16_avx512f, ccl_fp16_avx512fp16
+} ccl_fp16_impl_type;
+
+namespace ccl {
+// The two knobs of the reference's env_data that this path reads (src/common/env/env.cpp:711-720): which
+// CPU implementation's results to reproduce.  Defaults: avx512bf (round to nearest even) and avx512f;
+// CCL_BF16 = scalar | avx512f | avx512bf and CCL_FP16 = f16c | avx512f are read once, like the reference.
+struct env_data {
+    ccl_bf16_impl_type bf16_impl_type = ccl_bf16_avx512bf;
+    ccl_fp16_impl_type fp16_impl_type = ccl_fp16_avx512f;
+};
+struct global_data {
+    static env_data& env();
+};
+}  // namespace ccl
+
+// src/common/datatype/datatype.hpp:31-54 and the predefined table of datatype.cpp:79-106
+class ccl_datatype {
+public:
+    ccl_datatype() = default;
+    ccl_datatype(ccl::datatype idx, size_t size) : m_idx(idx), m_size(size) {}
+    ccl::datatype idx() const noexcept { return m_idx; }
+    size_t size() const;
+
+private:
+    ccl::datatype m_idx = ccl::datatype::int8;
+    size_t m_size = sizeof(int8_t);
+};
+class ccl_datatype_storage {
+public:
+    const ccl_datatype& get(ccl::datatype idx) const;
+    const std::string& name(const ccl_datatype& dtype) const;
+    static const ccl_datatype_storage& instance();
+
+private:
+    ccl_datatype_storage();
+    ccl_datatype table[12];
+    std::string names[12];
+};
+
+// What this path needs of a schedule: the stream its kernels go to (a hipStream_t).
+struct ccl_sched {
+    void* stream = nullptr;
+};
+
+// src/comp/comp.hpp:23-51
+ccl::status ccl_comp_copy(const void* in_buf, void* out_buf, size_t bytes, bool use_nontemporal = false,
+                          ccl_sched* sched = nullptr);
+
+ccl::status ccl_comp_reduce(ccl_sched* sched, const void* in_buf, size_t in_count, void* inout_buf,
+                            size_t* out_count, const ccl_datatype& dtype, ccl::reduction reduction,
+                            ccl::reduction_fn reduction_fn, const ccl::fn_context* context = nullptr);
+
+// tmp and acc (the reference's fp32 scratch arrays) are accepted and ignored: the kernel accumulates in registers.
+ccl::status ccl_comp_batch_reduce(const void* in_buf, const std::vector<size_t>& offsets, size_t in_count,
+                                  void* inout_buf, size_t* out_count, const ccl_datatype& dtype,
+                                  ccl::reduction reduction, ccl::reduction_fn reduction_fn,
+                                  const ccl::fn_context* context, int bf16_keep_precision_mode, float* tmp,
+                                  float* acc, ccl_sched* sched = nullptr);
+
+const char* ccl_reduction_to_str(ccl::reduction type);
+
+// src/comp/bf16/bf16.hpp:26-38, src/comp/fp16/fp16.hpp:21-25
+void ccl_bf16_reduce(const void* in_buf, size_t in_cnt, void* inout_buf, size_t* out_cnt, ccl::reduction reduction_op,
+                     ccl_sched* sched = nullptr);
+void ccl_fp16_reduce(const void* in_buf, size_t in_cnt, void* inout_buf, size_t* out_cnt, ccl::reduction reduction_op,
+                     ccl_sched* sched = nullptr);
+void ccl_convert_fp32_to_bf16_arrays(void* fp32_buf, void* bf16_buf, size_t count, ccl_sched* sched = nullptr);
+void ccl_convert_bf16_to_fp32_arrays(void* bf16_buf, float* fp32_buf, size_t count, ccl_sched* sched = nullptr);
+
+// The N-input local reduce of the device path (reduce_monolithic_kernel_N and friends, src/kernels/kernels.cl:269-421):
+// out = own OP peers[0] OP peers[1] ..., own first, peers in argument order.  keep_precision as in batch reduce.
+ccl::status ccl_comp_reduce_n(ccl_sched* sched, const void* own_buf, const std::vector<const void*>& peer_bufs,
+                              size_t count, void* out_buf, const ccl_datatype& dtype, ccl::reduction reduction,
+                              int bf16_keep_precision_mode = 0);

@@ -1,0 +1,223 @@
+// GPU test of the C++ operator surface (oneccl_amd/csrc/ccl_comp.hpp), written the way the reference's own
+// functional tests are (tests/functional/test_impl.hpp:242-324): every "rank" r fills its buffer with
+// c1*r + c2*buf_idx (+1 for prod), the buffers are reduced, and the result is checked against the closed
+// form within the reference's tolerance (test_impl.hpp:160-204) -- and, beyond what the reference checks,
+// bit for bit against the CPU oracle.  Exit status 0 = all checks passed.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <string>
+#include <vector>
+
+#include "../../oneccl_amd/csrc/ccl_comp.hpp"
+#include "../../oracle/ccl_comp_oracle.h"
+
+#define CK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { printf("HIP error %s at line %d\n", hipGetErrorString(e_), __LINE__); exit(2); } } while (0)
+static int g_fail = 0, g_checks = 0;
+#define EXPECT(cond, ...) do { g_checks++; if (!(cond)) { g_fail++; printf("FAIL line %d: ", __LINE__); printf(__VA_ARGS__); printf("\n"); } } while (0)
+
+static const ccl_datatype& DT(ccl::datatype d) { return ccl_datatype_storage::instance().get(d); }
+
+template <class T> struct DevBuf {
+    T* p = nullptr; size_t n;
+    explicit DevBuf(size_t n_) : n(n_) { CK(hipMalloc(&p, (n ? n : 1) * sizeof(T))); }
+    explicit DevBuf(const std::vector<T>& h) : n(h.size()) { CK(hipMalloc(&p, (n ? n : 1) * sizeof(T))); CK(hipMemcpy(p, h.data(), n * sizeof(T), hipMemcpyHostToDevice)); }
+    ~DevBuf() { (void)hipFree(p); }
+    std::vector<T> host() const { std::vector<T> h(n); CK(hipDeviceSynchronize()); CK(hipMemcpy(h.data(), p, n * sizeof(T), hipMemcpyDeviceToHost)); return h; }
+};
+
+static uint16_t to_lp(float v, ccl::datatype d) {
+    uint32_t u; memcpy(&u, &v, 4);
+    return d == ccl::datatype::bfloat16 ? orc_bf16_narrow_rne(u) : orc_fp16_narrow(u);
+}
+static float from_lp(uint16_t h, ccl::datatype d) {
+    uint32_t u = d == ccl::datatype::bfloat16 ? orc_bf16_widen(h) : orc_fp16_widen(h);
+    float f; memcpy(&f, &u, 4); return f;
+}
+
+// element of rank r's buffer, as the functional tests fill it (test.hpp:73-86, test_impl.hpp:242-252)
+static double fill_value(ccl::datatype d, int r, int buf_idx, ccl::reduction op) {
+    double c1 = 1, c2 = 1;
+    if (d == ccl::datatype::bfloat16) { c1 = 0.5; c2 = 1; }
+    if (d == ccl::datatype::float16) { c1 = 0.01; c2 = 0.01; }
+    return c1 * r + c2 * buf_idx + (op == ccl::reduction::prod ? 1 : 0);
+}
+
+template <class T>
+static void closed_form_case(ccl::datatype d, size_t count, int N, int buf_idx, ccl::reduction op, hipStream_t stream) {
+    const bool lp = d == ccl::datatype::bfloat16 || d == ccl::datatype::float16;
+    std::vector<std::vector<T>> send(N, std::vector<T>(count));
+    std::vector<double> vals(N);
+    for (int r = 0; r < N; r++) {
+        vals[r] = fill_value(d, r, buf_idx, op);
+        T x;
+        if (lp) { uint16_t h = to_lp((float)vals[r], d); memcpy(&x, &h, sizeof(T)); vals[r] = from_lp(h, d); }
+        else x = (T)vals[r];
+        for (size_t i = 0; i < count; i++) send[r][i] = x;
+    }
+    double expected = vals[0];
+    for (int r = 1; r < N; r++) {
+        if (op == ccl::reduction::sum) expected += vals[r];
+        else if (op == ccl::reduction::prod) expected *= vals[r];
+        else if (op == ccl::reduction::min) expected = fmin(expected, vals[r]);
+        else expected = fmax(expected, vals[r]);
+    }
+    // oracle: chain of pairwise calls, recv <- rank 0, then ranks 1..N-1 (reduce_scatter.cpp:111-136)
+    std::vector<T> want = send[0];
+    for (int r = 1; r < N; r++)
+        orc_comp_reduce(send[r].data(), count, want.data(), (int)d, (int)op, ORC_BF16_AVX512BF, ORC_FP16_AVX512F);
+    ccl_sched sched; sched.stream = stream;
+    // (1) chain of ccl_comp_reduce
+    {
+        DevBuf<T> recv(send[0]);
+        for (int r = 1; r < N; r++) {
+            DevBuf<T> in(send[r]);
+            size_t out_count = 12345;
+            ccl::status st = ccl_comp_reduce(&sched, in.p, count, recv.p, &out_count, DT(d), op, nullptr);
+            EXPECT(st == ccl::status::success, "status");
+            EXPECT(out_count == (lp ? count : (size_t)12345), "out_count semantics (only 16-bit paths report it)");
+            CK(hipStreamSynchronize(stream));
+        }
+        std::vector<T> got = recv.host();
+        EXPECT(memcmp(got.data(), want.data(), count * sizeof(T)) == 0, "chain vs oracle dtype %d op %d count %zu", (int)d, (int)op, count);
+        double g = lp ? from_lp(*(uint16_t*)&got[count - 1], d) : (double)got[count - 1];
+        double eps = d == ccl::datatype::bfloat16 ? 2 * pow(2, -7) : d == ccl::datatype::float16 ? 2 * pow(2, -10)
+                     : d == ccl::datatype::float32 ? pow(2, -23) : 0;
+        double le = log2((double)N) * eps, max_err = fabs(expected) * le / (1 - le);
+        EXPECT(fabs(g - expected) <= max_err + (lp ? fabs(expected) * eps : 0), "closed form dtype %d op %d: got %g expected %g", (int)d, (int)op, g, expected);
+    }
+    // (2) ccl_comp_batch_reduce over slices of one buffer (pairwise mode) and the N-input form
+    {
+        std::vector<T> all;
+        std::vector<size_t> offsets;
+        for (int r = 0; r < N; r++) { offsets.push_back(all.size()); all.insert(all.end(), send[r].begin(), send[r].end()); }
+        DevBuf<T> buf(all);
+        ccl_comp_batch_reduce(buf.p, offsets, count, buf.p, nullptr, DT(d), op, nullptr, nullptr, 0, nullptr, nullptr, &sched);
+        std::vector<T> got = buf.host();
+        EXPECT(memcmp(got.data(), want.data(), count * sizeof(T)) == 0, "batch reduce vs oracle dtype %d op %d", (int)d, (int)op);
+        EXPECT(memcmp(got.data() + count, all.data() + count, (all.size() - count) * sizeof(T)) == 0, "batch reduce touched an input slice");
+        std::vector<DevBuf<T>*> peers;
+        std::vector<const void*> pp;
+        DevBuf<T> own(send[0]), out(count);
+        for (int r = 1; r < N; r++) { peers.push_back(new DevBuf<T>(send[r])); pp.push_back(peers.back()->p); }
+        ccl_comp_reduce_n(&sched, own.p, pp, count, out.p, DT(d), op, 0);
+        std::vector<T> got2 = out.host();
+        EXPECT(memcmp(got2.data(), want.data(), count * sizeof(T)) == 0, "reduce_n vs oracle dtype %d op %d", (int)d, (int)op);
+        for (auto* p : peers) delete p;
+    }
+}
+
+static void custom_sum_i32(const void* in, size_t n, void* inout, size_t* out_count, ccl::datatype dt, const ccl::fn_context* ctx) {
+    const int32_t* a = (const int32_t*)in; int32_t* b = (int32_t*)inout;
+    for (size_t i = 0; i < n; i++) b[i] = 2 * b[i] + a[i];
+    if (out_count) *out_count = n;
+    (void)dt; (void)ctx;
+}
+
+int main() {
+    int ndev = 0; CK(hipGetDeviceCount(&ndev));
+    if (ndev < 1) { printf("no GPU\n"); return 2; }
+    hipStream_t stream; CK(hipStreamCreate(&stream));
+    const char* env_bf16 = getenv("CCL_BF16");
+    printf("bf16 impl %d (CCL_BF16=%s)\n", (int)ccl::global_data::env().bf16_impl_type, env_bf16 ? env_bf16 : "unset");
+
+    if (!env_bf16) {
+        const size_t sizes[] = { 17, 32771, 262144 };   // tests/functional/conf.cpp:51-53
+        const ccl::reduction ops[] = { ccl::reduction::sum, ccl::reduction::prod, ccl::reduction::min, ccl::reduction::max };
+        for (size_t count : sizes)
+            for (ccl::reduction op : ops)
+                for (int buf_idx : { 0, 3 }) {
+                    closed_form_case<int32_t>(ccl::datatype::int32, count, 4, buf_idx, op, stream);
+                    closed_form_case<float>(ccl::datatype::float32, count, 4, buf_idx, op, stream);
+                    closed_form_case<uint16_t>(ccl::datatype::float16, count, 4, buf_idx, op, stream);
+                    closed_form_case<uint16_t>(ccl::datatype::bfloat16, count, 4, buf_idx, op, stream);
+                }
+        closed_form_case<int8_t>(ccl::datatype::int8, 1000, 4, 1, ccl::reduction::sum, stream);
+        closed_form_case<uint64_t>(ccl::datatype::uint64, 1000, 4, 1, ccl::reduction::prod, stream);
+        closed_form_case<double>(ccl::datatype::float64, 1000, 4, 1, ccl::reduction::max, stream);
+    }
+
+    ccl_sched sched; sched.stream = stream;
+    // keep-precision batch reduce: 1 + 3 * 2^-8 in bf16 -> 3f82 in the body, 3f81 in the truncated tail (count 17)
+    {
+        const size_t count = 17;
+        std::vector<uint16_t> all;
+        std::vector<size_t> offsets;
+        const uint16_t v[4] = { 0x3f80, 0x3b80, 0x3b80, 0x3b80 };
+        for (int r = 0; r < 4; r++) { offsets.push_back(all.size()); all.insert(all.end(), count, v[r]); }
+        DevBuf<uint16_t> buf(all);
+        std::vector<float> scratch;     // the reference needs tmp/acc; here they may be null
+        ccl_comp_batch_reduce(buf.p, offsets, count, buf.p, nullptr, DT(ccl::datatype::bfloat16), ccl::reduction::sum,
+                              nullptr, nullptr, 1, nullptr, nullptr, &sched);
+        std::vector<uint16_t> got = buf.host();
+        std::vector<uint16_t> want(all.begin(), all.begin() + count);
+        std::vector<float> tmp(count), acc(count);
+        int impl = (int)ccl::global_data::env().bf16_impl_type;
+        orc_comp_batch_reduce(all.data(), offsets.data(), 4, count, want.data(), ORC_BFLOAT16, ORC_SUM, 1, tmp.data(), acc.data(), impl, ORC_FP16_AVX512F);
+        EXPECT(memcmp(got.data(), want.data(), count * 2) == 0, "keep-precision batch reduce vs oracle");
+        if (impl == ccl_bf16_avx512bf) EXPECT(got[0] == 0x3f82 && got[15] == 0x3f82 && got[16] == 0x3f81, "recorded values: body %04x tail %04x", got[0], got[16]);
+        else EXPECT(got[0] == 0x3f81 && got[16] == 0x3f81, "truncating impl: %04x %04x", got[0], got[16]);
+        // pairwise sum 1 + 1.5 * 2^-8: 3f81 with round-to-nearest-even, 3f80 with truncation
+        DevBuf<uint16_t> io(std::vector<uint16_t>(20, 0x3f80)), in(std::vector<uint16_t>(20, 0x3bc0));
+        size_t oc = 0;
+        ccl_bf16_reduce(in.p, 20, io.p, &oc, ccl::reduction::sum, &sched);
+        EXPECT(oc == 20, "ccl_bf16_reduce out_cnt");
+        EXPECT(io.host()[7] == (impl == ccl_bf16_avx512bf ? 0x3f81 : 0x3f80), "pairwise rounding per impl: %04x", io.host()[7]);
+    }
+    // custom reduction: the host callback sees host copies; a missing callback throws
+    {
+        std::vector<int32_t> a(1000), b(1000);
+        for (int i = 0; i < 1000; i++) { a[i] = i; b[i] = 7 - i; }
+        DevBuf<int32_t> da(a), db(b);
+        size_t oc = 0;
+        ccl_comp_reduce(&sched, da.p, 1000, db.p, &oc, DT(ccl::datatype::int32), ccl::reduction::custom, custom_sum_i32);
+        std::vector<int32_t> got = db.host();
+        bool ok = oc == 1000;
+        for (int i = 0; i < 1000; i++) ok = ok && got[i] == 2 * (7 - i) + i;
+        EXPECT(ok, "custom reduction result");
+        bool threw = false;
+        try { ccl_comp_reduce(&sched, da.p, 1000, db.p, &oc, DT(ccl::datatype::int32), ccl::reduction::custom, nullptr); }
+        catch (const ccl::exception& e) { threw = strstr(e.what(), "custom reduction requires user callback") != nullptr; }
+        EXPECT(threw, "missing callback must throw ccl::exception");
+    }
+    // in_count == 0 succeeds without looking at anything; an unknown dtype throws
+    {
+        EXPECT(ccl_comp_reduce(nullptr, nullptr, 0, nullptr, nullptr, ccl_datatype((ccl::datatype)77, 3), ccl::reduction::sum, nullptr) == ccl::status::success, "count 0");
+        EXPECT(ccl_comp_copy(nullptr, nullptr, 0) == ccl::status::success, "copy 0 bytes");
+        DevBuf<int32_t> x(16);
+        bool threw = false;
+        try { ccl_comp_reduce(&sched, x.p, 16, x.p, nullptr, ccl_datatype((ccl::datatype)77, 4), ccl::reduction::sum, nullptr); }
+        catch (const ccl::exception&) { threw = true; }
+        EXPECT(threw, "unknown dtype must throw");
+        EXPECT(!strcmp(ccl_reduction_to_str(ccl::reduction::custom), "custom") && !strcmp(ccl_reduction_to_str((ccl::reduction)9), "unknown"), "reduction names");
+        EXPECT(DT(ccl::datatype::bfloat16).size() == 2 && ccl_datatype_storage::instance().name(DT(ccl::datatype::uint64)) == "uint64", "datatype table");
+    }
+    // copy and array converters
+    {
+        std::vector<uint8_t> src(100003);
+        for (size_t i = 0; i < src.size(); i++) src[i] = (uint8_t)(i * 7 + 1);
+        DevBuf<uint8_t> a(src), b(src.size());
+        ccl_comp_copy(a.p + 1, b.p + 1, src.size() - 1, true, &sched);
+        std::vector<uint8_t> got = b.host();
+        EXPECT(memcmp(got.data() + 1, src.data() + 1, src.size() - 1) == 0, "copy");
+        std::vector<uint32_t> f(22, 0x3f808000u);
+        f[1] = 0x007fffffu; f[17] = 0x007fffffu; f[2] = 0x7f800001u; f[18] = 0x7f800001u;
+        DevBuf<uint32_t> df(f); DevBuf<uint16_t> dh(22);
+        ccl_convert_fp32_to_bf16_arrays(df.p, dh.p, 22, &sched);
+        std::vector<uint16_t> h = dh.host(), want(22);
+        orc_convert_fp32_to_bf16_arrays(f.data(), want.data(), 22, (int)ccl::global_data::env().bf16_impl_type);
+        EXPECT(memcmp(h.data(), want.data(), 44) == 0, "fp32->bf16 arrays (tail truncates): %04x %04x %04x %04x", h[1], h[17], h[2], h[18]);
+        DevBuf<uint32_t> back(22);
+        ccl_convert_bf16_to_fp32_arrays(dh.p, (float*)back.p, 22, &sched);
+        std::vector<uint32_t> w = back.host();
+        bool ok = true;
+        for (int i = 0; i < 22; i++) ok = ok && w[i] == ((uint32_t)h[i] << 16);
+        EXPECT(ok, "bf16->fp32 arrays");
+    }
+    CK(hipStreamDestroy(stream));
+    printf("%d checks, %d failed\n", g_checks, g_fail);
+    return g_fail ? 1 : 0;
+}
