@@ -39,9 +39,9 @@ WORKLOADS = {
                      desc="mi_ccl_comp_copy of 2,007,564,288 bytes (counter calibration: reads and writes that many bytes)"),
 }
 
-# HBM traffic per launch of the default workload measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (see profiles/); None until measured.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two runs), each scaled by what the
+# same counter reads for a plain copy of known size (x2.0000 and x1.0000): profiles/reduce_phased_bf16_sum_8x2GiB.md.
+MEASURED_TRAFFIC_BYTES = {"c5_bf16": (15_684_328 + 1_965_092) * 1024}
 
 
 def make_buffers(torch, w, seed):

@@ -1,0 +1,133 @@
+#!/usr/bin/env python3
+"""Measures the other benchmark configurations on one MI355X (bench.py covers the headline one):
+
+  C1  2-input in-place fp32 sum, 16,777,216 elements per buffer
+  C2  8-input bf16 sum, 33,554,432 elements per buffer
+  C3  datatype x op sweep, 4 inputs, 1 KiB ... 1 GiB per buffer (x4 steps)
+  C4  fusion: 256 bf16 tensors, counts log-uniform [2,048, 2,097,152], 256-byte aligned offsets, 8-input sum against
+      7 peer fusion buffers: pack + reduce + unpack, and the fused single pass
+
+    python bench_configs.py [--out gpurun_out/configs.json] [--skip c3]
+
+Writes a JSON file and prints a markdown table.  Bytes are algorithmic: (N + 1) x chunk for a reduce, 2 x payload
+for pack and unpack.  Buffers of 64 MiB rotate over several sets so that the 256 MB Infinity Cache cannot hold them.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+
+def timed(torch, fn, steps, warm):
+    for i in range(warm):
+        fn(i)
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(steps):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps * 1e3      # us
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--out", default=os.path.join(ROOT, "gpurun_out", "configs.json"))
+    ap.add_argument("--skip", default="")
+    args = ap.parse_args()
+    import numpy as np
+    import torch
+    import oneccl_amd.comp as comp
+    comp.lib()
+    torch.cuda.set_device(0)
+    res = {}
+    rows = []
+
+    def add(name, us, byts, extra=""):
+        gbs = byts / us / 1e3
+        res[name] = dict(us=round(us, 2), GBps=round(gbs, 1), bytes=byts, pct_hbm_peak=round(gbs / 80.0, 2))
+        rows.append(f"| {name} | {byts:,} | {us:,.1f} | {gbs:,.0f} | {gbs / 80.0:.1f} % | {extra} |")
+
+    # ---- C1
+    n1 = 16_777_216
+    sets = [[torch.empty(n1, dtype=torch.float32, device="cuda").uniform_(-1, 1) for _ in range(2)] for _ in range(8)]
+    us = timed(torch, lambda i: comp.comp_reduce(comp.FLOAT32, comp.SUM, sets[i % 8][1], n1, sets[i % 8][0]), 64, 16)
+    add("C1 fp32 sum, 2 inputs in place, 64 MiB", us, 3 * n1 * 4, "8 rotating buffer sets")
+    del sets
+    # ---- C2
+    n2 = 33_554_432
+    sets = [[torch.empty(n2, dtype=torch.bfloat16, device="cuda").normal_(0, 1) for _ in range(8)] for _ in range(6)]
+    outs = [torch.empty_like(s[0]) for s in sets]
+    us = timed(torch, lambda i: comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, sets[i % 6], outs[i % 6], n2,
+                                                  lp_mode=comp.LP_KEEP_PRECISION), 64, 16)
+    add("C2 bf16 sum, 8 inputs, 64 MiB (fp32 acc, RNE once)", us, 9 * n2 * 2, "6 rotating buffer sets")
+    us = timed(torch, lambda i: comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, sets[0], outs[0], n2,
+                                                  lp_mode=comp.LP_KEEP_PRECISION), 64, 16)
+    add("C2 same, one buffer set (Infinity Cache assisted)", us, 9 * n2 * 2, "")
+    del sets, outs
+    # ---- C3
+    if "c3" not in args.skip:
+        cases = [("int8 sum", comp.INT8, comp.SUM, torch.int8, 1), ("int32 sum", comp.INT32, comp.SUM, torch.int32, 4),
+                 ("int64 max", comp.INT64, comp.MAX, torch.int64, 8), ("fp16 sum", comp.FLOAT16, comp.SUM, torch.float16, 2),
+                 ("fp32 min", comp.FLOAT32, comp.MIN, torch.float32, 4), ("fp64 prod", comp.FLOAT64, comp.PROD, torch.float64, 8)]
+        for label, dt, op, tdt, esz in cases:
+            for k in range(11):
+                size = 1024 * 4 ** k
+                cnt = size // esz
+                nsets = max(1, min(8, (1 << 30) // (5 * size)))
+                if tdt.is_floating_point:
+                    lo, hi = (0.9, 1.1) if op == comp.PROD else (-2.0, 2.0)
+                    mk = lambda: torch.empty(cnt, dtype=torch.float32, device="cuda").uniform_(lo, hi).to(tdt)
+                else:
+                    info = torch.iinfo(tdt)
+                    mk = lambda: torch.randint(info.min, info.max, (cnt,), dtype=tdt, device="cuda")
+                ss = [[mk() for _ in range(4)] for _ in range(nsets)]
+                oo = [torch.empty_like(s[0]) for s in ss]
+                steps = 200 if size <= (1 << 22) else 30
+                us = timed(torch, lambda i: comp.comp_reduce_n(dt, op, ss[i % nsets], oo[i % nsets], cnt), steps, 10)
+                add(f"C3 {label}, 4 inputs, {size >> 10} KiB per buffer", us, 5 * size, f"{nsets} set(s)")
+                del ss, oo
+    # ---- C4
+    rng = np.random.default_rng(4)
+    counts = [int(round(math.exp(rng.uniform(math.log(2048), math.log(2_097_152))))) for _ in range(256)]
+    payload = sum(counts) * 2
+    plan = comp.FusionPlan(counts, comp.BFLOAT16, 256)
+    nelem = plan.nbytes // 2
+    tens = [torch.empty(c, dtype=torch.bfloat16, device="cuda").normal_(0, 0.02) for c in counts]
+    outs = [torch.empty_like(t) for t in tens]
+    fb = torch.empty(nelem, dtype=torch.bfloat16, device="cuda")
+    peers = [torch.empty(nelem, dtype=torch.bfloat16, device="cuda").normal_(0, 0.02) for _ in range(7)]
+    us_pack = timed(torch, lambda i: plan.pack(tens, fb), 50, 10)
+    us_red = timed(torch, lambda i: comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, [fb] + peers, fb, nelem,
+                                                      lp_mode=comp.LP_KEEP_PRECISION), 50, 10)
+    us_unpack = timed(torch, lambda i: plan.unpack(fb, outs), 50, 10)
+
+    def three(i):
+        plan.pack(tens, fb)
+        comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, [fb] + peers, fb, nelem, lp_mode=comp.LP_KEEP_PRECISION)
+        plan.unpack(fb, outs)
+    us_three = timed(torch, three, 50, 10)
+    us_fused = timed(torch, lambda i: plan.reduce(comp.SUM, tens, peers, outs, lp_mode=comp.LP_KEEP_PRECISION), 50, 10)
+    add(f"C4 pack, 256 tensors, payload {payload:,} B", us_pack, 2 * payload)
+    add("C4 8-input reduce over the fusion buffer", us_red, 9 * payload)
+    add("C4 unpack", us_unpack, 2 * payload)
+    add("C4 pack + reduce + unpack (3 launches)", us_three, 13 * payload)
+    add("C4 fused single pass (tensors + 7 peers -> tensors)", us_fused, 9 * payload,
+        f"{us_three / us_fused:.2f}x faster than the 3-step sequence")
+    plan.close()
+
+    os.makedirs(os.path.dirname(args.out), exist_ok=True)
+    with open(args.out, "w") as f:
+        json.dump(res, f, indent=1)
+    print("| configuration | algorithmic bytes | us per call | GB/s | of 8 TB/s | note |")
+    print("|---|---|---|---|---|---|")
+    print("\n".join(rows))
+
+
+if __name__ == "__main__":
+    main()
