@@ -380,10 +380,32 @@ __device__ __forceinline__ void phase_barrier(PhaseSync* ps, unsigned gen, bool&
     __syncthreads();
 }
 
+// Vectors per lane per phase that are staged in registers on top of the kPhaseU staged in LDS.  Register staging
+// needs fully unrolled code, so it is switched on per traits class (specialise before instantiating).
+template <class TR>
+struct PhaseRegs {
+    static constexpr int value = 16;
+};
+
+template <class TR, int OP, int N>
+__device__ __forceinline__ u32x4 reduce_one_vector(const u32x4* const (&s)[N], uint64_t i) {
+    u32x4 x[N];
+#pragma unroll
+    for (int j = 0; j < N; j++) x[j] = ld_stream(s[j] + i);
+    Accs<TR> a = vec_init<TR>(x[0]);
+#pragma unroll
+    for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j], a);
+    return vec_finish<TR>(a);
+}
+
 template <class TR, int OP, int N>
 __global__ void __launch_bounds__(kPhaseBlock)
 reduce_phased_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint32_t tail, PhaseSync* ps) {
     typedef typename TR::elem_t E;
+    // register budget of a 1024-lane block is 128 per lane: N in-flight loads (4 registers each) plus addressing
+    // and accumulators leave room for this many staged vectors
+    constexpr int kFit = (N <= 2) ? 12 : (N <= 4) ? 10 : (N <= 6) ? 8 : 6;
+    constexpr int R = PhaseRegs<TR>::value < kFit ? PhaseRegs<TR>::value : kFit;
     __shared__ u32x4 stage[kPhaseU * kPhaseBlock];
     const u32x4* s[N];
 #pragma unroll
@@ -391,26 +413,29 @@ reduce_phased_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, u
     u32x4* d = (u32x4*)((E*)dst + head);
     const uint64_t gthreads = (uint64_t)gridDim.x * kPhaseBlock;
     const uint64_t gtid = (uint64_t)blockIdx.x * kPhaseBlock + threadIdx.x;
-    const uint64_t per_phase = gthreads * kPhaseU;
+    const uint64_t per_phase = gthreads * (kPhaseU + R);
     bool give_up = false;
     unsigned gen = 0;
     if (threadIdx.x == 0) gen = MI_ALOAD(&ps->rel.v);     // read before this block's first arrival
     for (uint64_t p0 = 0; p0 < nvec; p0 += per_phase) {
-        for (int u = 0; u < kPhaseU; u++) {
+        u32x4 r[R > 0 ? R : 1];
+#pragma unroll
+        for (int u = 0; u < R; u++) {
             const uint64_t i = p0 + (uint64_t)u * gthreads + gtid;
-            if (i < nvec) {
-                u32x4 x[N];
-#pragma unroll
-                for (int j = 0; j < N; j++) x[j] = ld_stream(s[j] + i);
-                Accs<TR> a = vec_init<TR>(x[0]);
-#pragma unroll
-                for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j], a);
-                stage[u * kPhaseBlock + threadIdx.x] = vec_finish<TR>(a);
-            }
+            if (i < nvec) r[u] = reduce_one_vector<TR, OP, N>(s, i);
+        }
+        for (int u = 0; u < kPhaseU; u++) {
+            const uint64_t i = p0 + (uint64_t)(R + u) * gthreads + gtid;
+            if (i < nvec) stage[u * kPhaseBlock + threadIdx.x] = reduce_one_vector<TR, OP, N>(s, i);
         }
         phase_barrier(ps, ++gen, give_up);      // all reads of this phase are done
-        for (int u = 0; u < kPhaseU; u++) {
+#pragma unroll
+        for (int u = 0; u < R; u++) {
             const uint64_t i = p0 + (uint64_t)u * gthreads + gtid;
+            if (i < nvec) st_stream(d + i, r[u]);
+        }
+        for (int u = 0; u < kPhaseU; u++) {
+            const uint64_t i = p0 + (uint64_t)(R + u) * gthreads + gtid;
             if (i < nvec) st_stream(d + i, stage[u * kPhaseBlock + threadIdx.x]);
         }
         phase_barrier(ps, ++gen, give_up);      // all writes of this phase are issued

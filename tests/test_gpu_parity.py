@@ -316,7 +316,7 @@ def test_phased_kernel_parity(comp, dtype, op, n):
     per_phase = comp.get_param("num_cus") * 1024 * 9 * (16 // esz)      # elements one phase covers
     comp.set_param("variant", 8)
     try:
-        for count, shift in ((5, 0), (1000, 1), (per_phase // 3 + 7, 0), (2 * per_phase + 12345, 3)):
+        for count, shift in ((5, 0), (1000, 1), (per_phase // 3 + 7, 0), (5 * per_phase + 12345, 3)):
             if count * esz * (n + 1) > 6 << 30:
                 count = (6 << 30) // (esz * (n + 1))
             srcs = make_inputs(rng, dtype, count + shift, op, n)
