@@ -2,6 +2,11 @@
 #include "fusion_kernels.hpp"
 
 namespace mi {
+// seven rounding steps per element make this the heaviest traits class; deeper register staging spills
+template <>
+struct PhaseRegs<Bf16PairwiseTraits<true, true>> {
+    static constexpr int fit(int n) { return n <= 4 ? 20 : 12; }
+};
 template hipError_t launch_reduce<Bf16PairwiseTraits<true, true>>(const LaunchArgs&);
 template hipError_t launch_fusion_reduce<Bf16PairwiseTraits<true, true>>(const FusionLaunchArgs&);
 }  // namespace mi

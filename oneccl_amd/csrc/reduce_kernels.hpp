@@ -329,16 +329,18 @@ reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint
 //
 // HBM on this part loses about a quarter of its bandwidth when reads and writes are interleaved (an
 // 8-read + 1-write stream sustains ~5.5 TB/s where reads alone reach ~7.1 TB/s and writes alone ~6 TB/s).
-// This kernel keeps the two apart in time, chip-wide: one 1024-lane block per CU reduces kPhaseU vectors per
-// lane into LDS (read phase: HBM sees only reads), all blocks meet at a barrier, then every block streams
-// its LDS contents out (write phase: HBM sees only writes), and they meet again.
+// This kernel keeps the two apart in time, chip-wide: one 512-lane block per CU reduces up to 44 vectors per
+// lane into LDS and registers (read phase: HBM sees only reads), all blocks meet at a barrier, then every block
+// streams its staged results out (write phase: HBM sees only writes), and they meet again.  Each phase boundary
+// costs a few microseconds of idle HBM, so a phase holds as much as the CU can: 160 KiB of LDS plus up to 24
+// vectors per lane in registers (8 waves per CU leave 256 registers per lane).
 //
 // The barrier carries no data between blocks -- it only aligns them in time -- so a block that waits too
 // long simply goes on (and stops waiting for the rest of the launch): the result is the same whether the
 // barrier holds or not, and no wave can spin forever.
 
-constexpr int kPhaseBlock = 1024;                 // 16 wavefronts, one block per CU
-constexpr int kPhaseU = 10;                       // vectors per lane per phase: 10 x 16 B x 1024 lanes = 160 KiB, all of a CU's LDS
+constexpr int kPhaseBlock = 512;                  // 8 wavefronts, one block per CU
+constexpr int kPhaseU = 20;                       // vectors per lane per phase staged in LDS: 20 x 16 B x 512 lanes = 160 KiB
 constexpr int kPhaseGroups = 16;                  // arrival counters (same-address atomics serialise)
 constexpr long long kPhaseSpinTicks = 20000;      // 100 MHz ticks: 200 us
 
@@ -380,32 +382,61 @@ __device__ __forceinline__ void phase_barrier(PhaseSync* ps, unsigned gen, bool&
     __syncthreads();
 }
 
-// Vectors per lane per phase that are staged in registers on top of the kPhaseU staged in LDS.  Register staging
-// needs fully unrolled code, so it is switched on per traits class (specialise before instantiating).
+// Vectors per lane per phase that are staged in registers on top of the kPhaseU staged in LDS, by number of
+// inputs.  A 512-lane block has 256 registers per lane; the in-flight loads (about eight, 4 registers each),
+// addressing and accumulators leave room for roughly this many staged vectors.  A traits class with lighter or
+// heavier arithmetic specialises this before its kernels are instantiated; the build fails on any scratch use.
 template <class TR>
 struct PhaseRegs {
-    static constexpr int value = 16;
+    static constexpr int fit(int n) { return n <= 4 ? 20 : 22; }
 };
 
-template <class TR, int OP, int N>
-__device__ __forceinline__ u32x4 reduce_one_vector(const u32x4* const (&s)[N], uint64_t i) {
-    u32x4 x[N];
+// G vectors per lane at once: all G x N loads are issued before the first is used, so that a lane keeps about
+// eight 128-bit loads in flight whatever N is.  Callers branch around this (a real branch keeps the compiler
+// from hoisting the loads of later steps, which would spill).
+template <class TR, int OP, int N, int G>
+__device__ __forceinline__ void reduce_group(const u32x4* const (&s)[N], const uint64_t (&idx)[G], u32x4 (&out)[G]) {
+    u32x4 x[G][N];
 #pragma unroll
-    for (int j = 0; j < N; j++) x[j] = ld_stream(s[j] + i);
-    Accs<TR> a = vec_init<TR>(x[0]);
+    for (int g = 0; g < G; g++)
 #pragma unroll
-    for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j], a);
-    return vec_finish<TR>(a);
+        for (int j = 0; j < N; j++) x[g][j] = ld_stream(s[j] + idx[g]);
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        Accs<TR> a = vec_init<TR>(x[g][0]);
+#pragma unroll
+        for (int j = 1; j < N; j++) vec_step<TR, OP>(x[g][j], a);
+        out[g] = vec_finish<TR>(a);
+    }
+}
+
+// the same for a group that may reach past the end of the buffer: slots at or beyond nvec are left alone
+template <class TR, int OP, int N, int G>
+__device__ __forceinline__ void reduce_group_guarded(const u32x4* const (&s)[N], const uint64_t (&idx)[G],
+                                                     uint64_t nvec, u32x4 (&out)[G]) {
+    if (idx[G - 1] < nvec) {
+        reduce_group<TR, OP, N, G>(s, idx, out);
+    }
+    else {
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            if (idx[g] < nvec) {
+                const uint64_t one[1] = { idx[g] };
+                u32x4 o[1];
+                reduce_group<TR, OP, N, 1>(s, one, o);
+                out[g] = o[0];
+            }
+        }
+    }
 }
 
 template <class TR, int OP, int N>
 __global__ void __launch_bounds__(kPhaseBlock)
 reduce_phased_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint32_t tail, PhaseSync* ps) {
     typedef typename TR::elem_t E;
-    // register budget of a 1024-lane block is 128 per lane: N in-flight loads (4 registers each) plus addressing
-    // and accumulators leave room for this many staged vectors
-    constexpr int kFit = (N <= 2) ? 12 : (N <= 4) ? 10 : (N <= 6) ? 8 : 6;
-    constexpr int R = PhaseRegs<TR>::value < kFit ? PhaseRegs<TR>::value : kFit;
+    constexpr int G = (N <= 2) ? 4 : (N <= 4) ? 2 : 1;       // vectors per lane per step
+    constexpr int R = PhaseRegs<TR>::fit(N) / G * G;           // vectors per lane staged in registers
+    static_assert(kPhaseU % G == 0, "LDS steps must be a multiple of the group size");
     __shared__ u32x4 stage[kPhaseU * kPhaseBlock];
     const u32x4* s[N];
 #pragma unroll
@@ -420,13 +451,23 @@ reduce_phased_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, u
     for (uint64_t p0 = 0; p0 < nvec; p0 += per_phase) {
         u32x4 r[R > 0 ? R : 1];
 #pragma unroll
-        for (int u = 0; u < R; u++) {
-            const uint64_t i = p0 + (uint64_t)u * gthreads + gtid;
-            if (i < nvec) r[u] = reduce_one_vector<TR, OP, N>(s, i);
+        for (int u = 0; u < R; u += G) {
+            uint64_t idx[G];
+            u32x4 out[G];
+#pragma unroll
+            for (int g = 0; g < G; g++) idx[g] = p0 + (uint64_t)(u + g) * gthreads + gtid;
+            reduce_group_guarded<TR, OP, N, G>(s, idx, nvec, out);
+#pragma unroll
+            for (int g = 0; g < G; g++) r[u + g] = out[g];
         }
-        for (int u = 0; u < kPhaseU; u++) {
-            const uint64_t i = p0 + (uint64_t)(R + u) * gthreads + gtid;
-            if (i < nvec) stage[u * kPhaseBlock + threadIdx.x] = reduce_one_vector<TR, OP, N>(s, i);
+        for (int u = 0; u < kPhaseU; u += G) {
+            uint64_t idx[G];
+            u32x4 out[G];
+#pragma unroll
+            for (int g = 0; g < G; g++) idx[g] = p0 + (uint64_t)(R + u + g) * gthreads + gtid;
+            reduce_group_guarded<TR, OP, N, G>(s, idx, nvec, out);
+#pragma unroll
+            for (int g = 0; g < G; g++) stage[(u + g) * kPhaseBlock + threadIdx.x] = out[g];
         }
         phase_barrier(ps, ++gen, give_up);      // all reads of this phase are done
 #pragma unroll
@@ -542,7 +583,9 @@ inline hipError_t launch_fixed_unroll(const LaunchArgs& a, uint32_t head, uint64
     constexpr int kDefault = (N <= 4) ? 4 : 2;
     if constexpr (N >= 2) {
         const bool can = a.tune.sync != nullptr && a.tune.num_cus >= kPhaseGroups;
-        const bool big = (long)((uint64_t)(N + 1) * nvec * 16u >> 1) >= (a.tune.phased_min_bytes >> 1);
+        // with two or three inputs the streaming kernel holds up longer (less to interleave per write)
+        const uint64_t traffic = (uint64_t)(N + 1) * nvec * 16u;
+        const bool big = traffic >= (uint64_t)a.tune.phased_min_bytes * (N <= 3 ? 3u : 1u);
         if (can && (a.tune.variant == 8 || (a.tune.variant == 0 && big)))
             return launch_phased<TR, OP, N>(a, head, nvec, tail);
     }

@@ -313,7 +313,7 @@ def test_phased_kernel_parity(comp, dtype, op, n):
     import torch
     rng = np.random.default_rng(300 + dtype)
     esz = O.DTYPE_SIZE[dtype]
-    per_phase = comp.get_param("num_cus") * 1024 * 9 * (16 // esz)      # elements one phase covers
+    per_phase = comp.get_param("num_cus") * 512 * 20 * (16 // esz)      # elements one phase covers
     comp.set_param("variant", 8)
     try:
         for count, shift in ((5, 0), (1000, 1), (per_phase // 3 + 7, 0), (5 * per_phase + 12345, 3)):
