@@ -350,6 +350,20 @@ int mi_ccl_comp_copy(const void* in, void* out, size_t bytes, int use_nontempora
         return MI_CCL_INVALID_ARGUMENTS;
     Tuning t = current_tuning();
     const uintptr_t mis = (uintptr_t)out & 15u;
+    // large copies go through the one-input reduce (a copy for plain types), which separates reads from writes
+    if (((uintptr_t)in & 15u) == mis && t.sync && t.variant == 0 &&
+        2 * (uint64_t)bytes >= 3 * (uint64_t)t.phased_min_bytes) {
+        LaunchArgs a;
+        const void* srcs[1] = { in };
+        a.srcs = srcs;
+        a.n = 1;
+        a.dst = out;
+        a.count = bytes;
+        a.op = OP_SUM;
+        a.stream = (hipStream_t)stream;
+        a.tune = t;
+        return status_of(launch_reduce<U8Traits>(a));
+    }
     if (((uintptr_t)in & 15u) != mis) {
         int grid = grid_for((bytes + kBlock - 1) / kBlock, t);
         hipLaunchKernelGGL(copy_bytes_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream,

@@ -434,7 +434,7 @@ template <class TR, int OP, int N>
 __global__ void __launch_bounds__(kPhaseBlock)
 reduce_phased_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint32_t tail, PhaseSync* ps) {
     typedef typename TR::elem_t E;
-    constexpr int G = (N <= 2) ? 4 : (N <= 4) ? 2 : 1;       // vectors per lane per step
+    constexpr int G = (N == 1) ? 10 : (N == 2) ? 4 : (N <= 4) ? 2 : 1;       // vectors per lane per step
     constexpr int R = PhaseRegs<TR>::fit(N) / G * G;           // vectors per lane staged in registers
     static_assert(kPhaseU % G == 0, "LDS steps must be a multiple of the group size");
     __shared__ u32x4 stage[kPhaseU * kPhaseBlock];
@@ -581,7 +581,7 @@ template <class TR, int OP, int N>
 inline hipError_t launch_fixed_unroll(const LaunchArgs& a, uint32_t head, uint64_t nvec, uint32_t tail) {
     // loads in flight per lane = N * UNROLL
     constexpr int kDefault = (N <= 4) ? 4 : 2;
-    if constexpr (N >= 2) {
+    {
         const bool can = a.tune.sync != nullptr && a.tune.num_cus >= kPhaseGroups;
         // with two or three inputs the streaming kernel holds up longer (less to interleave per write)
         const uint64_t traffic = (uint64_t)(N + 1) * nvec * 16u;

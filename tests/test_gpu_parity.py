@@ -225,6 +225,15 @@ def test_copy_and_converters(comp):
                 got = to_host(dd, np.uint8)
                 assert (got[sb:sb + nbytes] == src[sa:sa + nbytes]).all()
                 assert (got[:sb] == 0).all() and (got[sb + nbytes:] == 0).all()
+    # a copy large enough for the phased one-input kernel, with head and tail bytes
+    nbytes = (800 << 20) + 5
+    src_d = torch.randint(-128, 127, (nbytes + 32,), dtype=torch.int8, device="cuda")
+    dst_d = torch.zeros(nbytes + 32, dtype=torch.int8, device="cuda")
+    comp.comp_copy(src_d.data_ptr() + 3, dst_d.data_ptr() + 19, nbytes, use_nontemporal=True)
+    torch.cuda.synchronize()
+    assert torch.equal(dst_d[19:19 + nbytes], src_d[3:3 + nbytes])
+    assert int(dst_d[:19].count_nonzero()) == 0 and int(dst_d[19 + nbytes:].count_nonzero()) == 0
+    del src_d, dst_d
     L = O.lib()
     for count in (1, 5, 16, 22, 1000, 65536 + 7):
         f32 = rng.integers(0, 2**32, count, dtype=np.uint32)
