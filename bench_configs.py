@@ -121,12 +121,23 @@ def main():
         f"{us_three / us_fused:.2f}x faster than the 3-step sequence")
     plan.close()
 
+    # small-message latency from C++ (no Python in the loop)
+    lat = os.path.join(ROOT, "tests", "cpp", "bench_latency")
+    lat_lines = []
+    if os.path.exists(lat):
+        import subprocess
+        lat_lines = subprocess.run([lat], capture_output=True, text=True, timeout=120).stdout.strip().splitlines()
+        res["latency_cpp"] = lat_lines
+
     os.makedirs(os.path.dirname(args.out), exist_ok=True)
     with open(args.out, "w") as f:
         json.dump(res, f, indent=1)
     print("| configuration | algorithmic bytes | us per call | GB/s | of 8 TB/s | note |")
     print("|---|---|---|---|---|---|")
     print("\n".join(rows))
+    if lat_lines:
+        print("\nSmall messages issued from C++ (tests/cpp/bench_latency, 4-input int32 sum):\n")
+        print("\n".join("    " + l for l in lat_lines))
 
 
 if __name__ == "__main__":
