@@ -163,6 +163,134 @@ fusion_reduce_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers
     }
 }
 
+// The same reduce with reads and writes separated in time (see reduce_phased_kernel): each block takes kPhaseU / 2
+// work items per phase (an item is 16 KiB of one tensor = two vectors per lane), keeps their results in LDS, and
+// writes them after the chip-wide barrier.  Item (phase, slot, block) = phase * slots * blocks + slot * blocks + block.
+// Head/tail elements of tensors that do not start on a 16-byte boundary, and tensors whose streams disagree modulo
+// 16 bytes, are written directly (they are a few bytes, or a rare layout).  NT = 1 + number of peers.
+template <class TR, int OP, int NT>
+__global__ void __launch_bounds__(kPhaseBlock)
+fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, const uint64_t* off, const uint64_t* bytes,
+                            const FusionItem* items, uint32_t nitems, uint32_t t0, PhaseSync* ps) {
+    typedef typename TR::elem_t E;
+    constexpr uint32_t ES = sizeof(E);
+    constexpr int S = kPhaseU / 2;
+    constexpr int NP = NT - 1;
+    static_assert(kFusionChunk == 2 * 16 * kPhaseBlock, "an item is two vectors per lane");
+    static_assert(S <= 64, "one descriptor per lane of a wave");
+    __shared__ u32x4 stage[kPhaseU * kPhaseBlock];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    bool give_up = false;
+    unsigned gen = 0;
+    if (tid == 0) gen = MI_ALOAD(&ps->rel.v);
+    const uint64_t per_phase = (uint64_t)S * gridDim.x;
+    for (uint64_t p0 = 0; p0 < nitems; p0 += per_phase) {
+        // Lane k of every wave fetches the descriptor of this block's k-th item of the phase, so that the chain
+        // item -> tensor tables -> pointers is walked once, for all items at once, instead of once per item.
+        uint64_t d_a = 0, d_o = 0, d_poff = 0;
+        uint32_t d_nb = 0;      // 0: no item in this slot
+        if (lane < (uint32_t)S) {
+            const uint64_t it = p0 + (uint64_t)lane * gridDim.x + blockIdx.x;
+            if (it < nitems) {
+                const FusionItem w = items[it];
+                const uint64_t lo = (uint64_t)w.c * kFusionChunk;
+                const uint64_t left = bytes[w.t] - lo;
+                d_nb = left < kFusionChunk ? (uint32_t)left : kFusionChunk;
+                d_a = (uint64_t)(uintptr_t)own.p[w.t - t0] + lo;
+                d_o = (uint64_t)(uintptr_t)out.p[w.t - t0] + lo;
+                d_poff = off[w.t] + lo;
+            }
+        }
+        for (int k = 0; k < S; k++) {
+            const uint32_t nb = __shfl(d_nb, k, 64);
+            if (nb == 0) break;
+            const unsigned char* a = (const unsigned char*)(uintptr_t)__shfl(d_a, k, 64);
+            unsigned char* o = (unsigned char*)(uintptr_t)__shfl(d_o, k, 64);
+            const uint64_t poff = __shfl(d_poff, k, 64);
+            const uint32_t mis = (uint32_t)(uintptr_t)a & 15u;
+            bool same = (((uint32_t)(uintptr_t)o & 15u) == mis);
+#pragma unroll
+            for (int j = 0; j < NP; j++)
+                same = same && ((((uint32_t)(uintptr_t)peers.p[j] + (uint32_t)poff) & 15u) == mis);
+            const uint32_t nelem = nb / ES;
+            if (same) {
+                uint32_t head = mis ? (16u - mis) / ES : 0;
+                if (head > nelem) head = nelem;
+                const uint32_t nvec = (nelem - head) / TR::VEC, tail = nelem - head - nvec * TR::VEC;
+                const u32x4* s[NT];
+                s[0] = (const u32x4*)(a + head * ES);
+#pragma unroll
+                for (int j = 0; j < NP; j++) s[j + 1] = (const u32x4*)((const unsigned char*)peers.p[j] + poff + head * ES);
+                const uint64_t idx[2] = { tid, tid + (uint32_t)kPhaseBlock };
+                u32x4 res[2];
+                if constexpr (TR::VEC * NT <= 64) {
+                    reduce_group_guarded<TR, OP, NT, 2>(s, idx, nvec, res);
+                }
+                else {      // 16 one-byte elements x 7-8 inputs: both vectors at once would not fit the registers
+                    const uint64_t i0[1] = { idx[0] }, i1[1] = { idx[1] };
+                    u32x4 r0[1], r1[1];
+                    reduce_group_guarded<TR, OP, NT, 1>(s, i0, nvec, r0);
+                    reduce_group_guarded<TR, OP, NT, 1>(s, i1, nvec, r1);
+                    res[0] = r0[0];
+                    res[1] = r1[0];
+                }
+                stage[(2 * k) * kPhaseBlock + tid] = res[0];
+                stage[(2 * k + 1) * kPhaseBlock + tid] = res[1];
+                if (tid < head + tail) {
+                    const uint32_t i = (tid < head) ? tid : head + nvec * TR::VEC + (tid - head);
+                    typename TR::acc_t r = TR::init(((const E*)a)[i]);
+#pragma unroll
+                    for (int j = 0; j < NP; j++)
+                        r = TR::template step<OP>(((const E*)((const unsigned char*)peers.p[j] + poff))[i], r);
+                    ((E*)o)[i] = TR::finish(r);
+                }
+            }
+            else {
+                for (uint32_t i = tid; i < nelem; i += kPhaseBlock) {
+                    typename TR::acc_t r = TR::init(((const E*)a)[i]);
+#pragma unroll
+                    for (int j = 0; j < NP; j++)
+                        r = TR::template step<OP>(((const E*)((const unsigned char*)peers.p[j] + poff))[i], r);
+                    ((E*)o)[i] = TR::finish(r);
+                }
+            }
+        }
+        phase_barrier(ps, ++gen, give_up);
+        for (int k = 0; k < S; k++) {
+            const uint32_t nb = __shfl(d_nb, k, 64);
+            if (nb == 0) break;
+            const unsigned char* a = (const unsigned char*)(uintptr_t)__shfl(d_a, k, 64);
+            unsigned char* o = (unsigned char*)(uintptr_t)__shfl(d_o, k, 64);
+            const uint64_t poff = __shfl(d_poff, k, 64);
+            const uint32_t mis = (uint32_t)(uintptr_t)a & 15u;
+            bool same = (((uint32_t)(uintptr_t)o & 15u) == mis);
+#pragma unroll
+            for (int j = 0; j < NP; j++)
+                same = same && ((((uint32_t)(uintptr_t)peers.p[j] + (uint32_t)poff) & 15u) == mis);
+            if (same) {
+                const uint32_t nelem = nb / ES;
+                uint32_t head = mis ? (16u - mis) / ES : 0;
+                if (head > nelem) head = nelem;
+                const uint32_t nvec = (nelem - head) / TR::VEC;
+                u32x4* d = (u32x4*)(o + head * ES);
+                if (tid < nvec) st_stream(d + tid, stage[(2 * k) * kPhaseBlock + tid]);
+                if (tid + kPhaseBlock < nvec) st_stream(d + tid + kPhaseBlock, stage[(2 * k + 1) * kPhaseBlock + tid]);
+            }
+        }
+        phase_barrier(ps, ++gen, give_up);
+    }
+}
+
+template <class TR, int OP, int NT>
+inline hipError_t launch_fusion_phased(const FusionLaunchArgs& a, const FusionPtrs& own, const FusionPtrs& out,
+                                       const PeerPtrs& pp, uint64_t i0, uint64_t i1, size_t t0) {
+    int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
+    hipLaunchKernelGGL((fusion_reduce_phased_kernel<TR, OP, NT>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, own, out, pp,
+                       a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0, a.tune.sync);
+    return hipGetLastError();
+}
+
 template <class TR, int OP>
 inline hipError_t launch_fusion_op(const FusionLaunchArgs& a) {
     PeerPtrs pp;
@@ -177,10 +305,28 @@ inline hipError_t launch_fusion_op(const FusionLaunchArgs& a) {
             own.p[t - t0] = a.own[t];
             out.p[t - t0] = a.out[t];
         }
-        int grid = grid_for(i1 - i0, a.tune);
-        hipLaunchKernelGGL((fusion_reduce_kernel<TR, OP>), dim3(grid), dim3(kBlock), 0, a.stream, own, out, pp,
-                           a.n_peers, a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0);
-        hipError_t e = hipGetLastError();
+        hipError_t e = hipSuccess;
+        // large groups: separate reads from writes in time (at most 16 KiB of padding per item is over-counted)
+        const uint64_t traffic = (uint64_t)(a.n_peers + 2) * (i1 - i0) * kFusionChunk;
+        const bool phased = a.tune.sync && a.tune.num_cus >= kPhaseGroups && a.n_peers >= 1 && a.n_peers <= 7 &&
+                            (a.tune.variant == 8 || (a.tune.variant == 0 && traffic >= (uint64_t)a.tune.phased_min_bytes));
+        if (phased) {
+            switch (a.n_peers) {
+                case 1: e = launch_fusion_phased<TR, OP, 2>(a, own, out, pp, i0, i1, t0); break;
+                case 2: e = launch_fusion_phased<TR, OP, 3>(a, own, out, pp, i0, i1, t0); break;
+                case 3: e = launch_fusion_phased<TR, OP, 4>(a, own, out, pp, i0, i1, t0); break;
+                case 4: e = launch_fusion_phased<TR, OP, 5>(a, own, out, pp, i0, i1, t0); break;
+                case 5: e = launch_fusion_phased<TR, OP, 6>(a, own, out, pp, i0, i1, t0); break;
+                case 6: e = launch_fusion_phased<TR, OP, 7>(a, own, out, pp, i0, i1, t0); break;
+                default: e = launch_fusion_phased<TR, OP, 8>(a, own, out, pp, i0, i1, t0); break;
+            }
+        }
+        else {
+            int grid = grid_for(i1 - i0, a.tune);
+            hipLaunchKernelGGL((fusion_reduce_kernel<TR, OP>), dim3(grid), dim3(kBlock), 0, a.stream, own, out, pp,
+                               a.n_peers, a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0);
+            e = hipGetLastError();
+        }
         if (e != hipSuccess)
             return e;
     }

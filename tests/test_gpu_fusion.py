@@ -82,16 +82,25 @@ def test_pack_reduce_unpack_and_fused(comp, align, dtype):
         assert_same(g[:c], want[i], dtype, f"3-step tensor {i}")
         assert (g[c:] == 0).all(), "unpack wrote past the tensor"
 
-    # GPU, fused single pass, out of place and in place
-    outs2 = [to_dev(np.zeros(c + 4, np_t)) for c in counts]
-    plan.reduce(O.SUM, d_t, d_peers, outs2, lp_mode=lp)
-    torch.cuda.synchronize()
-    for i, c in enumerate(counts):
-        g = to_host(outs2[i], np_t)
-        assert_same(g[:c], want[i], dtype, f"fused tensor {i}")
-        assert (g[c:] == 0).all()
-    plan.reduce(O.SUM, d_t, d_peers, d_t, lp_mode=lp)
-    torch.cuda.synchronize()
+    # GPU, fused single pass, out of place (streaming kernel, then the phased one forced on) and in place
+    for variant in (2, 8):
+        comp.set_param("variant", variant)
+        try:
+            outs2 = [to_dev(np.zeros(c + 4, np_t)) for c in counts]
+            plan.reduce(O.SUM, d_t, d_peers, outs2, lp_mode=lp)
+            torch.cuda.synchronize()
+        finally:
+            comp.set_param("variant", 0)
+        for i, c in enumerate(counts):
+            g = to_host(outs2[i], np_t)
+            assert_same(g[:c], want[i], dtype, f"fused tensor {i} variant {variant}")
+            assert (g[c:] == 0).all()
+    comp.set_param("variant", 8)
+    try:
+        plan.reduce(O.SUM, d_t, d_peers, d_t, lp_mode=lp)
+        torch.cuda.synchronize()
+    finally:
+        comp.set_param("variant", 0)
     for i, c in enumerate(counts):
         sh = (i % 3) if align == 1 else 0
         g = to_host(holders[i], np_t)
@@ -116,11 +125,16 @@ def test_fusion_config_bf16_256_tensors(comp):
     want = O.fusion_unpack(fused.view(np.uint8), counts, offs, np.uint16)
     d_t = [to_dev(t) for t in tensors]
     d_peers = [to_dev(p) for p in peers]
-    outs = [torch.empty_like(t) for t in d_t]
-    plan.reduce(O.SUM, d_t, d_peers, outs, lp_mode=comp.LP_KEEP_PRECISION)
-    torch.cuda.synchronize()
-    for i in range(256):
-        assert (to_host(outs[i], np.uint16) == want[i]).all(), i
+    for variant in (0, 8):
+        comp.set_param("variant", variant)
+        try:
+            outs = [torch.zeros_like(t) for t in d_t]
+            plan.reduce(O.SUM, d_t, d_peers, outs, lp_mode=comp.LP_KEEP_PRECISION)
+            torch.cuda.synchronize()
+        finally:
+            comp.set_param("variant", 0)
+        for i in range(256):
+            assert (to_host(outs[i], np.uint16) == want[i]).all(), (i, variant)
     # per-tensor invariant: fused result == unfused 8-input reduce of the tensor with the peer slices
     i = 17
     lo = int(offs[i]) // 2
