@@ -236,9 +236,11 @@ f32_to_bf16_kernel(const uint32_t* in, uint16_t* out, uint64_t count, uint64_t r
     for (uint64_t q = (uint64_t)blockIdx.x * kBlock + threadIdx.x; q < nquad; q += stride) {
         u32x4 x = __builtin_nontemporal_load((const u32x4*)in + q);
         uint32_t r[4];
+        // the packed conversion the reduce kernels use (the element form serves the tail below)
+        const uint32_t p01 = RNE ? bf16_narrow_rne_pack2(x[0], x[1]) : 0u, p23 = RNE ? bf16_narrow_rne_pack2(x[2], x[3]) : 0u;
+        const uint32_t rne[4] = { p01 & 0xffffu, p01 >> 16, p23 & 0xffffu, p23 >> 16 };
 #pragma unroll
-        for (int k = 0; k < 4; k++)
-            r[k] = (RNE && q * 4 + k < rne_limit) ? bf16_narrow_rne(x[k]) : bf16_narrow_trunc(x[k]);
+        for (int k = 0; k < 4; k++) r[k] = (RNE && q * 4 + k < rne_limit) ? rne[k] : bf16_narrow_trunc(x[k]);
         uint2 o = make_uint2(r[0] | (r[1] << 16), r[2] | (r[3] << 16));
         ((uint2*)out)[q] = o;
     }

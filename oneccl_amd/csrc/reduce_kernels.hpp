@@ -69,6 +69,21 @@ __device__ __forceinline__ uint32_t bf16_narrow_rne(uint32_t u) {
 // fp32 -> bf16 by dropping the low half (src/comp/bf16/bf16.cpp:50-54, bf16_intrisics.hpp:67-70)
 __device__ __forceinline__ uint32_t bf16_narrow_trunc(uint32_t u) { return u >> 16; }
 
+// Two fp32 values -> two bf16 values packed in one dword (lo in the low half), same results as bf16_narrow_rne.
+// gfx950's v_cvt_pk_bf16_f32 rounds to nearest even, quiets NaNs and overflows to Inf exactly like VCVTNEPS2BF16
+// (all 2^32 inputs compared on the GPU); the one difference is that it keeps fp32 denormals, which the x86
+// instruction reads as zero, so those are replaced by a signed zero first (one v_cmp_class per value).
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t bf16_narrow_rne_pack2(uint32_t lo, uint32_t hi) {
+    constexpr int kDenormal = 0x10 | 0x80;      // class mask: negative denormal, positive denormal
+    float a = as_f32(lo), b = as_f32(hi);
+    a = __builtin_amdgcn_classf(a, kDenormal) ? as_f32(lo & 0x80000000u) : a;
+    b = __builtin_amdgcn_classf(b, kDenormal) ? as_f32(hi & 0x80000000u) : b;
+    const f32x2 f = { a, b };
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+}
+
 // compare on the float value, select on the bits: the returned operand's bits are never touched
 template <int OP, bool VEC_SEM>
 __device__ __forceinline__ uint32_t f32_minmax_bits(uint32_t in, uint32_t io) {
@@ -217,26 +232,97 @@ struct Accs {
     typename TR::acc_t v[TR::VEC];
 };
 
+// Vector-level operations on the 128-bit unit a lane moves.  The default walks the VEC elements one by one with
+// the traits' init / step / finish; traits with a cheaper packed form specialise VecOps.
+template <class TR>
+struct VecOps {
+    static __device__ __forceinline__ Accs<TR> init(u32x4 x) {
+        Lanes<TR> l = __builtin_bit_cast(Lanes<TR>, x);
+        Accs<TR> a;
+#pragma unroll
+        for (int k = 0; k < TR::VEC; k++) a.v[k] = TR::init(l.v[k]);
+        return a;
+    }
+    template <int OP>
+    static __device__ __forceinline__ void step(u32x4 x, Accs<TR>& a) {
+        Lanes<TR> l = __builtin_bit_cast(Lanes<TR>, x);
+#pragma unroll
+        for (int k = 0; k < TR::VEC; k++) a.v[k] = TR::template step<OP>(l.v[k], a.v[k]);
+    }
+    static __device__ __forceinline__ u32x4 finish(const Accs<TR>& a) {
+        Lanes<TR> l;
+#pragma unroll
+        for (int k = 0; k < TR::VEC; k++) l.v[k] = TR::finish(a.v[k]);
+        return __builtin_bit_cast(u32x4, l);
+    }
+};
+
+// bf16 rounded to nearest even after every pair: the accumulator stays in storage format (two bf16 per dword, in
+// a.v[0..3]); both halves of a dword are widened, combined and narrowed together by the packed conversion.
+template <bool VEC_SEM>
+struct VecOps<Bf16PairwiseTraits<true, VEC_SEM>> {
+    typedef Bf16PairwiseTraits<true, VEC_SEM> TR;
+    static __device__ __forceinline__ Accs<TR> init(u32x4 x) {
+        Accs<TR> a;
+#pragma unroll
+        for (int k = 0; k < 4; k++) a.v[k] = x[k];
+        return a;
+    }
+    template <int OP>
+    static __device__ __forceinline__ void step(u32x4 x, Accs<TR>& a) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t in = x[k], io = a.v[k];
+            const uint32_t lo = f32_step_bits<OP, VEC_SEM>(in << 16, io << 16);
+            const uint32_t hi = f32_step_bits<OP, VEC_SEM>(in & 0xffff0000u, io & 0xffff0000u);
+            a.v[k] = bf16_narrow_rne_pack2(lo, hi);
+        }
+    }
+    static __device__ __forceinline__ u32x4 finish(const Accs<TR>& a) {
+        return u32x4{ a.v[0], a.v[1], a.v[2], a.v[3] };
+    }
+};
+
+// bf16 accumulated in fp32 and rounded to nearest even once: element-wise init and step, packed narrowing.
+template <>
+struct VecOps<Bf16KeepTraits<true>> {
+    typedef Bf16KeepTraits<true> TR;
+    static __device__ __forceinline__ Accs<TR> init(u32x4 x) {
+        Accs<TR> a;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            a.v[2 * k] = x[k] << 16;
+            a.v[2 * k + 1] = x[k] & 0xffff0000u;
+        }
+        return a;
+    }
+    template <int OP>
+    static __device__ __forceinline__ void step(u32x4 x, Accs<TR>& a) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            a.v[2 * k] = f32_step_bits<OP, false>(x[k] << 16, a.v[2 * k]);
+            a.v[2 * k + 1] = f32_step_bits<OP, false>(x[k] & 0xffff0000u, a.v[2 * k + 1]);
+        }
+    }
+    static __device__ __forceinline__ u32x4 finish(const Accs<TR>& a) {
+        u32x4 r;
+#pragma unroll
+        for (int k = 0; k < 4; k++) r[k] = bf16_narrow_rne_pack2(a.v[2 * k], a.v[2 * k + 1]);
+        return r;
+    }
+};
+
 template <class TR>
 __device__ __forceinline__ Accs<TR> vec_init(u32x4 x) {
-    Lanes<TR> l = __builtin_bit_cast(Lanes<TR>, x);
-    Accs<TR> a;
-#pragma unroll
-    for (int k = 0; k < TR::VEC; k++) a.v[k] = TR::init(l.v[k]);
-    return a;
+    return VecOps<TR>::init(x);
 }
 template <class TR, int OP>
 __device__ __forceinline__ void vec_step(u32x4 x, Accs<TR>& a) {
-    Lanes<TR> l = __builtin_bit_cast(Lanes<TR>, x);
-#pragma unroll
-    for (int k = 0; k < TR::VEC; k++) a.v[k] = TR::template step<OP>(l.v[k], a.v[k]);
+    VecOps<TR>::template step<OP>(x, a);
 }
 template <class TR>
 __device__ __forceinline__ u32x4 vec_finish(const Accs<TR>& a) {
-    Lanes<TR> l;
-#pragma unroll
-    for (int k = 0; k < TR::VEC; k++) l.v[k] = TR::finish(a.v[k]);
-    return __builtin_bit_cast(u32x4, l);
+    return VecOps<TR>::finish(a);
 }
 
 __device__ __forceinline__ u32x4 ld_stream(const u32x4* p) { return __builtin_nontemporal_load(p); }

@@ -256,21 +256,23 @@ def test_copy_and_converters(comp):
 
 def test_bf16_narrowing_exhaustive_on_gpu(comp):
     """All 2^32 fp32 patterns through the GPU's round-to-nearest-even narrowing vs the oracle (itself
-    exhaustively equal to VCVTNEPS2BF16)."""
+    exhaustively equal to VCVTNEPS2BF16).  The kernel converts pairs with the packed hardware conversion, so every
+    pattern is sent twice: once at an even index (low half of the pair) and once at an odd one (high half)."""
     import torch
     L = O.lib()
-    chunk = 1 << 26
+    chunk = 1 << 27
     d_out = torch.empty(chunk, dtype=torch.int16, device="cuda")
     want = np.empty(chunk, np.uint16)
-    for c in range(0, 1 << 32, chunk):
-        x = torch.arange(c, c + chunk, dtype=torch.int64, device="cuda")
-        src = torch.where(x >= 2**31, x - 2**32, x).to(torch.int32)      # the fp32 bit pattern as int32
-        comp.convert_fp32_to_bf16_arrays(src, d_out, chunk, bf16_impl=2)
-        torch.cuda.synchronize()
-        host = np.arange(c, c + chunk, dtype=np.uint64).astype(np.uint32)
-        L.orc_convert_fp32_to_bf16_arrays(host.ctypes.data, want.ctypes.data, chunk, 2)
-        got = to_host(d_out, np.uint16)
-        assert (got == want).all(), hex(c + int(np.flatnonzero(got != want)[0]))
+    for shift in (0, 1):
+        for c in range(0, 1 << 32, chunk):
+            x = (torch.arange(c, c + chunk, dtype=torch.int64, device="cuda") + shift) & 0xFFFFFFFF
+            src = torch.where(x >= 2**31, x - 2**32, x).to(torch.int32)      # the fp32 bit pattern as int32
+            comp.convert_fp32_to_bf16_arrays(src, d_out, chunk, bf16_impl=2)
+            torch.cuda.synchronize()
+            host = ((np.arange(c, c + chunk, dtype=np.uint64) + shift) & 0xFFFFFFFF).astype(np.uint32)
+            L.orc_convert_fp32_to_bf16_arrays(host.ctypes.data, want.ctypes.data, chunk, 2)
+            got = to_host(d_out, np.uint16)
+            assert (got == want).all(), (shift, hex(c + int(np.flatnonzero(got != want)[0])))
 
 
 @pytest.mark.parametrize("dtype,impl", [(O.FLOAT16, 3), (O.BFLOAT16, 2)])
