@@ -40,7 +40,7 @@ WORKLOADS = {
 }
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two runs), each scaled by what the
-# same counter reads for a plain copy of known size (x2.0000 and x1.0000): profiles/reduce_phased_bf16_sum_8x2GiB.md.
+# same counter reads for a plain copy of known size (x2.0000 and x1.0000); the summary is kept under profiles/.
 MEASURED_TRAFFIC_BYTES = {"c5_bf16": (15_684_982 + 1_963_266) * 1024}
 
 

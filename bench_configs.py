@@ -7,7 +7,7 @@
   C4  fusion: 256 bf16 tensors, counts log-uniform [2,048, 2,097,152], 256-byte aligned offsets, 8-input sum against
       7 peer fusion buffers: pack + reduce + unpack, and the fused single pass
 
-    python bench_configs.py [--out gpurun_out/configs.json] [--skip c3]
+    python bench_configs.py [--out results/configs.json] [--skip c3]
 
 Writes a JSON file and prints a markdown table.  Bytes are algorithmic: (N + 1) x chunk for a reduce, 2 x payload
 for pack and unpack.  Buffers of 64 MiB rotate over several sets so that the 256 MB Infinity Cache cannot hold them.
@@ -37,7 +37,7 @@ def timed(torch, fn, steps, warm):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--out", default=os.path.join(ROOT, "gpurun_out", "configs.json"))
+    ap.add_argument("--out", default=os.path.join(ROOT, "results", "configs.json"))
     ap.add_argument("--skip", default="")
     args = ap.parse_args()
     import numpy as np
