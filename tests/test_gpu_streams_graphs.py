@@ -1,0 +1,78 @@
+"""Launch-context tests: the reduce captured in a HIP graph and replayed, and two large (phased) reduces
+overlapping on two streams.  The phased kernel's grid barrier only aligns blocks in time, so neither replay nor
+overlap may change a single bit."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from gpu_util import to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def comp():
+    import torch
+    assert torch.cuda.is_available()
+    import oneccl_amd.comp as c
+    c.lib()
+    return c
+
+
+@pytest.mark.parametrize("variant", [2, 8])
+def test_graph_capture_and_replay(comp, variant):
+    import torch
+    rng = np.random.default_rng(variant)
+    count, n = 3_000_017, 8
+    srcs = [O.bf16_from_f32(rng.standard_normal(count).astype(np.float32)) for _ in range(n)]
+    want = O.reduce_n(srcs, O.BFLOAT16, O.SUM, keep=1, threads=8)
+    d = [to_dev(s) for s in srcs]
+    out = torch.zeros_like(d[0])
+    comp.set_param("variant", variant)
+    try:
+        comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, d, out, count, lp_mode=comp.LP_KEEP_PRECISION)   # warm up, eager
+        torch.cuda.synchronize()
+        assert (to_host(out, np.uint16) == want).all()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, d, out, count, lp_mode=comp.LP_KEEP_PRECISION)
+        for rep in range(4):
+            out.fill_(0)                     # eager work between the replays
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            assert (to_host(out, np.uint16) == want).all(), f"replay {rep}"
+            # an eager launch between replays shares the barrier words with the captured one
+            comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, d, out, count, lp_mode=comp.LP_KEEP_PRECISION)
+            torch.cuda.synchronize()
+            assert (to_host(out, np.uint16) == want).all()
+    finally:
+        comp.set_param("variant", 0)
+
+
+def test_two_phased_reduces_overlapping_on_two_streams(comp):
+    import torch
+    rng = np.random.default_rng(11)
+    count, n = 40_000_003, 4              # 4 x 160 MB fp32 per reduce: several phases each
+    a = [rng.standard_normal(count).astype(np.float32) for _ in range(n)]
+    b = [rng.standard_normal(count).astype(np.float32) for _ in range(n)]
+    want_a = O.reduce_n(a, O.FLOAT32, O.SUM, threads=16)
+    want_b = O.reduce_n(b, O.FLOAT32, O.MAX, threads=16)
+    da, db = [to_dev(x) for x in a], [to_dev(x) for x in b]
+    oa, ob = torch.zeros_like(da[0]), torch.zeros_like(db[0])
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    comp.set_param("variant", 8)
+    try:
+        for _ in range(3):
+            comp.comp_reduce_n(comp.FLOAT32, comp.SUM, da, oa, count, stream=s1)
+            comp.comp_reduce_n(comp.FLOAT32, comp.MAX, db, ob, count, stream=s2)
+        torch.cuda.synchronize()
+    finally:
+        comp.set_param("variant", 0)
+    assert (to_host(oa, np.float32).view(np.uint32) == want_a.view(np.uint32)).all()
+    assert (to_host(ob, np.float32).view(np.uint32) == want_b.view(np.uint32)).all()
+    # and the barrier words are left consistent: a following launch runs at full speed and is exact
+    comp.comp_reduce_n(comp.FLOAT32, comp.SUM, da, oa, count)
+    torch.cuda.synchronize()
+    assert (to_host(oa, np.float32).view(np.uint32) == want_a.view(np.uint32)).all()
