@@ -184,7 +184,7 @@ def main():
     value = algo_bytes / (ms_per_step * 1e-3) / 1e9
     achieved = algo_bytes / (kernel_ms * 1e-3) / 1e9
     out = {
-        "metric": "N-way reduce GB/s (bf16 sum, 8 inputs x 2 GiB)" if args.workload == "c5_bf16"
+        "metric": "N-way reduce GB/s and % of HBM peak (bf16 sum, 8 inputs x 2 GiB)" if args.workload == "c5_bf16"
                   else f"N-way reduce GB/s ({args.workload})",
         "value": round(value, 1),
         "unit": "GB/s",

@@ -343,3 +343,51 @@ def test_phased_kernel_parity(comp, dtype, op, n):
             assert (got[:shift] == 0).all()
     finally:
         comp.set_param("variant", 0)
+
+
+def test_randomised_calls_against_oracle(comp):
+    """400 seeded random calls: dtype, op, input count (1..12), element count, 16-bit mode, per-buffer element
+    shifts (shared or mixed misalignment), output aliasing an input or not, kernel choice forced or automatic."""
+    import torch
+    rng = np.random.default_rng(20260101)
+    for case in range(400):
+        dtype = int(rng.integers(0, 12))
+        op = int(rng.integers(0, 4))
+        n = int(rng.integers(1, 13))
+        count = int(rng.choice([1, 2, 3, 15, 16, 17, 255, 1000, 4097, 65535, 200_003]))
+        esz = O.DTYPE_SIZE[dtype]
+        np_t = O.NP_STORAGE[dtype]
+        lp, impl, keep, quirk = lp_variants(dtype)[int(rng.integers(0, len(lp_variants(dtype))))]
+        kind = "bits" if dtype in (O.FLOAT16, O.BFLOAT16) and rng.random() < 0.5 else "config"
+        srcs = make_inputs(rng, dtype, count, op, n, kind)
+        same_shift = rng.random() < 0.6
+        base_shift = int(rng.integers(0, 16 // esz + 1))
+        shifts = [base_shift if same_shift else int(rng.integers(0, 16 // esz + 1)) for _ in range(n + 1)]
+        pad = 32
+        holders, ptrs = [], []
+        for s_, sh in zip(srcs, shifts):
+            h = np.zeros(count + 2 * pad, np_t)
+            h[pad + sh:pad + sh + count] = s_
+            holders.append(to_dev(h))
+            ptrs.append(holders[-1].data_ptr() + (pad + sh) * esz)
+        alias = int(rng.integers(-1, n))            # -1: separate output
+        if alias >= 0:
+            out_holder, out_lo = holders[alias], pad + shifts[alias]
+        else:
+            out_holder, out_lo = to_dev(np.zeros(count + 2 * pad, np_t)), pad + shifts[n]
+        variant = int(rng.choice([0, 0, 2, 8]))
+        comp.set_param("variant", variant)
+        try:
+            comp.comp_reduce_n(dtype, op, ptrs, out_holder.data_ptr() + out_lo * esz, count, lp_mode=lp, bf16_impl=impl)
+            torch.cuda.synchronize()
+        finally:
+            comp.set_param("variant", 0)
+        want = O.reduce_n(srcs, dtype, op, keep=keep, quirk_tail=quirk, bf16_impl=impl)
+        got = to_host(out_holder, np_t)
+        what = (f"case {case}: dtype={O.DTYPE_NAMES[dtype]} op={O.OP_NAMES[op]} n={n} count={count} lp={lp} impl={impl} "
+                f"shifts={shifts} alias={alias} variant={variant} kind={kind}")
+        assert_same(got[out_lo:out_lo + count], want, dtype, what)
+        if alias < 0:
+            assert (got[:out_lo] == 0).all() and (got[out_lo + count:] == 0).all(), what + ": wrote outside the destination"
+        else:
+            assert (got[:out_lo] == 0).all() and (got[out_lo + count:] == 0).all(), what + ": wrote outside the aliased input"
