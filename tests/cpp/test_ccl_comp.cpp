@@ -9,10 +9,12 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <memory>
 #include <string>
 #include <vector>
 
 #include "../../oneccl_amd/csrc/ccl_comp.hpp"
+#include "../../oneccl_amd/csrc/ccl_fusion.hpp"
 #include "../../oracle/ccl_comp_oracle.h"
 
 #define CK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { printf("HIP error %s at line %d\n", hipGetErrorString(e_), __LINE__); exit(2); } } while (0)
@@ -216,6 +218,80 @@ int main() {
         bool ok = true;
         for (int i = 0; i < 22; i++) ok = ok && w[i] == ((uint32_t)h[i] << 16);
         EXPECT(ok, "bf16->fp32 arrays");
+    }
+    // fusion manager over the HIP backend: 700 small bf16 gradient tensors arrive as individual requests, are fused
+    // (tight layout, at most 256 per launch), reduced against 7 peer fusion buffers by ONE 8-input reduce per launch,
+    // and unpacked.  Peer j holds the constant c_j everywhere, so the expected tensor does not depend on where the
+    // manager placed it in the buffer, while a misplaced or mis-sized copy would show.
+    {
+        ccl_fusion_hip_backend backend;
+        ccl_fusion_config cfg;
+        cfg.cycle_ms = 0;
+        const int NPEER = 7;
+        std::vector<DevBuf<uint16_t>*> peer_bufs;
+        std::vector<uint16_t> peer_val(NPEER);
+        size_t buf_elems = cfg.bytes_threshold * cfg.count_threshold / 2;
+        for (int j = 0; j < NPEER; j++) {
+            peer_val[j] = to_lp(0.25f * (float)(j + 1), ccl::datatype::bfloat16);
+            peer_bufs.push_back(new DevBuf<uint16_t>(std::vector<uint16_t>(buf_elems, peer_val[j])));
+        }
+        int launches = 0;
+        ccl_fused_allreduce_fn allreduce = [&](void* buf, size_t n, const ccl_datatype& dt, ccl::reduction op, const void*, void* st) {
+            std::vector<const void*> peers;
+            for (auto* p : peer_bufs) peers.push_back(p->p);
+            ccl_sched s2; s2.stream = st;
+            ccl_comp_reduce_n(&s2, buf, peers, n, buf, dt, op, /*keep precision*/ 1);
+            launches++;
+        };
+        ccl_fusion_manager mgr(&backend, allreduce, cfg);
+        const int K = 700;
+        std::vector<std::vector<uint16_t>> host(K);
+        std::vector<DevBuf<uint16_t>*> send(K), recv(K);
+        std::vector<std::unique_ptr<ccl_fusion_request>> reqs(K);
+        int refused = 0;
+        for (int t = 0; t < K; t++) {
+            size_t n = 1 + (size_t)((t * 2654435761u) % 9000);     // up to 18 KB: some exceed the 16 KiB threshold
+            host[t].resize(n);
+            for (size_t i = 0; i < n; i++) host[t][i] = to_lp(0.001f * (float)((t * 31 + i) % 2001) - 1.0f, ccl::datatype::bfloat16);
+            send[t] = new DevBuf<uint16_t>(host[t]);
+            recv[t] = new DevBuf<uint16_t>(n + 4);
+            CK(hipMemset(recv[t]->p, 0, (n + 4) * 2));
+            reqs[t].reset(new ccl_fusion_request);
+            reqs[t]->send_buf = send[t]->p; reqs[t]->recv_buf = recv[t]->p; reqs[t]->count = n;
+            reqs[t]->dtype = DT(ccl::datatype::bfloat16); reqs[t]->reduction = ccl::reduction::sum; reqs[t]->stream = stream;
+            if (!mgr.add(reqs[t].get())) {      // too large to fuse: the caller runs it unfused
+                refused++;
+                std::vector<const void*> peers;
+                for (auto* p : peer_bufs) peers.push_back(p->p);
+                ccl_comp_reduce_n(&sched, send[t]->p, peers, n, recv[t]->p, DT(ccl::datatype::bfloat16), ccl::reduction::sum, 1);
+            }
+            if (t % 50 == 49) mgr.execute();
+        }
+        reqs[K - 1]->urgent = true;             // a waiter on the last request flushes what is left
+        for (int i = 0; i < 20; i++) mgr.execute();
+        CK(hipStreamSynchronize(stream));
+        bool all_done = true, all_ok = true;
+        for (int t = 0; t < K; t++) {
+            all_done = all_done && reqs[t]->is_completed();
+            std::vector<uint16_t> got = recv[t]->host();
+            std::vector<uint16_t> want = host[t];
+            std::vector<std::vector<uint16_t>> pv(NPEER);
+            std::vector<const void*> srcs = { want.data() };
+            for (int j = 0; j < NPEER; j++) { pv[j].assign(want.size(), peer_val[j]); srcs.push_back(pv[j].data()); }
+            std::vector<uint16_t> exp(want.size());
+            orc_reduce_n(srcs.data(), NPEER + 1, exp.data(), want.size(), ORC_BFLOAT16, ORC_SUM, 1, 0, (int)ccl::global_data::env().bf16_impl_type, ORC_FP16_AVX512F);
+            bool ok = memcmp(got.data(), exp.data(), want.size() * 2) == 0;
+            for (size_t i = want.size(); i < got.size(); i++) ok = ok && got[i] == 0;
+            if (!ok && all_ok) printf("  fused tensor %d (count %zu) differs\n", t, want.size());
+            all_ok = all_ok && ok;
+        }
+        EXPECT(all_done, "every fused request completed");
+        EXPECT(all_ok, "every tensor equals the 8-input reduce of its own data with the peers");
+        EXPECT(refused > 0 && mgr.stats().fused_ops == (size_t)(K - refused), "fused %zu + unfused %d = %d", mgr.stats().fused_ops, refused, K);
+        EXPECT(launches == (int)mgr.stats().fused_launches && launches >= 3 && launches < 40, "%d fused launches for %d requests", launches, K - refused);
+        mgr.reset();
+        for (auto* p : peer_bufs) delete p;
+        for (int t = 0; t < K; t++) { delete send[t]; delete recv[t]; }
     }
     CK(hipStreamDestroy(stream));
     printf("%d checks, %d failed\n", g_checks, g_fail);
