@@ -102,6 +102,15 @@ int mi_ccl_fp16_reduce(const void* in, size_t count, void* inout, int op, void* 
 int mi_ccl_comp_reduce_n(int dtype, int op, const void* const* srcs, int n, void* dst, size_t count,
                          int lp_mode, int bf16_impl, void* stream);
 
+/* The same reduce with the result stored to each of m buffers (1 <= m <= 16) in one pass: (n + m) x bytes of
+ * memory traffic instead of (n + 1 + 2(m - 1)) x bytes for a reduce followed by m - 1 copies.  dsts is a HOST
+ * array of m device pointers; a destination may be one of the sources.  Replaces allreduce_kernel
+ * (src/kernels/kernels.cl:190-217, launched from ze_onesided_allreduce_entry.cpp:66-108: n = 2, m = 2) and, with
+ * n == 1 and MI_CCL_LP_PAIRWISE (a byte copy for every dtype), write_monolithic_kernel_{1..7}
+ * (src/kernels/kernels.cl:423-560, launched from ze_a2a_allgatherv_entry.cpp:526-585: m = peer count). */
+int mi_ccl_comp_reduce_write_n(int dtype, int op, const void* const* srcs, int n, void* const* dsts, int m,
+                               size_t count, int lp_mode, int bf16_impl, void* stream);
+
 /* Slice form of the same: slice i starts at in_buf + offsets[i] elements (offsets: HOST array); inout is
  * slice 0 and receives the result.  Replaces ccl_comp_batch_reduce (src/comp/comp.cpp:202-249); the tmp and
  * acc scratch arrays of the reference are not needed.  keep_precision != 0 requires dtype bfloat16 and

@@ -24,7 +24,7 @@ DTYPE_SIZE = [1, 1, 2, 2, 4, 4, 8, 8, 2, 4, 8, 2]
 EXPORTS = [
     "mi_ccl_datatype_size", "mi_ccl_datatype_name", "mi_ccl_reduction_to_str", "mi_ccl_status_str",
     "mi_ccl_kernel_name", "mi_ccl_comp_reduce", "mi_ccl_bf16_reduce", "mi_ccl_fp16_reduce",
-    "mi_ccl_comp_reduce_n", "mi_ccl_comp_batch_reduce", "mi_ccl_comp_copy",
+    "mi_ccl_comp_reduce_n", "mi_ccl_comp_reduce_write_n", "mi_ccl_comp_batch_reduce", "mi_ccl_comp_copy",
     "mi_ccl_convert_fp32_to_bf16_arrays", "mi_ccl_convert_bf16_to_fp32_arrays", "mi_ccl_fusion_offsets",
     "mi_ccl_fusion_plan_create", "mi_ccl_fusion_plan_destroy", "mi_ccl_fusion_plan_bytes",
     "mi_ccl_fusion_plan_offset", "mi_ccl_fusion_pack", "mi_ccl_fusion_unpack", "mi_ccl_fusion_reduce",
@@ -61,6 +61,7 @@ def lib():
     L.mi_ccl_bf16_reduce.argtypes = [vp, sz, vp, i, i, vp]
     L.mi_ccl_fp16_reduce.argtypes = [vp, sz, vp, i, vp]
     L.mi_ccl_comp_reduce_n.argtypes = [i, i, vp, i, vp, sz, i, i, vp]
+    L.mi_ccl_comp_reduce_write_n.argtypes = [i, i, vp, i, vp, i, sz, i, i, vp]
     L.mi_ccl_comp_batch_reduce.argtypes = [vp, vp, sz, sz, vp, i, i, i, i, vp]
     L.mi_ccl_comp_copy.argtypes = [vp, vp, sz, i, vp]
     L.mi_ccl_convert_fp32_to_bf16_arrays.argtypes = [vp, vp, sz, i, vp]
@@ -149,6 +150,14 @@ def comp_reduce_n(dtype, op, srcs, dst, count, lp_mode=LP_PAIRWISE, bf16_impl=BF
     arr = _ptr_array(srcs)
     _check(lib().mi_ccl_comp_reduce_n(dtype, op, arr, len(srcs), _ptr(dst), count, lp_mode, bf16_impl,
                                       _stream(stream)), "mi_ccl_comp_reduce_n")
+
+
+def comp_reduce_write_n(dtype, op, srcs, dsts, count, lp_mode=LP_PAIRWISE, bf16_impl=BF16_AVX512BF, stream=None):
+    """Every dsts[k] = srcs[0] OP srcs[1] OP ... in argument order, one pass; one source and LP_PAIRWISE is a
+    copy of one buffer to len(dsts) buffers."""
+    s, d = _ptr_array(srcs), _ptr_array(dsts)
+    _check(lib().mi_ccl_comp_reduce_write_n(dtype, op, s, len(srcs), d, len(dsts), count, lp_mode, bf16_impl,
+                                            _stream(stream)), "mi_ccl_comp_reduce_write_n")
 
 
 def comp_batch_reduce(in_buf, offsets, count, inout, dtype, op, keep_precision, bf16_impl=BF16_AVX512BF,

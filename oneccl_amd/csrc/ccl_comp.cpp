@@ -197,3 +197,21 @@ ccl::status ccl_comp_reduce_n(ccl_sched* sched, const void* own_buf, const std::
                                           count, lp, (int)ccl::global_data::env().bf16_impl_type, stream_of(sched)),
                      "ccl_comp_reduce_n");
 }
+
+ccl::status ccl_comp_reduce_write_n(ccl_sched* sched, const void* own_buf, const std::vector<const void*>& peer_bufs,
+                                    size_t count, const std::vector<void*>& out_bufs, const ccl_datatype& dtype,
+                                    ccl::reduction reduction, int bf16_keep_precision_mode) {
+    if (!count)
+        return ccl::status::success;
+    if (reduction == ccl::reduction::custom)
+        fail("custom reduction is not available for the N-input device reduce");
+    std::vector<const void*> srcs;
+    srcs.reserve(peer_bufs.size() + 1);
+    srcs.push_back(own_buf);
+    srcs.insert(srcs.end(), peer_bufs.begin(), peer_bufs.end());
+    int lp = bf16_keep_precision_mode ? MI_CCL_LP_KEEP_PRECISION : MI_CCL_LP_PAIRWISE;
+    return to_status(mi_ccl_comp_reduce_write_n((int)dtype.idx(), (int)reduction, srcs.data(), (int)srcs.size(),
+                                                out_bufs.data(), (int)out_bufs.size(), count, lp,
+                                                (int)ccl::global_data::env().bf16_impl_type, stream_of(sched)),
+                     "ccl_comp_reduce_write_n");
+}

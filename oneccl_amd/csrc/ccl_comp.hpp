@@ -152,3 +152,10 @@ void ccl_convert_bf16_to_fp32_arrays(void* bf16_buf, float* fp32_buf, size_t cou
 ccl::status ccl_comp_reduce_n(ccl_sched* sched, const void* own_buf, const std::vector<const void*>& peer_bufs,
                               size_t count, void* out_buf, const ccl_datatype& dtype, ccl::reduction reduction,
                               int bf16_keep_precision_mode = 0);
+
+// The same reduce with the result stored to every buffer of out_bufs in one pass: the reference's allreduce_kernel
+// (src/kernels/kernels.cl:190-217: own and peer output) and, with no peers, write_monolithic_kernel_N
+// (src/kernels/kernels.cl:423-560: the own buffer copied to N peers).
+ccl::status ccl_comp_reduce_write_n(ccl_sched* sched, const void* own_buf, const std::vector<const void*>& peer_bufs,
+                                    size_t count, const std::vector<void*>& out_bufs, const ccl_datatype& dtype,
+                                    ccl::reduction reduction, int bf16_keep_precision_mode = 0);

@@ -131,13 +131,15 @@ static hipError_t dispatch(int dtype, bool keep, int bf16_impl, const LaunchArgs
     }
 }
 
-static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void* dst, size_t count, int lp_mode,
-                         int bf16_impl, void* stream) {
+static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void* const* dsts, int m, size_t count,
+                         int lp_mode, int bf16_impl, void* stream) {
     if (count == 0)
         return MI_CCL_SUCCESS;
+    if (m < 1 || m > kMaxDsts || !dsts)
+        return MI_CCL_INVALID_ARGUMENTS;
     if (dtype < 0 || dtype >= MI_CCL_DATATYPE_LAST || op < MI_CCL_SUM || op > MI_CCL_MAX)
         return MI_CCL_INVALID_ARGUMENTS;
-    if (n < 1 || n > kMaxSrcs || !srcs || !dst)
+    if (n < 1 || n > kMaxSrcs || !srcs)
         return MI_CCL_INVALID_ARGUMENTS;
     if (bf16_impl < MI_CCL_BF16_SCALAR || bf16_impl > MI_CCL_BF16_AVX512BF)
         return MI_CCL_INVALID_ARGUMENTS;
@@ -149,8 +151,9 @@ static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void
     if ((lp_mode & MI_CCL_LP_TAIL_QUIRK) && !keep)
         return MI_CCL_INVALID_ARGUMENTS;
     const size_t esz = kDtypeSize[dtype];
-    if (((uintptr_t)dst % esz) != 0)
-        return MI_CCL_INVALID_ARGUMENTS;
+    for (int k = 0; k < m; k++)
+        if (!dsts[k] || ((uintptr_t)dsts[k] % esz) != 0)
+            return MI_CCL_INVALID_ARGUMENTS;
     for (int j = 0; j < n; j++)
         if (!srcs[j] || ((uintptr_t)srcs[j] % esz) != 0)
             return MI_CCL_INVALID_ARGUMENTS;
@@ -158,7 +161,9 @@ static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void
     LaunchArgs a;
     a.srcs = srcs;
     a.n = n;
-    a.dst = dst;
+    a.dst = dsts[0];
+    a.dsts = dsts;
+    a.m = m;
     a.count = count;
     a.op = op;
     a.stream = (hipStream_t)stream;
@@ -176,8 +181,11 @@ static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void
         }
         const void* shifted[kMaxSrcs];
         for (int j = 0; j < n; j++) shifted[j] = (const char*)srcs[j] + limit * esz;
+        void* shifted_dst[kMaxDsts];
+        for (int k = 0; k < m; k++) shifted_dst[k] = (char*)dsts[k] + limit * esz;
         a.srcs = shifted;
-        a.dst = (char*)dst + limit * esz;
+        a.dst = shifted_dst[0];
+        a.dsts = shifted_dst;
         a.count = count - limit;
         return status_of(dispatch(dtype, true, MI_CCL_BF16_AVX512F, a));
     }
@@ -312,7 +320,7 @@ int mi_ccl_comp_reduce(int dtype, int op, const void* in, size_t count, void* in
     if (count == 0)
         return MI_CCL_SUCCESS;
     const void* srcs[2] = { inout, in };
-    return reduce_n_impl(dtype, op, srcs, 2, inout, count, MI_CCL_LP_PAIRWISE, bf16_impl, stream);
+    return reduce_n_impl(dtype, op, srcs, 2, &inout, 1, count, MI_CCL_LP_PAIRWISE, bf16_impl, stream);
 }
 
 int mi_ccl_bf16_reduce(const void* in, size_t count, void* inout, int op, int bf16_impl, void* stream) {
@@ -325,7 +333,12 @@ int mi_ccl_fp16_reduce(const void* in, size_t count, void* inout, int op, void* 
 
 int mi_ccl_comp_reduce_n(int dtype, int op, const void* const* srcs, int n, void* dst, size_t count, int lp_mode,
                          int bf16_impl, void* stream) {
-    return reduce_n_impl(dtype, op, srcs, n, dst, count, lp_mode, bf16_impl, stream);
+    return reduce_n_impl(dtype, op, srcs, n, &dst, 1, count, lp_mode, bf16_impl, stream);
+}
+
+int mi_ccl_comp_reduce_write_n(int dtype, int op, const void* const* srcs, int n, void* const* dsts, int m, size_t count,
+                               int lp_mode, int bf16_impl, void* stream) {
+    return reduce_n_impl(dtype, op, srcs, n, dsts, m, count, lp_mode, bf16_impl, stream);
 }
 
 int mi_ccl_comp_batch_reduce(const void* in_buf, const size_t* offsets, size_t n_offsets, size_t count, void* inout,
@@ -342,7 +355,7 @@ int mi_ccl_comp_batch_reduce(const void* in_buf, const size_t* offsets, size_t n
     srcs[0] = inout; /* inout_buf => in_buf + offsets[0] (comp.cpp:217) */
     for (size_t i = 1; i < n_offsets; i++) srcs[i] = (const char*)in_buf + kDtypeSize[dtype] * offsets[i];
     int lp = bf16_keep_precision_mode ? (MI_CCL_LP_KEEP_PRECISION | MI_CCL_LP_TAIL_QUIRK) : MI_CCL_LP_PAIRWISE;
-    return reduce_n_impl(dtype, op, srcs, (int)n_offsets, inout, count, lp, bf16_impl, stream);
+    return reduce_n_impl(dtype, op, srcs, (int)n_offsets, &inout, 1, count, lp, bf16_impl, stream);
 }
 
 int mi_ccl_comp_copy(const void* in, void* out, size_t bytes, int use_nontemporal, void* stream) {

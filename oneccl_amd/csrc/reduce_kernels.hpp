@@ -19,6 +19,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kBlock = 256;     // 4 wavefronts of 64 lanes
 constexpr int kMaxFixedN = 8;   // inputs unrolled at compile time
 constexpr int kMaxSrcs = 64;    // inputs of the run-time-N kernels
+constexpr int kMaxDsts = 16;    // outputs of the multi-destination kernels
 
 enum { OP_SUM = 0, OP_PROD = 1, OP_MIN = 2, OP_MAX = 3 };
 
@@ -28,6 +29,9 @@ struct SrcTable {               // by-value kernel argument
 template <int N>
 struct SrcFixed {
     const void* p[N];
+};
+struct DstTable {               // by-value kernel argument
+    void* p[kMaxDsts];
 };
 
 struct Tuning {
@@ -48,6 +52,8 @@ struct LaunchArgs {
     int op;
     hipStream_t stream;
     Tuning tune;
+    void* const* dsts = nullptr;    // m > 1: host array of m device pointers, the result goes to each (dst is unused)
+    int m = 1;
 };
 
 // ---------------------------------------------------------------------------------------------------
@@ -623,6 +629,121 @@ reduce_elem_kernel(SrcTable src, int n, void* dst, uint64_t count) {
 }
 
 // ---------------------------------------------------------------------------------------------------
+// Several destinations: the reduced vector is stored to each of m buffers (the reference's allreduce_kernel stores
+// to the own and to the peer's output, kernels.cl:190-217; with one input this is write_monolithic_kernel_N,
+// kernels.cl:423-560).  Inputs and outputs are run-time counts.  A lane reads its element from every input before
+// it stores it anywhere, so a destination may be one of the inputs.
+
+template <class TR, int OP, int UNROLL>
+__device__ __forceinline__ void reduce_rt_tile(const SrcTable& src, int n, uint32_t head, const uint64_t (&idx)[UNROLL],
+                                               uint64_t nvec, u32x4 (&out)[UNROLL]) {
+    typedef typename TR::elem_t E;
+    Accs<TR> a[UNROLL];
+    const u32x4* s0 = (const u32x4*)((const E*)src.p[0] + head);
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) a[u] = vec_init<TR>((idx[u] < nvec) ? ld_stream(s0 + idx[u]) : u32x4{ 0, 0, 0, 0 });
+    for (int j = 1; j < n; j++) {
+        const u32x4* sj = (const u32x4*)((const E*)src.p[j] + head);
+        u32x4 x[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) x[u] = (idx[u] < nvec) ? ld_stream(sj + idx[u]) : u32x4{ 0, 0, 0, 0 };
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) vec_step<TR, OP>(x[u], a[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) out[u] = vec_finish<TR>(a[u]);
+}
+
+template <class TR, int OP>
+__device__ __forceinline__ void reduce_multi_edges(const SrcTable& src, int n, const DstTable& dst, int m, uint32_t head,
+                                                   uint64_t nvec, uint32_t tail) {
+    typedef typename TR::elem_t E;
+    uint32_t t = threadIdx.x;
+    if (t < head + tail) {
+        uint64_t i = (t < head) ? t : (uint64_t)head + nvec * TR::VEC + (t - head);
+        typename TR::acc_t a = TR::init(((const E*)src.p[0])[i]);
+        for (int j = 1; j < n; j++) a = TR::template step<OP>(((const E*)src.p[j])[i], a);
+        const E r = TR::finish(a);
+        for (int k = 0; k < m; k++) ((E*)dst.p[k])[i] = r;
+    }
+}
+
+template <class TR, int OP, int UNROLL>
+__global__ void __launch_bounds__(kBlock)
+reduce_multi_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uint64_t nvec, uint32_t tail,
+                    int xcd_chunked) {
+    typedef typename TR::elem_t E;
+    constexpr uint64_t kTile = (uint64_t)kBlock * UNROLL;
+    const uint64_t ntiles = (nvec + kTile - 1) / kTile;
+    for (TileIter it(ntiles, xcd_chunked); it.tile < it.end; it.tile += it.stride) {
+        uint64_t idx[UNROLL];
+        u32x4 v[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) idx[u] = it.tile * kTile + threadIdx.x + (uint64_t)u * kBlock;
+        reduce_rt_tile<TR, OP, UNROLL>(src, n, head, idx, nvec, v);
+        for (int k = 0; k < m; k++) {
+            u32x4* d = (u32x4*)((E*)dst.p[k] + head);
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++)
+                if (idx[u] < nvec) st_stream(d + idx[u], v[u]);
+        }
+    }
+    if (blockIdx.x == 0 && (head | tail)) reduce_multi_edges<TR, OP>(src, n, dst, m, head, nvec, tail);
+}
+
+// The phased form of the same: kPhaseU vectors per lane are reduced into LDS while HBM sees only reads, then stored
+// to every destination while it sees only writes.
+template <class TR, int OP>
+__global__ void __launch_bounds__(kPhaseBlock)
+reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uint64_t nvec, uint32_t tail,
+                           PhaseSync* ps) {
+    typedef typename TR::elem_t E;
+    constexpr int G = 4;
+    static_assert(kPhaseU % G == 0, "LDS steps must be a multiple of the group size");
+    __shared__ u32x4 stage[kPhaseU * kPhaseBlock];
+    const uint64_t gthreads = (uint64_t)gridDim.x * kPhaseBlock;
+    const uint64_t gtid = (uint64_t)blockIdx.x * kPhaseBlock + threadIdx.x;
+    const uint64_t per_phase = gthreads * kPhaseU;
+    bool give_up = false;
+    unsigned gen = 0;
+    if (threadIdx.x == 0) gen = MI_ALOAD(&ps->rel.v);
+    for (uint64_t p0 = 0; p0 < nvec; p0 += per_phase) {
+        for (int u = 0; u < kPhaseU; u += G) {
+            uint64_t idx[G];
+            u32x4 v[G];
+#pragma unroll
+            for (int g = 0; g < G; g++) idx[g] = p0 + (uint64_t)(u + g) * gthreads + gtid;
+            reduce_rt_tile<TR, OP, G>(src, n, head, idx, nvec, v);
+#pragma unroll
+            for (int g = 0; g < G; g++) stage[(u + g) * kPhaseBlock + threadIdx.x] = v[g];
+        }
+        phase_barrier(ps, ++gen, give_up);
+        for (int k = 0; k < m; k++) {
+            u32x4* d = (u32x4*)((E*)dst.p[k] + head);
+            for (int u = 0; u < kPhaseU; u++) {
+                const uint64_t i = p0 + (uint64_t)u * gthreads + gtid;
+                if (i < nvec) st_stream(d + i, stage[u * kPhaseBlock + threadIdx.x]);
+            }
+        }
+        phase_barrier(ps, ++gen, give_up);
+    }
+    if (blockIdx.x == 0 && (head | tail)) reduce_multi_edges<TR, OP>(src, n, dst, m, head, nvec, tail);
+}
+
+template <class TR, int OP>
+__global__ void __launch_bounds__(kBlock)
+reduce_multi_elem_kernel(SrcTable src, int n, DstTable dst, int m, uint64_t count) {
+    typedef typename TR::elem_t E;
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < count; i += stride) {
+        typename TR::acc_t a = TR::init(((const E*)src.p[0])[i]);
+        for (int j = 1; j < n; j++) a = TR::template step<OP>(((const E*)src.p[j])[i], a);
+        const E r = TR::finish(a);
+        for (int k = 0; k < m; k++) ((E*)dst.p[k])[i] = r;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
 // host-side launch
 
 inline int grid_for(uint64_t ntiles, const Tuning& t) {
@@ -687,9 +808,48 @@ inline hipError_t launch_fixed_unroll(const LaunchArgs& a, uint32_t head, uint64
 }
 
 template <class TR, int OP>
+inline hipError_t launch_multi_op(const LaunchArgs& a) {
+    typedef typename TR::elem_t E;
+    constexpr uint32_t VEC = TR::VEC;
+    SrcTable s;
+    DstTable d;
+    for (int j = 0; j < a.n; j++) s.p[j] = a.srcs[j];
+    for (int k = 0; k < a.m; k++) d.p[k] = a.dsts[k];
+    const uintptr_t mis = (uintptr_t)a.dsts[0] & 15u;
+    bool same = true;
+    for (int j = 0; j < a.n; j++) same = same && (((uintptr_t)a.srcs[j] & 15u) == mis);
+    for (int k = 0; k < a.m; k++) same = same && (((uintptr_t)a.dsts[k] & 15u) == mis);
+    if (!same || (mis % sizeof(E)) != 0) {
+        int grid = grid_for((a.count + kBlock - 1) / kBlock, a.tune);
+        hipLaunchKernelGGL((reduce_multi_elem_kernel<TR, OP>), dim3(grid), dim3(kBlock), 0, a.stream, s, a.n, d, a.m,
+                           (uint64_t)a.count);
+        return hipGetLastError();
+    }
+    uint64_t head = mis ? (16u - mis) / sizeof(E) : 0;
+    if (head > a.count) head = a.count;
+    const uint64_t nvec = (a.count - head) / VEC;
+    const uint32_t tail = (uint32_t)(a.count - head - nvec * VEC);
+    const bool can = a.tune.sync != nullptr && a.tune.num_cus >= kPhaseGroups;
+    const uint64_t traffic = (uint64_t)(a.n + a.m) * nvec * 16u;
+    if (can && (a.tune.variant == 8 || (a.tune.variant == 0 && traffic >= (uint64_t)a.tune.phased_min_bytes))) {
+        int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
+        hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
+                           a.m, (uint32_t)head, nvec, tail, a.tune.sync);
+        return hipGetLastError();
+    }
+    constexpr int UNROLL = 4;
+    const uint64_t tile = (uint64_t)kBlock * UNROLL;
+    int grid = grid_for((nvec + tile - 1) / tile, a.tune);
+    hipLaunchKernelGGL((reduce_multi_kernel<TR, OP, UNROLL>), dim3(grid), dim3(kBlock), 0, a.stream, s, a.n, d, a.m,
+                       (uint32_t)head, nvec, tail, a.tune.xcd_chunked);
+    return hipGetLastError();
+}
+
+template <class TR, int OP>
 inline hipError_t launch_op(const LaunchArgs& a) {
     typedef typename TR::elem_t E;
     constexpr uint32_t VEC = TR::VEC;
+    if (a.m > 1) return launch_multi_op<TR, OP>(a);
     // common misalignment of all buffers to 16 bytes, in elements; mixed misalignment -> element kernel
     const uintptr_t mis = (uintptr_t)a.dst & 15u;
     bool same = true;

@@ -22,6 +22,8 @@
  *   orc_convert_*_arrays tail       recorded probe values of the reference library (tail truncation)
  *   orc_comp_batch_reduce           composition; recorded probe values (1+3*2^-8 -> 3f82 body / 3f81 tail)
  *   orc_fusion_*                    pack/unpack round trip, offsets closed form
+ *   orc_reduce_write_n              composition of orc_reduce_n (pinned above) and memcpy: every destination equals
+ *                                   orc_reduce_n's output; closed forms of the reference's functional tests
  * NaN payload and sign of NaN *results* are not pinned by the reference itself (operand order of a
  * commutative SSE/AVX add is the compiler's choice); tests compare NaN-ness only.
  */
@@ -366,6 +368,25 @@ int orc_reduce_n(const void* const* srcs, int n, void* dst, size_t count, int dt
     reduce_n_range(srcs, n, dst, 0, count, count, dtype, op, lp_keep_precision, quirk_tail, bf16_impl,
                    fp16_impl);
     return ORC_OK;
+}
+
+/* kernels.cl:190-217 and :423-560: every element is read from all inputs before it is stored anywhere, so the
+ * result is formed apart and copied out; that also covers a destination that is one of the sources. */
+int orc_reduce_write_n(const void* const* srcs, int n, void* const* dsts, int m, size_t count, int dtype, int op,
+                       int lp_keep_precision, int quirk_tail, int bf16_impl, int fp16_impl) {
+    size_t esz = orc_datatype_size(dtype);
+    if (esz == 0 || m < 1)
+        return ORC_INVALID_ARGUMENTS;
+    if (count == 0)
+        return ORC_OK;
+    void* res = malloc(count * esz);
+    if (!res)
+        return ORC_INVALID_ARGUMENTS;
+    int rc = orc_reduce_n(srcs, n, res, count, dtype, op, lp_keep_precision, quirk_tail, bf16_impl, fp16_impl);
+    if (rc == ORC_OK)
+        for (int k = 0; k < m; k++) memcpy(dsts[k], res, count * esz);
+    free(res);
+    return rc;
 }
 
 struct mt_job {

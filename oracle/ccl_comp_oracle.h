@@ -67,6 +67,12 @@ int orc_comp_batch_reduce(const void* in_buf, const size_t* offsets, size_t n_of
 int orc_reduce_n(const void* const* srcs, int n, void* dst, size_t count, int dtype, int op,
                  int lp_keep_precision, int quirk_tail, int bf16_impl, int fp16_impl);
 
+/* The N-input reduce whose result goes to m buffers: allreduce_kernel (kernels.cl:190-217: one reduce, the result
+ * stored to the own and to the peer's output) and, with n == 1, write_monolithic_kernel_N (kernels.cl:423-560: one
+ * input copied to N peers).  Same arithmetic as orc_reduce_n; a destination may be one of the sources. */
+int orc_reduce_write_n(const void* const* srcs, int n, void* const* dsts, int m, size_t count, int dtype, int op,
+                       int lp_keep_precision, int quirk_tail, int bf16_impl, int fp16_impl);
+
 /* comp.cpp:60-74 */
 int orc_comp_copy(const void* in, void* out, size_t bytes);
 

@@ -69,6 +69,8 @@ def lib():
         L.orc_reduce_n.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int,
                                    C.c_int, C.c_int, C.c_int]
         L.orc_reduce_n_mt.argtypes = L.orc_reduce_n.argtypes + [C.c_int]
+        L.orc_reduce_write_n.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_size_t, C.c_int, C.c_int,
+                                         C.c_int, C.c_int, C.c_int, C.c_int]
         L.orc_comp_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         L.orc_fusion_offsets.restype = C.c_size_t
         L.orc_fusion_offsets.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p]
@@ -126,6 +128,22 @@ def reduce_n(srcs, dtype, op, keep=0, quirk_tail=0, bf16_impl=BF16_AVX512BF, fp1
         rc = lib().orc_reduce_n(ptrs, n, _vp(out), count, dtype, op, keep, quirk_tail, bf16_impl, fp16_impl)
     assert rc == 0, rc
     return out
+
+
+def reduce_write_n(srcs, m, dtype, op, keep=0, quirk_tail=0, bf16_impl=BF16_AVX512BF, fp16_impl=FP16_AVX512F,
+                   alias=None):
+    """The N-input reduce stored to m buffers; returns the m arrays.  alias = (k, j): destination k IS source j
+    (a private copy of the sources is reduced, so the caller's arrays stay as they were)."""
+    srcs = [np.ascontiguousarray(s).copy() for s in srcs]
+    outs = [np.empty_like(srcs[0]) for _ in range(m)]
+    if alias is not None:
+        outs[alias[0]] = srcs[alias[1]]
+    sp = (C.c_void_p * len(srcs))(*[s.ctypes.data for s in srcs])
+    dp = (C.c_void_p * m)(*[o.ctypes.data for o in outs])
+    rc = lib().orc_reduce_write_n(sp, len(srcs), dp, m, srcs[0].size, dtype, op, keep, quirk_tail, bf16_impl,
+                                  fp16_impl)
+    assert rc == 0, rc
+    return outs
 
 
 def batch_reduce(buf, offsets, count, dtype, op, keep, bf16_impl=BF16_AVX512BF, fp16_impl=FP16_AVX512F):

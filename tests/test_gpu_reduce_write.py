@@ -1,0 +1,154 @@
+"""GPU parity of mi_ccl_comp_reduce_write_n (one N-input reduce stored to m buffers; with one input, a copy to m
+buffers) against the oracle, through the C ABI.  Bit-exact; two NaNs of a floating type compare equal."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from gpu_util import assert_same, make_inputs, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def comp():
+    import torch
+    assert torch.cuda.is_available(), "needs a GPU"
+    import oneccl_amd.comp as c
+    c.lib()
+    return c
+
+
+def lp_variants(dtype):
+    if dtype == O.BFLOAT16:
+        return [(0, 0, 0, 0), (0, 1, 0, 0), (0, 2, 0, 0), (1, 2, 1, 0), (3, 2, 1, 1)]
+    return [(0, 2, 0, 0)]
+
+
+@pytest.mark.parametrize("dtype", range(12))
+@pytest.mark.parametrize("op", range(4))
+def test_reduce_write_n_all_dtypes_ops(comp, dtype, op):
+    import torch
+    rng = np.random.default_rng(5000 + dtype * 4 + op)
+    for n, m in [(1, 1), (1, 2), (1, 7), (2, 2), (3, 5), (8, 8), (9, 3), (16, 16)]:
+        for count in (1, 15, 17, 1000, 4099, 70001):
+            if n > 8 and count < 1000:
+                continue
+            kind = "bits" if dtype in (O.FLOAT16, O.BFLOAT16) and count % 2 else "config"
+            srcs = make_inputs(rng, dtype, count, op, n, kind)
+            d = [to_dev(s) for s in srcs]
+            for lp, impl, keep, quirk in lp_variants(dtype):
+                outs = [torch.zeros(count + 8, dtype=d[0].dtype, device="cuda") for _ in range(m)]
+                comp.comp_reduce_write_n(dtype, op, d, outs, count, lp_mode=lp, bf16_impl=impl)
+                torch.cuda.synchronize()
+                want = O.reduce_write_n(srcs, m, dtype, op, keep=keep, quirk_tail=quirk, bf16_impl=impl)
+                for k in range(m):
+                    got = to_host(outs[k], O.NP_STORAGE[dtype])
+                    assert_same(got[:count], want[k], dtype,
+                                f"dtype={O.DTYPE_NAMES[dtype]} op={O.OP_NAMES[op]} n={n} m={m} k={k} count={count} "
+                                f"lp={lp} impl={impl}")
+                    assert not got[count:].view(np.uint8).any(), "wrote past the end"
+
+
+def test_one_input_is_a_byte_copy_for_every_dtype(comp):
+    """write_monolithic_kernel_N: the input reaches every peer buffer unchanged, whatever bits it holds."""
+    import torch
+    rng = np.random.default_rng(11)
+    for dtype in range(12):
+        esz = O.NP_STORAGE[dtype]().itemsize
+        src = rng.integers(0, 256, 30011 * esz, dtype=np.uint8)
+        d = torch.from_numpy(src.copy()).cuda()
+        outs = [torch.zeros_like(d) for _ in range(7)]
+        comp.comp_reduce_write_n(dtype, O.SUM, [d], outs, 30011)
+        torch.cuda.synchronize()
+        for o in outs:
+            assert (o.cpu().numpy() == src).all(), O.DTYPE_NAMES[dtype]
+
+
+@pytest.mark.parametrize("variant", [2, 8])
+def test_destination_aliases_a_source_and_misaligned_buffers(comp, variant):
+    """In place (destination k is source j, as allreduce_kernel's output may be its input), buffers that share a
+    misalignment to 16 bytes (vector path with head and tail) and buffers that do not (element path)."""
+    import torch
+    rng = np.random.default_rng(12)
+    comp.set_param("variant", variant)
+    try:
+        for dtype, op in [(O.BFLOAT16, O.SUM), (O.FLOAT32, O.MIN), (O.INT16, O.PROD), (O.FLOAT64, O.SUM)]:
+            np_t = O.NP_STORAGE[dtype]
+            count, n, m = 50021, 4, 3
+            srcs = make_inputs(rng, dtype, count, op, n)
+            keep = 1 if dtype == O.BFLOAT16 else 0
+            # in place
+            d = [to_dev(s) for s in srcs]
+            outs = [d[2], torch.empty_like(d[0]), d[0]]
+            comp.comp_reduce_write_n(dtype, op, d, outs, count, lp_mode=keep)
+            torch.cuda.synchronize()
+            want = O.reduce_n(srcs, dtype, op, keep=keep)
+            for o in outs:
+                assert_same(to_host(o, np_t), want, dtype, f"in place {O.DTYPE_NAMES[dtype]}")
+            # shared and mixed misalignment, in elements
+            for offs_s, offs_d in [([3, 3, 3, 3], [3, 3, 3]), ([0, 1, 2, 3], [1, 0, 5])]:
+                if np.dtype(np_t).itemsize == 8:
+                    offs_s, offs_d = [o % 2 for o in offs_s], [o % 2 for o in offs_d]
+                big = [to_dev(np.concatenate([np.zeros(o, np_t), s])) for o, s in zip(offs_s, srcs)]
+                dv = [b[o:] for b, o in zip(big, offs_s)]
+                obig = [torch.zeros(count + o + 4, dtype=dv[0].dtype, device="cuda") for o in offs_d]
+                ov = [b[o:] for b, o in zip(obig, offs_d)]
+                comp.comp_reduce_write_n(dtype, op, dv, ov, count, lp_mode=keep)
+                torch.cuda.synchronize()
+                for b, o in zip(obig, offs_d):
+                    got = to_host(b, np_t)
+                    assert_same(got[o:o + count], want, dtype, f"misaligned {offs_s} {offs_d}")
+                    assert not got[:o].view(np.uint8).any() and not got[o + count:].view(np.uint8).any()
+    finally:
+        comp.set_param("variant", 0)
+
+
+def test_phased_form_over_several_phases(comp):
+    """The phased kernel forced on (variant 8) from a few elements to several phases of one launch
+    (a phase holds gridDim x 512 x 20 vectors = about 42 MB per buffer)."""
+    import torch
+    rng = np.random.default_rng(13)
+    comp.set_param("variant", 8)
+    try:
+        for dtype, n, m, count in [(O.BFLOAT16, 8, 2, 5), (O.BFLOAT16, 8, 8, 50_000_017), (O.FLOAT32, 2, 2, 23_000_003),
+                                   (O.UINT8, 1, 7, 100_000_001)]:
+            np_t = O.NP_STORAGE[dtype]
+            srcs = make_inputs(rng, dtype, count, O.SUM, n)
+            d = [to_dev(s) for s in srcs]
+            outs = [torch.empty_like(d[0]) for _ in range(m)]
+            keep = 1 if dtype == O.BFLOAT16 else 0
+            comp.comp_reduce_write_n(dtype, O.SUM, d, outs, count, lp_mode=keep)
+            torch.cuda.synchronize()
+            want = O.reduce_n(srcs, dtype, O.SUM, keep=keep, threads=8)
+            for o in outs:
+                assert_same(to_host(o, np_t), want, dtype, f"phased {O.DTYPE_NAMES[dtype]} n={n} m={m} count={count}")
+    finally:
+        comp.set_param("variant", 0)
+
+
+def test_equals_reduce_n_followed_by_copies_at_a_large_size(comp):
+    """Size-independent property at 1 GiB per buffer: every destination equals mi_ccl_comp_reduce_n's output."""
+    import torch
+    count = 1 << 29
+    g = torch.Generator(device="cuda")
+    g.manual_seed(3)
+    srcs = [torch.empty(count, dtype=torch.bfloat16, device="cuda").normal_(0, 1e-3, generator=g) for _ in range(4)]
+    ref = torch.empty_like(srcs[0])
+    comp.comp_reduce_n(O.BFLOAT16, O.SUM, srcs, ref, count, lp_mode=1)
+    outs = [torch.empty_like(ref) for _ in range(4)]
+    comp.comp_reduce_write_n(O.BFLOAT16, O.SUM, srcs, outs, count, lp_mode=1)
+    torch.cuda.synchronize()
+    for o in outs:
+        assert torch.equal(o.view(torch.int16), ref.view(torch.int16))
+
+
+def test_errors(comp):
+    import torch
+    a = torch.zeros(64, dtype=torch.float32, device="cuda")
+    with pytest.raises(comp.CclError):
+        comp.comp_reduce_write_n(O.FLOAT32, O.SUM, [a], [a] * 17, 64)
+    with pytest.raises(comp.CclError):
+        comp.comp_reduce_write_n(O.FLOAT32, 4, [a], [a], 64)
+    with pytest.raises(comp.CclError):
+        comp.comp_reduce_write_n(O.FLOAT32, O.SUM, [a], [a], 64, lp_mode=1)     # keep precision is for bf16
+    comp.comp_reduce_write_n(O.FLOAT32, O.SUM, [a], [a, a], 0)                  # count 0: nothing to do

@@ -437,3 +437,29 @@ def test_against_reference_code_every_bf16_pair_sampled():
     assert R.ref_bf16_reduce(a.ctypes.data, a.size, want.ctypes.data, O.SUM, 2) == 0
     got = O.comp_reduce(a, b, O.BFLOAT16, O.SUM, bf16_impl=2)
     assert O.same_bits_or_both_nan(got, want, O.BFLOAT16).all()
+
+
+def test_reduce_write_n_is_reduce_n_stored_m_times():
+    """allreduce_kernel (kernels.cl:190-217) stores one reduce to two outputs, write_monolithic_kernel_N
+    (kernels.cl:423-560) copies one input to N: every destination must equal orc_reduce_n's result, also when a
+    destination is one of the sources, and one input in pairwise mode must come back byte for byte."""
+    rng = np.random.default_rng(77)
+    for dtype, op, n, m in [(O.BFLOAT16, O.SUM, 2, 2), (O.FLOAT32, O.MAX, 3, 4), (O.INT8, O.PROD, 8, 7),
+                            (O.FLOAT16, O.MIN, 5, 1)]:
+        np_t = O.NP_STORAGE[dtype]
+        srcs = [rng.integers(0, 256, 1003 * np.dtype(np_t).itemsize, dtype=np.uint8).view(np_t) for _ in range(n)]
+        if dtype == O.FLOAT32:
+            srcs = [rng.standard_normal(1003).astype(np.float32) for _ in range(n)]
+        want = O.reduce_n(srcs, dtype, op)
+        for alias in (None, (m - 1, n - 1)):
+            outs = O.reduce_write_n(srcs, m, dtype, op, alias=alias)
+            for o in outs:
+                assert O.same_bits_or_both_nan(o, want, dtype).all()
+    src = rng.integers(0, 65536, 517, dtype=np.uint16)      # any bf16 bit pattern, NaNs and denormals included
+    for o in O.reduce_write_n([src], 7, O.BFLOAT16, O.SUM):
+        assert (o == src).all()
+    # closed form of the reference's functional tests (test_impl.hpp:242-324): rank r sends r + i
+    n, cnt = 8, 64
+    srcs = [(np.arange(cnt) % 5 + r).astype(np.float32) for r in range(n)]
+    for o in O.reduce_write_n(srcs, 8, O.FLOAT32, O.SUM):
+        assert (o == n * (n - 1) / 2 + n * (np.arange(cnt) % 5)).all()
