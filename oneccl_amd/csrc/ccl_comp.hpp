@@ -18,6 +18,7 @@
 #include <stdint.h>
 
 #include <exception>
+#include <memory>
 #include <string>
 #include <vector>
 
@@ -117,9 +118,28 @@ private:
     std::string names[12];
 };
 
-// What this path needs of a schedule: the stream its kernels go to (a hipStream_t).
+// What this path needs of a schedule (src/sched/sched.hpp, src/sched/sched_base.hpp): the stream its kernels go to
+// (a hipStream_t), the user's reduction callback and match id (ccl_coll_attr, src/coll/coll_param.hpp), and -- for
+// callers that drive scheduler entries, ccl_sched_entry.hpp -- the entry list with the reference's progress rule.
+struct ccl_coll_attr {
+    ccl::reduction_fn reduction_fn = nullptr;
+    std::string match_id;
+};
+class sched_entry;
 struct ccl_sched {
     void* stream = nullptr;
+    ccl_coll_attr coll_attr;
+
+    // the rest is defined in ccl_sched_entry.cpp and only needed with entries
+    std::vector<std::shared_ptr<void>> owned_buffers;      // declared before the entries: destroyed after them
+    std::vector<std::shared_ptr<sched_entry>> entries;
+    size_t start_idx = 0;
+    sched_entry* add_entry(std::shared_ptr<sched_entry> entry);
+    void add_barrier();                         // the last entry becomes a barrier (src/sched/sched.cpp:596-605)
+    void do_progress();                         // src/sched/sched.cpp:439-490
+    bool is_completed() const { return start_idx == entries.size(); }
+    void renew();                               // every entry back to not_started, for the next run of the schedule
+    void* alloc_buffer(size_t bytes);           // device memory owned by the schedule (sched_base.cpp alloc_buffer)
 };
 
 // src/comp/comp.hpp:23-51

@@ -32,3 +32,14 @@ def test_cpp_surface_default_env():
 def test_cpp_surface_ccl_bf16_knob(impl, idx):
     out = run({"CCL_BF16": impl})
     assert f"bf16 impl {idx}" in out
+
+
+def test_scheduler_entries_and_device_custom_reduction():
+    """tests/cpp/test_sched_entries.cpp: COPY / RECV_REDUCE / REDUCE_LOCAL / REDUCE_MONOLITHIC / WRITE_MONOLITHIC
+    entries driven by ccl_sched::do_progress over a loop-back transport, and the device-functor custom reduction."""
+    exe = os.path.join(HERE, "cpp", "test_sched_entries")
+    if not os.path.exists(exe):
+        pytest.fail("tests/cpp/test_sched_entries is not built: run __graft_entry__.build()")
+    p = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stdout[-4000:] + p.stderr[-2000:]
+    assert "0 failed" in p.stdout
