@@ -55,6 +55,12 @@ enum mi_ccl_status {
  *            min/max as avx512f */
 enum mi_ccl_bf16_impl { MI_CCL_BF16_SCALAR = 0, MI_CCL_BF16_AVX512F = 1, MI_CCL_BF16_AVX512BF = 2 };
 
+/* ccl_fp16_impl_type, src/comp/fp16/fp16_utils.hpp:26-32 (CCL_FP16, env.cpp:715-720).  f16c and avx512f work
+ * through fp32 and give the same bits; avx512fp16 works on the fp16 values (fp16_intrisics.cpp:24-35): same bits
+ * for sum and prod, and min/max return the chosen operand untouched where the other two quiet a signalling NaN.
+ * Process-wide like the reference's: mi_ccl_set_param("fp16_impl", value); default avx512f. */
+enum mi_ccl_fp16_impl { MI_CCL_FP16_F16C = 2, MI_CCL_FP16_AVX512F = 3, MI_CCL_FP16_AVX512FP16 = 4 };
+
 /* How 16-bit floating types are carried through an N-input reduce (flags, OR them):
  *   MI_CCL_LP_PAIRWISE        round to the 16-bit type after every pair: a chain of ccl_comp_reduce calls
  *                             (comp.cpp:236-245; the only mode the reference has for float16)
@@ -170,7 +176,8 @@ int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* ow
 /* Launch-shape knobs, the counterpart of CCL_KERNEL_GROUP_SIZE / CCL_KERNEL_MEM_ALIGN
  * (src/common/env/env.cpp:251-253).  Names: "waves_per_cu" (resident blocks per CU the grid is sized
  * for), "max_blocks" (cap on the grid; 0 = no cap), "xcd_chunked" (0/1: give each of the 8 XCDs one
- * contiguous share of the buffer), "variant" (kernel variant selector, 0 = default).
+ * contiguous share of the buffer), "variant" (kernel variant selector, 0 = default), "phased_min_bytes",
+ * and "fp16_impl" (enum mi_ccl_fp16_impl above).
  * Returns invalid_arguments for an unknown name or out-of-range value. */
 int mi_ccl_set_param(const char* name, long value);
 long mi_ccl_get_param(const char* name);

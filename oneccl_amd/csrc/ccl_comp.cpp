@@ -45,10 +45,25 @@ ccl::env_data parse_env() {
             e.fp16_impl_type = ccl_fp16_f16c;
         else if (!strcmp(v, "avx512f"))
             e.fp16_impl_type = ccl_fp16_avx512f;
+        else if (!strcmp(v, "avx512fp16"))
+            e.fp16_impl_type = ccl_fp16_avx512fp16;
         else
             fail(std::string("unsupported FP16 impl type: ") + v);
     }
     return e;
+}
+
+// the library's float16 mode follows ccl::global_data::env().fp16_impl_type, which a caller may also set by hand
+int bf16_impl_for(const ccl_datatype& dtype) {
+    const ccl::env_data& e = ccl::global_data::env();
+    if (dtype.idx() == ccl::datatype::float16) {
+        int impl = (int)e.fp16_impl_type;
+        if (impl < MI_CCL_FP16_F16C || impl > MI_CCL_FP16_AVX512FP16)
+            fail("float16 reduction needs fp16_impl_type f16c, avx512f or avx512fp16");     // fp16.cpp:41-53 has no other path
+        if (mi_ccl_get_param("fp16_impl") != impl)
+            mi_ccl_set_param("fp16_impl", impl);
+    }
+    return (int)e.bf16_impl_type;
 }
 
 // ccl::reduction::custom: the callback is host code, so both buffers are staged to the host and the result is
@@ -126,7 +141,7 @@ ccl::status ccl_comp_reduce(ccl_sched* sched, const void* in_buf, size_t in_coun
     if (out_count && (dtype.idx() == ccl::datatype::bfloat16 || dtype.idx() == ccl::datatype::float16))
         *out_count = in_count;
     return to_status(mi_ccl_comp_reduce((int)dtype.idx(), (int)reduction, in_buf, in_count, inout_buf,
-                                        (int)ccl::global_data::env().bf16_impl_type, stream_of(sched)),
+                                        bf16_impl_for(dtype), stream_of(sched)),
                      "ccl_comp_reduce");
 }
 
@@ -150,7 +165,7 @@ ccl::status ccl_comp_batch_reduce(const void* in_buf, const std::vector<size_t>&
         *out_count = in_count;
     return to_status(mi_ccl_comp_batch_reduce(in_buf, offsets.data(), offsets.size(), in_count, inout_buf,
                                               (int)dtype.idx(), (int)reduction, bf16_keep_precision_mode,
-                                              (int)ccl::global_data::env().bf16_impl_type, stream_of(sched)),
+                                              bf16_impl_for(dtype), stream_of(sched)),
                      "ccl_comp_batch_reduce");
 }
 
@@ -167,6 +182,7 @@ void ccl_fp16_reduce(const void* in_buf, size_t in_cnt, void* inout_buf, size_t*
                      ccl_sched* sched) {
     if (out_cnt)
         *out_cnt = in_cnt;                                             // fp16.cpp:48-50
+    bf16_impl_for(ccl_datatype_storage::instance().get(ccl::datatype::float16));
     to_status(mi_ccl_fp16_reduce(in_buf, in_cnt, inout_buf, (int)reduction_op, stream_of(sched)), "ccl_fp16_reduce");
 }
 
@@ -194,7 +210,7 @@ ccl::status ccl_comp_reduce_n(ccl_sched* sched, const void* own_buf, const std::
     srcs.insert(srcs.end(), peer_bufs.begin(), peer_bufs.end());
     int lp = bf16_keep_precision_mode ? MI_CCL_LP_KEEP_PRECISION : MI_CCL_LP_PAIRWISE;
     return to_status(mi_ccl_comp_reduce_n((int)dtype.idx(), (int)reduction, srcs.data(), (int)srcs.size(), out_buf,
-                                          count, lp, (int)ccl::global_data::env().bf16_impl_type, stream_of(sched)),
+                                          count, lp, bf16_impl_for(dtype), stream_of(sched)),
                      "ccl_comp_reduce_n");
 }
 
@@ -212,6 +228,6 @@ ccl::status ccl_comp_reduce_write_n(ccl_sched* sched, const void* own_buf, const
     int lp = bf16_keep_precision_mode ? MI_CCL_LP_KEEP_PRECISION : MI_CCL_LP_PAIRWISE;
     return to_status(mi_ccl_comp_reduce_write_n((int)dtype.idx(), (int)reduction, srcs.data(), (int)srcs.size(),
                                                 out_bufs.data(), (int)out_bufs.size(), count, lp,
-                                                (int)ccl::global_data::env().bf16_impl_type, stream_of(sched)),
+                                                bf16_impl_for(dtype), stream_of(sched)),
                      "ccl_comp_reduce_write_n");
 }

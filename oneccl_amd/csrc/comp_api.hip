@@ -25,6 +25,7 @@ MI_DECLARE(U64Traits);
 MI_DECLARE(F32Traits);
 MI_DECLARE(F64Traits);
 MI_DECLARE(Fp16PairwiseTraits);
+MI_DECLARE(Fp16NativeTraits);
 typedef Bf16PairwiseTraits<false, false> Bf16PairScalar;
 typedef Bf16PairwiseTraits<false, true> Bf16PairAvx512f;
 typedef Bf16PairwiseTraits<true, true> Bf16PairAvx512bf;
@@ -42,6 +43,7 @@ static std::atomic<int> g_max_blocks{ 0 };
 static std::atomic<int> g_xcd_chunked{ 0 };
 static std::atomic<int> g_variant{ 0 };
 static std::atomic<long> g_phased_min_bytes{ 512L << 20 };
+static std::atomic<int> g_fp16_impl{ MI_CCL_FP16_AVX512F };
 static std::atomic<int> g_num_cus[64];
 
 // Barrier words of the phased kernel: one copy per device (each GPU holds its own instance of a
@@ -86,6 +88,7 @@ Tuning current_tuning() {
     t.num_cus = num_cus();
     t.phased_min_bytes = g_phased_min_bytes.load(std::memory_order_relaxed);
     t.sync = phase_sync();
+    t.fp16_impl = g_fp16_impl.load(std::memory_order_relaxed);
     return t;
 }
 
@@ -115,7 +118,9 @@ static hipError_t dispatch(int dtype, bool keep, int bf16_impl, const LaunchArgs
         case MI_CCL_UINT32: return launch_reduce<U32Traits>(a);
         case MI_CCL_INT64: return launch_reduce<I64Traits>(a);
         case MI_CCL_UINT64: return launch_reduce<U64Traits>(a);
-        case MI_CCL_FLOAT16: return launch_reduce<Fp16PairwiseTraits>(a);
+        case MI_CCL_FLOAT16:
+            return a.tune.fp16_impl == MI_CCL_FP16_AVX512FP16 ? launch_reduce<Fp16NativeTraits>(a)
+                                                              : launch_reduce<Fp16PairwiseTraits>(a);
         case MI_CCL_FLOAT32: return launch_reduce<F32Traits>(a);
         case MI_CCL_FLOAT64: return launch_reduce<F64Traits>(a);
         case MI_CCL_BFLOAT16:
@@ -458,6 +463,10 @@ int mi_ccl_set_param(const char* name, long value) {
         g_phased_min_bytes.store(value);
         return MI_CCL_SUCCESS;
     }
+    if (!strcmp(name, "fp16_impl") && value >= MI_CCL_FP16_F16C && value <= MI_CCL_FP16_AVX512FP16) {
+        g_fp16_impl.store((int)value);
+        return MI_CCL_SUCCESS;
+    }
     return MI_CCL_INVALID_ARGUMENTS;
 }
 
@@ -474,6 +483,8 @@ long mi_ccl_get_param(const char* name) {
         return g_variant.load();
     if (!strcmp(name, "phased_min_bytes"))
         return g_phased_min_bytes.load();
+    if (!strcmp(name, "fp16_impl"))
+        return g_fp16_impl.load();
     if (!strcmp(name, "num_cus"))
         return num_cus();
     return -1;

@@ -23,6 +23,7 @@ MI_DECLARE_FUSION(U64Traits);
 MI_DECLARE_FUSION(F32Traits);
 MI_DECLARE_FUSION(F64Traits);
 MI_DECLARE_FUSION(Fp16PairwiseTraits);
+MI_DECLARE_FUSION(Fp16NativeTraits);
 typedef Bf16PairwiseTraits<false, false> Bf16PairScalar;
 typedef Bf16PairwiseTraits<false, true> Bf16PairAvx512f;
 typedef Bf16PairwiseTraits<true, true> Bf16PairAvx512bf;
@@ -253,7 +254,10 @@ int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* ow
         case MI_CCL_UINT32: e = launch_fusion_reduce<U32Traits>(a); break;
         case MI_CCL_INT64: e = launch_fusion_reduce<I64Traits>(a); break;
         case MI_CCL_UINT64: e = launch_fusion_reduce<U64Traits>(a); break;
-        case MI_CCL_FLOAT16: e = launch_fusion_reduce<Fp16PairwiseTraits>(a); break;
+        case MI_CCL_FLOAT16:
+            e = a.tune.fp16_impl == MI_CCL_FP16_AVX512FP16 ? launch_fusion_reduce<Fp16NativeTraits>(a)
+                                                           : launch_fusion_reduce<Fp16PairwiseTraits>(a);
+            break;
         case MI_CCL_FLOAT32: e = launch_fusion_reduce<F32Traits>(a); break;
         case MI_CCL_FLOAT64: e = launch_fusion_reduce<F64Traits>(a); break;
         case MI_CCL_BFLOAT16:

@@ -42,6 +42,7 @@ struct Tuning {
     int num_cus;
     long phased_min_bytes;   // automatic choice: phased kernel when (N + 1) * bytes per buffer reaches this
     struct PhaseSync* sync;  // device-resident barrier words of the current device (may be null)
+    int fp16_impl;           // which CPU implementation's float16 results to reproduce: 2, 3 (through fp32) or 4 (native)
 };
 
 struct LaunchArgs {
@@ -194,8 +195,12 @@ struct Bf16KeepTraits {
 // float16, rounded after every pair through fp32 (ccl_fp16_reduce f16c / avx512f implementations,
 // src/comp/fp16/fp16_intrisics.hpp:95-148): VCVTPH2PS both, one fp32 op, VCVTPS2PH round-to-nearest-even,
 // fp16 subnormals kept.  min/max return `inout` on ties/NaN and quiet a NaN they return (the x86 widening
-// conversion quiets it).
-struct Fp16PairwiseTraits {
+// conversion quiets it).  NATIVE: the avx512fp16 implementation (fp16_intrisics.cpp:24-35), which works on the
+// fp16 values themselves: the same bits for sum and prod (fp32 holds the exact sum or product of two fp16 values
+// closely enough that rounding twice equals rounding once), and min/max hand back the chosen operand untouched, a
+// signalling NaN included.
+template <bool NATIVE>
+struct Fp16Traits {
     typedef uint16_t elem_t;
     typedef uint32_t acc_t;     // fp16 bits in the low half
     static constexpr int VEC = 8;
@@ -211,11 +216,14 @@ struct Fp16PairwiseTraits {
             return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)r);
         }
         uint32_t r = (OP == OP_MIN) ? ((a < b) ? (uint32_t)in : io) : ((a > b) ? (uint32_t)in : io);
+        if (NATIVE) return r;
         bool nan = (r & 0x7c00u) == 0x7c00u && (r & 0x03ffu) != 0;
         return nan ? (r | 0x0200u) : r;
     }
     static __device__ __forceinline__ elem_t finish(acc_t a) { return (elem_t)a; }
 };
+typedef Fp16Traits<false> Fp16PairwiseTraits;
+typedef Fp16Traits<true> Fp16NativeTraits;
 
 typedef PlainTraits<int8_t, uint8_t> I8Traits;
 typedef PlainTraits<uint8_t, uint8_t> U8Traits;

@@ -15,8 +15,10 @@
  *   orc_bf16_reduce (scalar)        composition of pinned converters + std::min/max truth table
  *                                   (recorded probe values of the reference library)
  *   orc_fp16_reduce (f16c/avx512f)  reference ccl_fp16_reduce_impl_256/_512 compiled in place, golden
- *   orc_fp16_reduce (avx512fp16)    PARITY UNPINNED for min/max with signalling NaNs (needs gcc >= 12 to
- *                                   build the reference path); sum/prod equal the fp32 route exactly
+ *   orc_fp16_reduce (avx512fp16)    reference ccl_fp16_reduce_impl_512FP16 compiled in place with clang (gcc 11 lacks the
+ *                                   AVX512-FP16 intrinsics): all 2^32 (in, inout) pairs of every op compared once
+ *                                   (bit-exact for min/max, NaN payloads aside for sum/prod), golden vectors made
+ *                                   from it (tests/golden/ref_vectors_avx512fp16.npz)
  *   orc_comp_reduce plain types     IEEE single op per pair / two's-complement wrap: numpy closed forms,
  *                                   min/max truth table recorded from the reference library
  *   orc_convert_*_arrays tail       recorded probe values of the reference library (tail truncation)

@@ -28,13 +28,15 @@
 
 extern "C" {
 
-/* bit 0: avx512f+bw+vl, bit 1: avx512_bf16, bit 2: f16c */
+/* bit 0: avx512f+bw+vl, bit 1: avx512_bf16, bit 2: f16c, bit 3: avx512_fp16 */
 int ref_cpu_support(void) {
     unsigned a, b, c, d;
     int r = 0;
     if (__get_cpuid_count(7, 0, &a, &b, &c, &d)) {
         if ((b & (1u << 16)) && (b & (1u << 30)) && (b & (1u << 31)))
             r |= 1;
+        if ((b & (1u << 30)) && (d & (1u << 23)))     /* as fp16_utils.hpp:62-70 */
+            r |= 8;
     }
     if (__get_cpuid_count(7, 1, &a, &b, &c, &d)) {
         if (a & (1u << 5))
@@ -96,7 +98,9 @@ REF_TARGET_BF16 int ref_fp32_store_as_bf16_16(const void* src, void* dst, int im
     return -1;
 }
 
-/* impl: 2 = f16c (8 per iteration, memcpy'd tail), 3 = avx512f (16 per iteration, masked tail) */
+/* impl: 2 = f16c (8 per iteration, memcpy'd tail), 3 = avx512f (16 per iteration, masked tail),
+ * 4 = avx512fp16 (32 per iteration in native fp16, masked tail): only in a build whose compiler knows the
+ * AVX512-FP16 intrinsics (the reference's own CCL_FP16_AVX512FP16_COMPILER switch; see oracle/Makefile) */
 int ref_fp16_reduce(const void* in, size_t count, void* inout, int op, int impl) {
     int cpu = ref_cpu_support();
     if (count >= 0x7fffffffu || op < 0 || op > 3)
@@ -113,6 +117,14 @@ int ref_fp16_reduce(const void* in, size_t count, void* inout, int op, int impl)
         ccl_fp16_reduce_impl_512(in, inout, count, f[op]);
         return 0;
     }
+#ifdef CCL_FP16_AVX512FP16_COMPILER
+    if (impl == 4 && (cpu & 8)) {
+        static const ccl_fp16_reduction_func_ptr_512FP16 f[4] = { &fp16_sum_wrap_512FP16, &fp16_prod_wrap_512FP16,
+                                                                  &fp16_min_wrap_512FP16, &fp16_max_wrap_512FP16 };
+        ccl_fp16_reduce_impl_512FP16(in, inout, count, f[op]);
+        return 0;
+    }
+#endif
     return -1;
 }
 

@@ -21,6 +21,14 @@ def golden():
 
 
 @pytest.fixture(scope="session")
+def golden_fp16_native():
+    """Outputs of the reference's avx512fp16 reduce (tests/golden/make_golden.py avx512fp16); inputs of the
+    non-grid cases are the float16 inputs of ref_vectors.npz."""
+    import numpy as np
+    return np.load(os.path.join(HERE, "golden", "ref_vectors_avx512fp16.npz"), allow_pickle=False)
+
+
+@pytest.fixture(scope="session")
 def probes():
     import json
     with open(os.path.join(HERE, "golden", "reference_probes.json")) as f:

@@ -107,5 +107,55 @@ def main():
     print("wrote", path, len(out), "arrays", os.path.getsize(path), "bytes")
 
 
+def main_avx512fp16():
+    """Second fixture, ref_vectors_avx512fp16.npz: the reference's native-fp16 reduce
+    (ccl_fp16_reduce_impl_512FP16, src/comp/fp16/fp16_intrisics.hpp:150-200 with fp16_intrisics.cpp:23-41) on the
+    float16 inputs of ref_vectors.npz, on every pair of the special values, and on every pair of 512 patterns that
+    cover each exponent with its smallest and largest mantissa, both signs, quiet and signalling NaNs.  Needs
+    oracle/_ref/libccl_comp_ref_avx512fp16.so (built by clang, which knows the AVX512-FP16 intrinsics that gcc 11
+    lacks) and a CPU with avx512_fp16."""
+    import ctypes as C
+    here = os.path.dirname(os.path.abspath(__file__))
+    so = os.path.join(os.path.dirname(os.path.dirname(here)), "oracle", "_ref", "libccl_comp_ref_avx512fp16.so")
+    if not os.path.exists(so):
+        sys.exit("needs " + so)
+    R = C.CDLL(so)
+    R.ref_fp16_reduce.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int]
+    if not (R.ref_cpu_support() & 8):
+        sys.exit("needs a CPU with avx512_fp16")
+    base = np.load(os.path.join(here, "ref_vectors.npz"))
+    out = {}
+
+    def run(a, b, op):
+        r = b.copy()
+        assert R.ref_fp16_reduce(a.ctypes.data, a.size, r.ctypes.data, op, 4) == 0
+        return r
+
+    for key in base.files:
+        if key.startswith("fp16_") and key.endswith("_in"):
+            stem = key[:-3]
+            if "specials" in stem:
+                for op in range(4):
+                    out[f"fp16_specials_{O.OP_NAMES[op]}_impl4"] = run(base[key], base[stem + "_inout"], op)
+            else:
+                out[stem + "_impl4"] = run(base[key], base[stem + "_inout"], O.OP_NAMES.index(stem.split("_")[1]))
+    pats = []
+    for sign in (0, 0x8000):
+        for e in range(32):
+            for m in (0, 1, 0x1FF, 0x200, 0x201, 0x2AA, 0x3FE, 0x3FF):
+                pats.append(sign | (e << 10) | m)
+    pats = np.array(pats, dtype=np.uint16)
+    a, b = np.repeat(pats, pats.size), np.tile(pats, pats.size)
+    out["fp16_grid_in"], out["fp16_grid_inout"] = a, b
+    for op in range(4):
+        out[f"fp16_grid_{O.OP_NAMES[op]}_impl4"] = run(a, b, op)
+    path = os.path.join(here, "ref_vectors_avx512fp16.npz")
+    np.savez_compressed(path, **out)
+    print("wrote", path, len(out), "arrays", os.path.getsize(path), "bytes")
+
+
 if __name__ == "__main__":
+    if len(sys.argv) > 1 and sys.argv[1] == "avx512fp16":
+        main_avx512fp16()
+        sys.exit(0)
     main()

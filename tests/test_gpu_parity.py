@@ -391,3 +391,44 @@ def test_randomised_calls_against_oracle(comp):
             assert (got[:out_lo] == 0).all() and (got[out_lo + count:] == 0).all(), what + ": wrote outside the destination"
         else:
             assert (got[:out_lo] == 0).all() and (got[out_lo + count:] == 0).all(), what + ": wrote outside the aliased input"
+
+
+def test_fp16_native_mode_against_reference_made_vectors(comp, golden, golden_fp16_native):
+    """fp16_impl = avx512fp16 (mi_ccl_set_param): the GPU against what the reference's native-fp16 code produced --
+    bits for min/max (a signalling NaN that is handed back stays signalling), NaNs as a class for sum/prod --
+    then the N-input and multi-destination forms against the oracle in the same mode."""
+    import torch
+    from test_oracle_pins import _fp16_native_cases
+    assert comp.get_param("fp16_impl") == 3
+    comp.set_param("fp16_impl", 4)
+    try:
+        n = 0
+        for name, op, a, b, want in _fp16_native_cases(golden, golden_fp16_native):
+            da, db = to_dev(a), to_dev(b)
+            comp.comp_reduce(O.FLOAT16, op, da, a.size, db)
+            torch.cuda.synchronize()
+            got = to_host(db, np.uint16)
+            if op in (O.MIN, O.MAX):
+                assert (got == want).all(), (name, np.flatnonzero(got != want)[:8])
+            else:
+                assert_same(got, want, O.FLOAT16, name)
+            n += 1
+        assert n == 96
+        rng = np.random.default_rng(123)
+        for op in (O.MIN, O.MAX, O.SUM):
+            srcs = make_inputs(rng, O.FLOAT16, 70001, op, 5, "bits")
+            d = [to_dev(s) for s in srcs]
+            outs = [torch.empty_like(d[0]) for _ in range(3)]
+            comp.comp_reduce_write_n(O.FLOAT16, op, d, outs, 70001)
+            torch.cuda.synchronize()
+            want = O.reduce_n(srcs, O.FLOAT16, op, fp16_impl=O.FP16_AVX512FP16)
+            for o in outs:
+                got = to_host(o, np.uint16)
+                if op == O.SUM:
+                    assert_same(got, want, O.FLOAT16, "native fp16 sum")
+                else:
+                    assert (got == want).all()
+    finally:
+        comp.set_param("fp16_impl", 3)
+    with pytest.raises(comp.CclError):
+        comp.set_param("fp16_impl", 1)

@@ -463,3 +463,62 @@ def test_reduce_write_n_is_reduce_n_stored_m_times():
     srcs = [(np.arange(cnt) % 5 + r).astype(np.float32) for r in range(n)]
     for o in O.reduce_write_n(srcs, 8, O.FLOAT32, O.SUM):
         assert (o == n * (n - 1) / 2 + n * (np.arange(cnt) % 5)).all()
+
+
+def _fp16_native_cases(golden, native):
+    """(name, op, in, inout, want) for every case of the avx512fp16 fixture"""
+    for key in native.files:
+        if not key.endswith("_impl4"):
+            continue
+        stem = key[:-len("_impl4")]
+        if stem.startswith("fp16_specials_") or stem.startswith("fp16_grid_"):
+            fam = "specials" if "specials" in stem else "grid"
+            op = O.OP_NAMES.index(stem.split("_")[2])
+            src = golden if fam == "specials" else native
+            yield stem, op, src[f"fp16_{fam}_in"], src[f"fp16_{fam}_inout"], native[key]
+        else:
+            op = O.OP_NAMES.index(stem.split("_")[1])
+            yield stem, op, golden[stem + "_in"], golden[stem + "_inout"], native[key]
+
+
+def test_fp16_avx512fp16_against_reference_made_vectors(golden, golden_fp16_native):
+    """The native-fp16 implementation (fp16_intrisics.cpp:23-41): min/max return one operand untouched, so bits
+    are compared, signalling NaNs included; sum/prod compare NaNs as a class."""
+    n = 0
+    for name, op, a, b, want in _fp16_native_cases(golden, golden_fp16_native):
+        got = O.comp_reduce(a, b, O.FLOAT16, op, fp16_impl=O.FP16_AVX512FP16)
+        if op in (O.MIN, O.MAX):
+            assert (got == want).all(), (name, np.flatnonzero(got != want)[:8])
+        else:
+            assert O.same_bits_or_both_nan(got, want, O.FLOAT16).all(), name
+        n += 1
+    assert n == 4 * 11 * 2 + 4 + 4
+    # and the point of the mode: a signalling NaN handed back by min/max stays signalling, the other modes quiet it
+    a = np.array([0x7C01], np.uint16)
+    b = np.array([0x3C00], np.uint16)
+    assert O.comp_reduce(b, a, O.FLOAT16, O.MIN, fp16_impl=O.FP16_AVX512FP16)[0] == 0x7C01
+    assert O.comp_reduce(b, a, O.FLOAT16, O.MIN, fp16_impl=O.FP16_AVX512F)[0] == 0x7E01
+
+
+def test_fp16_avx512fp16_against_reference_library_when_built():
+    """Direct comparison with the reference's code compiled in place (oracle/_ref, clang build) on a million random
+    pairs per op; skipped where that library or the CPU feature is absent (the fixture test above still runs)."""
+    import ctypes as C
+    so = os.path.join(os.path.dirname(O.REF_SO), "libccl_comp_ref_avx512fp16.so")
+    if not os.path.exists(so):
+        pytest.skip("oracle/_ref/libccl_comp_ref_avx512fp16.so not built")
+    R = C.CDLL(so)
+    R.ref_fp16_reduce.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int]
+    if not (R.ref_cpu_support() & 8):
+        pytest.skip("CPU without avx512_fp16")
+    rng = np.random.default_rng(99)
+    for op in range(4):
+        a = rng.integers(0, 65536, 1_000_003, dtype=np.uint16)
+        b = rng.integers(0, 65536, 1_000_003, dtype=np.uint16)
+        want = b.copy()
+        assert R.ref_fp16_reduce(a.ctypes.data, a.size, want.ctypes.data, op, 4) == 0
+        got = O.comp_reduce(a, b, O.FLOAT16, op, fp16_impl=O.FP16_AVX512FP16)
+        if op in (O.MIN, O.MAX):
+            assert (got == want).all()
+        else:
+            assert O.same_bits_or_both_nan(got, want, O.FLOAT16).all()
