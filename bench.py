@@ -8,7 +8,8 @@ HBM.  Default workload: the Llama-3-8B-sized gradient share, 8 input buffers of 
 (N(0, 1e-3) cast to bf16), fp32 accumulation in input order, one round-to-nearest-even narrowing
 (ccl_comp_batch_reduce keep-precision semantics under CCL_BF16=avx512bf).  Prints ONE JSON line.
 
-Algorithmic bytes of a launch = (N + 1) x count x sizeof(element): N reads and one write.
+Algorithmic bytes of a launch = (N + M) x count x sizeof(element): N reads and M writes (M = 1 except for the
+write-side workloads).
 """
 import argparse
 import json
@@ -34,6 +35,11 @@ WORKLOADS = {
                     desc="8-input bf16 sum, 33,554,432 elements per buffer (64 MiB), rotating over 6 buffer sets"),
     "c1_fp32": dict(dtype="float32", n=2, count=16_777_216, keep=False, sets=8, in_place=True,
                     desc="2-input in-place fp32 sum, 16,777,216 elements per buffer (64 MiB), rotating over 8 buffer sets"),
+    # the write side: one reduce stored to m buffers (allreduce_kernel shape), and one buffer copied to 7 (all-gather write)
+    "rw_8to8_bf16": dict(dtype="bfloat16", n=8, m=8, count=1 << 29, keep=True, sets=1,
+                         desc="8-input bf16 sum stored to 8 buffers, 536,870,912 elements (1 GiB) per buffer"),
+    "write_1to7_bf16": dict(dtype="bfloat16", n=1, m=7, count=1 << 29, keep=False, sets=1,
+                            desc="one 1 GiB buffer copied to 7 buffers (write_monolithic_kernel_7 shape)"),
     # calibration for the rocprofv3 FETCH_SIZE / WRITE_SIZE counters: a plain copy of known size
     "copy_ref": dict(dtype="bfloat16", n=1, count=1_003_782_144, keep=False, sets=1, copy=True,
                      desc="mi_ccl_comp_copy of 2,007,564,288 bytes (counter calibration: reads and writes that many bytes)"),
@@ -137,14 +143,19 @@ def main():
     lp = comp.LP_KEEP_PRECISION if w["keep"] else comp.LP_PAIRWISE
     n, count = w["n"], w["count"]
     sets = [make_buffers(torch, w, 1234 + i) for i in range(w["sets"])]
+    m = w.get("m", 1)
     outs = [s[0] if w.get("in_place") else torch.empty_like(s[0]) for s in sets]
-    algo_bytes = (n + 1) * count * esz
+    extra_outs = [[torch.empty_like(s[0]) for _ in range(m - 1)] for s in sets]
+    algo_bytes = (n + m) * count * esz
     stream = torch.cuda.current_stream()
 
     def step(i):
         s = sets[i % len(sets)]
         if w.get("copy"):
             comp.comp_copy(s[0], outs[i % len(sets)], count * esz, use_nontemporal=True, stream=stream)
+        elif m > 1:
+            comp.comp_reduce_write_n(dt, comp.SUM, s, [outs[i % len(sets)]] + extra_outs[i % len(sets)], count,
+                                     lp_mode=lp, stream=stream)
         else:
             comp.comp_reduce_n(dt, comp.SUM, s, outs[i % len(sets)], count, lp_mode=lp, stream=stream)
 
@@ -161,6 +172,9 @@ def main():
         same = (got.view(np.uint8) == want.view(np.uint8)).all()
         if not same:
             sys.exit("GPU result differs from the oracle on the CPU-baseline sample")
+        for o in extra_outs[0]:
+            if not torch.equal(o.view(torch.int16), outs[0].view(torch.int16)):
+                sys.exit("the destinations of one launch differ")
         if w.get("in_place"):
             for b, c in zip(sets[0], snapshot):
                 b.copy_(c)
@@ -197,7 +211,7 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16" if dt == comp.BFLOAT16 else "f32",
         "data": "synthetic",
-        "config": {"workload": args.workload, "description": w["desc"], "inputs": n, "elements_per_buffer": count,
+        "config": {"workload": args.workload, "description": w["desc"], "inputs": n, "outputs": m, "elements_per_buffer": count,
                    "bytes_per_buffer": count * esz, "algorithmic_bytes_per_step": algo_bytes,
                    "lp_mode": "fp32 accumulate, RNE once" if w["keep"] else "native",
                    "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),

@@ -16,6 +16,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "ccl_sched_entry.hpp"
@@ -71,15 +72,15 @@ __global__ void __launch_bounds__(kBlock) reduce_elem_kernel(src_table<T> src, i
 }
 
 inline int cu_count() {
-    static int per_device[64] = {};
+    static std::atomic<int> per_device[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (!per_device[dev]) {
-        int n = 0;
+    int n = per_device[dev].load(std::memory_order_relaxed);
+    if (!n) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        per_device[dev] = n;
+        per_device[dev].store(n, std::memory_order_relaxed);
     }
-    return per_device[dev];
+    return n;
 }
 
 }  // namespace ccl_custom

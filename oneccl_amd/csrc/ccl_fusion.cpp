@@ -177,10 +177,24 @@ void ccl_fusion_manager::build_and_start() {
         if (!buf)
             fusion_fail("fusion buffer allocation failed");
     }
-    backend->pack(sends, counts, dtype, buf, first->stream);
-    allreduce(buf, sum_count, dtype, first->reduction, first->comm, first->stream);
-    backend->unpack(buf, recvs, counts, dtype, first->stream);
-    std::shared_ptr<void> token = backend->record(first->stream);
+    std::shared_ptr<void> token;
+    try {
+        backend->pack(sends, counts, dtype, buf, first->stream);
+        allreduce(buf, sum_count, dtype, first->reduction, first->comm, first->stream);
+        backend->unpack(buf, recvs, counts, dtype, first->stream);
+        token = backend->record(first->stream);
+    }
+    catch (...) {
+        // the gathered requests stay queued (the next flush tries them again); the buffer may still be in use by
+        // whatever was enqueued before the failure, so it is tracked until the stream has drained
+        try {
+            tracked.push_back(launched_t{ buf, backend->record(first->stream) });
+        }
+        catch (...) {
+            free_buffers.push_back(buf);
+        }
+        throw;
+    }
     for (ccl_fusion_request* r : exec_queue) {
         r->done_token = token;
         r->urgent.store(false, std::memory_order_relaxed);

@@ -35,7 +35,8 @@ struct ccl_fusion_request {
     void* stream = nullptr;                     // ... and one stream
     std::atomic<bool> urgent{ false };          // set by a waiter: flush the queue this request sits in
 
-    bool is_completed();                        // true once the fused operation that carried it has finished
+    // true once the fused operation that carried it has finished; call it from one thread at a time per request
+    bool is_completed();
 
 private:
     friend class ccl_fusion_manager;

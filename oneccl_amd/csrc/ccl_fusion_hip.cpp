@@ -9,6 +9,7 @@ struct ccl_fusion_hip_backend::impl {
     // (src/fusion/fusion.cpp:206-237)
     std::map<std::pair<int, std::vector<size_t>>, mi_ccl_fusion_plan*> plans;
     std::mutex lock;
+    static constexpr size_t kMaxPlans = 256;
 
     mi_ccl_fusion_plan* plan_for(const std::vector<size_t>& counts, const ccl_datatype& dtype) {
         std::lock_guard<std::mutex> g(lock);
@@ -16,6 +17,12 @@ struct ccl_fusion_hip_backend::impl {
         auto it = plans.find(key);
         if (it != plans.end())
             return it->second;
+        // a workload whose tensor sets never repeat must not grow the cache without bound: start over when it is
+        // full (destroying a plan frees device memory, which waits for the kernels that still read it)
+        if (plans.size() >= kMaxPlans) {
+            for (auto& kv : plans) mi_ccl_fusion_plan_destroy(kv.second);
+            plans.clear();
+        }
         mi_ccl_fusion_plan* plan = nullptr;
         int rc = mi_ccl_fusion_plan_create(counts.data(), counts.size(), (int)dtype.idx(), /*align=*/1, &plan);
         if (rc != MI_CCL_SUCCESS)
