@@ -278,7 +278,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                 if (tid + kPhaseBlock < nvec) st_stream(d + tid + kPhaseBlock, stage[(2 * k + 1) * kPhaseBlock + tid]);
             }
         }
-        phase_barrier(ps, ++gen, give_up);
+        if (p0 + per_phase < nitems) phase_barrier(ps, ++gen, give_up);
     }
 }
 

@@ -457,8 +457,8 @@ struct PhaseSync {
 #define MI_ALOAD(p) __hip_atomic_load((p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 #define MI_AADD(p, x) __hip_atomic_fetch_add((p), (x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 
-// Every block calls this the same number of times per launch, so the counters stay multiples of their
-// group sizes from launch to launch.  gen is the generation this block waits for.
+// Every block calls this the same number of times per launch (twice per phase, except after the last phase's
+// writes), so the counters stay multiples of their group sizes from launch to launch.  gen is the generation this block waits for.
 __device__ __forceinline__ void phase_barrier(PhaseSync* ps, unsigned gen, bool& give_up) {
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -579,7 +579,8 @@ reduce_phased_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, u
             const uint64_t i = p0 + (uint64_t)(R + u) * gthreads + gtid;
             if (i < nvec) st_stream(d + i, stage[u * kPhaseBlock + threadIdx.x]);
         }
-        phase_barrier(ps, ++gen, give_up);      // all writes of this phase are issued
+        // all writes of this phase are issued before the next phase reads; nothing follows the last phase
+        if (p0 + per_phase < nvec) phase_barrier(ps, ++gen, give_up);
     }
     if (blockIdx.x == 0 && (head | tail)) reduce_edges<TR, OP>(src, N, dst, head, nvec, tail);
 }
@@ -733,7 +734,7 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
                 if (i < nvec) st_stream(d + i, stage[u * kPhaseBlock + threadIdx.x]);
             }
         }
-        phase_barrier(ps, ++gen, give_up);
+        if (p0 + per_phase < nvec) phase_barrier(ps, ++gen, give_up);
     }
     if (blockIdx.x == 0 && (head | tail)) reduce_multi_edges<TR, OP>(src, n, dst, m, head, nvec, tail);
 }
