@@ -42,7 +42,7 @@ static std::atomic<int> g_waves_per_cu{ 8 };
 static std::atomic<int> g_max_blocks{ 0 };
 static std::atomic<int> g_xcd_chunked{ 0 };
 static std::atomic<int> g_variant{ 0 };
-static std::atomic<long> g_phased_min_bytes{ 512L << 20 };
+static std::atomic<long> g_phased_min_bytes{ 320L << 20 };
 static std::atomic<int> g_fp16_impl{ MI_CCL_FP16_AVX512F };
 static std::atomic<int> g_num_cus[64];
 

@@ -7,6 +7,11 @@ template <>
 struct PhaseRegs<Bf16PairwiseTraits<true, true>> {
     static constexpr int fit(int n) { return n <= 4 ? 20 : 12; }
 };
+// ... and with 7 or 8 inputs the streaming kernel is bound by them, not by loads in flight
+template <>
+struct StreamUnroll<Bf16PairwiseTraits<true, true>> {
+    static constexpr int get(int n) { return n <= 6 ? 4 : 2; }
+};
 template hipError_t launch_reduce<Bf16PairwiseTraits<true, true>>(const LaunchArgs&);
 template hipError_t launch_fusion_reduce<Bf16PairwiseTraits<true, true>>(const FusionLaunchArgs&);
 }  // namespace mi

@@ -782,6 +782,14 @@ struct HasUnrollVariants {
     static constexpr bool value = false;
 };
 
+// Vectors per lane per tile of the streaming kernel (N x this many 128-bit loads are in flight per lane).  Four
+// measures 3-7 % above two for every type at 5-8 inputs; a traits class with heavy per-element arithmetic
+// specialises this before its kernels are instantiated.
+template <class TR>
+struct StreamUnroll {
+    static constexpr int get(int) { return 4; }
+};
+
 template <class TR, int OP, int N>
 inline hipError_t launch_phased(const LaunchArgs& a, uint32_t head, uint64_t nvec, uint32_t tail) {
     SrcFixed<N> s;
@@ -795,8 +803,7 @@ inline hipError_t launch_phased(const LaunchArgs& a, uint32_t head, uint64_t nve
 
 template <class TR, int OP, int N>
 inline hipError_t launch_fixed_unroll(const LaunchArgs& a, uint32_t head, uint64_t nvec, uint32_t tail) {
-    // loads in flight per lane = N * UNROLL
-    constexpr int kDefault = (N <= 4) ? 4 : 2;
+    constexpr int kDefault = StreamUnroll<TR>::get(N);
     {
         const bool can = a.tune.sync != nullptr && a.tune.num_cus >= kPhaseGroups;
         // with two or three inputs the streaming kernel holds up longer (less to interleave per write)
