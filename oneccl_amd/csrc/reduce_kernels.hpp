@@ -847,7 +847,9 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
     const uint32_t tail = (uint32_t)(a.count - head - nvec * VEC);
     const bool can = a.tune.sync != nullptr && a.tune.num_cus >= kPhaseGroups;
     const uint64_t traffic = (uint64_t)(a.n + a.m) * nvec * 16u;
-    if (can && (a.tune.variant == 8 || (a.tune.variant == 0 && traffic >= (uint64_t)a.tune.phased_min_bytes))) {
+    // LDS staging only (no register-staged vectors): the phased form pays off later than in the one-output kernel,
+    // from about 512 MB of traffic with the default setting
+    if (can && (a.tune.variant == 8 || (a.tune.variant == 0 && traffic >= (uint64_t)a.tune.phased_min_bytes / 5 * 8))) {
         int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
                            a.m, (uint32_t)head, nvec, tail, a.tune.sync);
