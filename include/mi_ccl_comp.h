@@ -174,8 +174,8 @@ int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* ow
 /* ---- launch tuning ------------------------------------------------------------------------------- */
 
 /* Launch-shape knobs, the counterpart of CCL_KERNEL_GROUP_SIZE / CCL_KERNEL_MEM_ALIGN
- * (src/common/env/env.cpp:251-253).  Names: "waves_per_cu" (resident blocks per CU the grid is sized
- * for), "max_blocks" (cap on the grid; 0 = no cap), "xcd_chunked" (0/1: give each of the 8 XCDs one
+ * (src/common/env/env.cpp:251-253).  Names: "waves_per_cu" (blocks per CU the streaming kernels' grid is capped
+ * at; default 256, i.e. one tile per block up to 65,536 blocks), "max_blocks" (cap on the grid; 0 = no cap), "xcd_chunked" (0/1: give each of the 8 XCDs one
  * contiguous share of the buffer), "variant" (kernel variant selector, 0 = default), "phased_min_bytes",
  * and "fp16_impl" (enum mi_ccl_fp16_impl above).
  * Returns invalid_arguments for an unknown name or out-of-range value. */

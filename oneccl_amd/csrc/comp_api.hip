@@ -38,7 +38,7 @@ MI_DECLARE(Bf16KeepTraits<true>);
 // ---------------------------------------------------------------------------------------------------
 // tuning state and device facts
 
-static std::atomic<int> g_waves_per_cu{ 8 };
+static std::atomic<int> g_waves_per_cu{ 256 };
 static std::atomic<int> g_max_blocks{ 0 };
 static std::atomic<int> g_xcd_chunked{ 0 };
 static std::atomic<int> g_variant{ 0 };
@@ -443,7 +443,7 @@ int mi_ccl_convert_bf16_to_fp32_arrays(const void* bf16_buf, void* fp32_buf, siz
 int mi_ccl_set_param(const char* name, long value) {
     if (!name)
         return MI_CCL_INVALID_ARGUMENTS;
-    if (!strcmp(name, "waves_per_cu") && value >= 1 && value <= 64) {
+    if (!strcmp(name, "waves_per_cu") && value >= 1 && value <= 65536) {
         g_waves_per_cu.store((int)value);
         return MI_CCL_SUCCESS;
     }

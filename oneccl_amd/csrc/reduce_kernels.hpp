@@ -35,7 +35,7 @@ struct DstTable {               // by-value kernel argument
 };
 
 struct Tuning {
-    int waves_per_cu;   // resident 256-thread blocks per CU the grid is sized for
+    int waves_per_cu;   // 256-thread blocks per CU the grid is capped at (a block loops over tiles beyond that)
     int max_blocks;     // 0 = no cap
     int xcd_chunked;    // 1: each XCD streams one contiguous eighth of the buffer
     int variant;        // 0 = automatic; 1, 2, 4 = streaming kernel with that unroll depth; 8 = phased kernel
