@@ -94,7 +94,7 @@ __device__ __forceinline__ void copy_span(const unsigned char* src, unsigned cha
     }
 }
 
-// out_t[i] = own_t[i] OP peer_0[off_t + i] OP ... : one pass, same arithmetic as reduce_vec_rt_kernel
+// out_t[i] = own_t[i] OP peer_0[off_t + i] OP ... : one pass, same arithmetic as reduce_multi_kernel
 template <class TR, int OP>
 __global__ void __launch_bounds__(kBlock)
 fusion_reduce_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers, const uint64_t* off,

@@ -585,45 +585,6 @@ reduce_phased_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, u
     if (blockIdx.x == 0 && (head | tail)) reduce_edges<TR, OP>(src, N, dst, head, nvec, tail);
 }
 
-// Run-time N (9..64): inputs are folded in one after the other, UNROLL vectors of each in flight.
-template <class TR, int OP, int UNROLL>
-__global__ void __launch_bounds__(kBlock)
-reduce_vec_rt_kernel(SrcTable src, int n, void* dst, uint32_t head, uint64_t nvec, uint32_t tail,
-                     int xcd_chunked) {
-    typedef typename TR::elem_t E;
-    constexpr uint64_t kTile = (uint64_t)kBlock * UNROLL;
-    u32x4* d = (u32x4*)((E*)dst + head);
-    const uint64_t ntiles = (nvec + kTile - 1) / kTile;
-    for (TileIter it(ntiles, xcd_chunked); it.tile < it.end; it.tile += it.stride) {
-        const uint64_t base = it.tile * kTile + threadIdx.x;
-        Accs<TR> a[UNROLL];
-        const u32x4* s0 = (const u32x4*)((const E*)src.p[0] + head);
-#pragma unroll
-        for (int u = 0; u < UNROLL; u++) {
-            const uint64_t i = base + (uint64_t)u * kBlock;
-            u32x4 x = (i < nvec) ? ld_stream(s0 + i) : u32x4{ 0, 0, 0, 0 };
-            a[u] = vec_init<TR>(x);
-        }
-        for (int j = 1; j < n; j++) {
-            const u32x4* sj = (const u32x4*)((const E*)src.p[j] + head);
-            u32x4 x[UNROLL];
-#pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
-                const uint64_t i = base + (uint64_t)u * kBlock;
-                x[u] = (i < nvec) ? ld_stream(sj + i) : u32x4{ 0, 0, 0, 0 };
-            }
-#pragma unroll
-            for (int u = 0; u < UNROLL; u++) vec_step<TR, OP>(x[u], a[u]);
-        }
-#pragma unroll
-        for (int u = 0; u < UNROLL; u++) {
-            const uint64_t i = base + (uint64_t)u * kBlock;
-            if (i < nvec) st_stream(d + i, vec_finish<TR>(a[u]));
-        }
-    }
-    if (blockIdx.x == 0 && (head | tail)) reduce_edges<TR, OP>(src, n, dst, head, nvec, tail);
-}
-
 // One element per lane, any alignment of the buffers relative to each other.
 template <class TR, int OP>
 __global__ void __launch_bounds__(kBlock)
@@ -638,7 +599,7 @@ reduce_elem_kernel(SrcTable src, int n, void* dst, uint64_t count) {
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Several destinations: the reduced vector is stored to each of m buffers (the reference's allreduce_kernel stores
+// Run-time counts of inputs (up to 64) and destinations (up to 16): the reduced vector is stored to each of m buffers (the reference's allreduce_kernel stores
 // to the own and to the peer's output, kernels.cl:190-217; with one input this is write_monolithic_kernel_N,
 // kernels.cl:423-560).  Inputs and outputs are run-time counts.  A lane reads its element from every input before
 // it stores it anywhere, so a destination may be one of the inputs.
@@ -830,11 +791,11 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
     SrcTable s;
     DstTable d;
     for (int j = 0; j < a.n; j++) s.p[j] = a.srcs[j];
-    for (int k = 0; k < a.m; k++) d.p[k] = a.dsts[k];
-    const uintptr_t mis = (uintptr_t)a.dsts[0] & 15u;
+    for (int k = 0; k < a.m; k++) d.p[k] = a.dsts ? a.dsts[k] : a.dst;
+    const uintptr_t mis = (uintptr_t)d.p[0] & 15u;
     bool same = true;
     for (int j = 0; j < a.n; j++) same = same && (((uintptr_t)a.srcs[j] & 15u) == mis);
-    for (int k = 0; k < a.m; k++) same = same && (((uintptr_t)a.dsts[k] & 15u) == mis);
+    for (int k = 0; k < a.m; k++) same = same && (((uintptr_t)d.p[k] & 15u) == mis);
     if (!same || (mis % sizeof(E)) != 0) {
         int grid = grid_for((a.count + kBlock - 1) / kBlock, a.tune);
         hipLaunchKernelGGL((reduce_multi_elem_kernel<TR, OP>), dim3(grid), dim3(kBlock), 0, a.stream, s, a.n, d, a.m,
@@ -867,7 +828,7 @@ template <class TR, int OP>
 inline hipError_t launch_op(const LaunchArgs& a) {
     typedef typename TR::elem_t E;
     constexpr uint32_t VEC = TR::VEC;
-    if (a.m > 1) return launch_multi_op<TR, OP>(a);
+    if (a.m > 1 || a.n > kMaxFixedN) return launch_multi_op<TR, OP>(a);     // run-time counts of inputs and outputs
     // common misalignment of all buffers to 16 bytes, in elements; mixed misalignment -> element kernel
     const uintptr_t mis = (uintptr_t)a.dst & 15u;
     bool same = true;
@@ -894,16 +855,7 @@ inline hipError_t launch_op(const LaunchArgs& a) {
         case 6: return launch_fixed_unroll<TR, OP, 6>(a, (uint32_t)head, nvec, tail);
         case 7: return launch_fixed_unroll<TR, OP, 7>(a, (uint32_t)head, nvec, tail);
         case 8: return launch_fixed_unroll<TR, OP, 8>(a, (uint32_t)head, nvec, tail);
-        default: {
-            SrcTable s;
-            for (int j = 0; j < a.n; j++) s.p[j] = a.srcs[j];
-            constexpr int UNROLL = 4;
-            const uint64_t tile = (uint64_t)kBlock * UNROLL;
-            int grid = grid_for((nvec + tile - 1) / tile, a.tune);
-            hipLaunchKernelGGL((reduce_vec_rt_kernel<TR, OP, UNROLL>), dim3(grid), dim3(kBlock), 0, a.stream, s,
-                               a.n, a.dst, (uint32_t)head, nvec, tail, a.tune.xcd_chunked);
-            return hipGetLastError();
-        }
+        default: return hipErrorInvalidValue;
     }
 }
 
