@@ -76,3 +76,46 @@ def test_two_phased_reduces_overlapping_on_two_streams(comp):
     comp.comp_reduce_n(comp.FLOAT32, comp.SUM, da, oa, count)
     torch.cuda.synchronize()
     assert (to_host(oa, np.float32).view(np.uint32) == want_a.view(np.uint32)).all()
+
+
+@pytest.mark.parametrize("variant", [0, 8])
+def test_worker_threads_on_disjoint_partitions(comp, variant):
+    """What CCL_WORKER_COUNT = W does (parallelizer.cpp:230-241,374-379): W host threads, each with a stream of its
+    own, reduce disjoint count/W partitions of the same buffers at the same time through the C ABI.  The result is
+    the one-call result, bit for bit; variant 8 makes every partition a phased launch, so the launches share the
+    barrier words while they overlap."""
+    import threading
+    import torch
+    rng = np.random.default_rng(31 + variant)
+    count, n, W = 8_000_011, 4, 4
+    srcs = [O.bf16_from_f32(rng.standard_normal(count).astype(np.float32)) for _ in range(n)]
+    want = O.reduce_n(srcs, O.BFLOAT16, O.SUM, keep=1, threads=8)
+    d = [to_dev(s) for s in srcs]
+    out = torch.zeros_like(d[0])
+    streams = [torch.cuda.Stream() for _ in range(W)]
+    part = count // W
+    errors = []
+
+    def worker(w):
+        try:
+            lo, hi = part * w, (count if w == W - 1 else part * (w + 1))     # the last takes the remainder
+            for rep in range(5):
+                comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, [t[lo:hi] for t in d], out[lo:hi], hi - lo,
+                                   lp_mode=comp.LP_KEEP_PRECISION, stream=streams[w])
+            streams[w].synchronize()
+        except Exception as e:      # noqa: BLE001 - reported by the main thread
+            errors.append(e)
+
+    torch.cuda.synchronize()
+    comp.set_param("variant", variant)
+    try:
+        threads = [threading.Thread(target=worker, args=(w,)) for w in range(W)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+    finally:
+        comp.set_param("variant", 0)
+    torch.cuda.synchronize()
+    assert not errors, errors
+    assert (to_host(out, np.uint16) == want).all()
