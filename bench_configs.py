@@ -7,7 +7,9 @@
   C4  fusion: 256 bf16 tensors, counts log-uniform [2,048, 2,097,152], 256-byte aligned offsets, 8-input sum against
       7 peer fusion buffers: pack + reduce + unpack, and the fused single pass
 
-    python bench_configs.py [--out results/configs.json] [--skip c3]
+  types  every datatype x op at 512 MiB per buffer, 8 and 4 inputs
+
+    python bench_configs.py [--out results/configs.json] [--skip c3,types]
 
 Writes a JSON file and prints a markdown table.  Bytes are algorithmic: (N + 1) x chunk for a reduce, 2 x payload
 for pack and unpack.  Buffers of 64 MiB rotate over several sets so that the 256 MB Infinity Cache cannot hold them.
@@ -91,6 +93,31 @@ def main():
                 steps = 200 if size <= (1 << 22) else 30
                 us = timed(torch, lambda i: comp.comp_reduce_n(dt, op, ss[i % nsets], oo[i % nsets], cnt), steps, 10)
                 add(f"C3 {label}, 4 inputs, {size >> 10} KiB per buffer", us, 5 * size, f"{nsets} set(s)")
+                del ss, oo
+    # ---- every datatype x op at 512 MiB per buffer, 8 and 4 inputs: is any of them bound by arithmetic?
+    if "types" not in args.skip:
+        size = 512 << 20
+        tcases = [("int8", comp.INT8, torch.int8, None), ("int16", comp.INT16, torch.int16, None),
+                  ("int32", comp.INT32, torch.int32, None), ("int64", comp.INT64, torch.int64, None),
+                  ("fp16", comp.FLOAT16, torch.float16, None), ("fp32", comp.FLOAT32, torch.float32, None),
+                  ("fp64", comp.FLOAT64, torch.float64, None),
+                  ("bf16 pairwise", comp.BFLOAT16, torch.bfloat16, comp.LP_PAIRWISE),
+                  ("bf16 fp32-acc", comp.BFLOAT16, torch.bfloat16, comp.LP_KEEP_PRECISION)]
+        for nin in (8, 4):
+            for label, dt, tdt, lp in tcases:
+                cnt = size // torch.empty(0, dtype=tdt).element_size()
+                if tdt.is_floating_point:
+                    ss = [torch.empty(cnt, dtype=tdt, device="cuda").uniform_(0.9, 1.1) for _ in range(nin)]
+                else:
+                    ss = [torch.randint(-100, 100, (cnt,), dtype=tdt, device="cuda") for _ in range(nin)]
+                oo = torch.empty_like(ss[0])
+                cells = []
+                for op, opn in ((comp.SUM, "sum"), (comp.PROD, "prod"), (comp.MIN, "min"), (comp.MAX, "max")):
+                    us = timed(torch, lambda i: comp.comp_reduce_n(dt, op, ss, oo, cnt, lp_mode=lp or comp.LP_PAIRWISE), 10, 3)
+                    gbs = (nin + 1) * size / us / 1e3
+                    res[f"types {label} {opn} n={nin}"] = dict(us=round(us, 2), GBps=round(gbs, 1), bytes=(nin + 1) * size)
+                    cells.append(f"{opn} {gbs:,.0f}")
+                rows.append(f"| {label}, {nin} inputs, 512 MiB per buffer | {(nin + 1) * size:,} | | {' / '.join(cells)} | | GB/s per op |")
                 del ss, oo
     # ---- C4
     rng = np.random.default_rng(4)

@@ -210,15 +210,18 @@ struct Fp16Traits {
     }
     template <int OP>
     static __device__ __forceinline__ acc_t step(elem_t in, acc_t io) {
-        float a = widen(in), b = widen(io);
         if (OP == OP_SUM || OP == OP_PROD) {
+            float a = widen(in), b = widen(io);
             float r = (OP == OP_SUM) ? (b + a) : (b * a);
             return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)r);
         }
-        uint32_t r = (OP == OP_MIN) ? ((a < b) ? (uint32_t)in : io) : ((a > b) ? (uint32_t)in : io);
+        // ordering and NaN-ness of two fp16 values are the same before and after widening: compare them as they are
+        const _Float16 a = __builtin_bit_cast(_Float16, in), b = __builtin_bit_cast(_Float16, (uint16_t)io);
+        const bool take_in = (OP == OP_MIN) ? (a < b) : (a > b);
+        const uint32_t r = take_in ? (uint32_t)in : io;
         if (NATIVE) return r;
-        bool nan = (r & 0x7c00u) == 0x7c00u && (r & 0x03ffu) != 0;
-        return nan ? (r | 0x0200u) : r;
+        const _Float16 rf = take_in ? a : b;
+        return (rf != rf) ? (r | 0x0200u) : r;
     }
     static __device__ __forceinline__ elem_t finish(acc_t a) { return (elem_t)a; }
 };
