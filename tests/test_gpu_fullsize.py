@@ -78,3 +78,41 @@ def test_c5_fp32_4x4GiB_every_element(comp):
     # one IEEE add per pair in input order: same as torch's fp32 adds chained left to right
     ref = ((bufs[0] + bufs[1]) + bufs[2]) + bufs[3]
     assert torch.equal(ref.view(torch.int32), out.view(torch.int32))
+
+
+@pytest.mark.parametrize("variant", [0, 2])
+def test_more_than_2_pow_32_elements(comp, variant):
+    """Counts beyond 32 bits (the reference's vector loops stop at 2^31, its scalar loops do not): int8 sum and max
+    over 2^32 + 4,099 elements with buffers that start 3 bytes off a 16-byte boundary, in place, through the phased
+    (variant 0 at this size) and the streaming kernel; then the same buffers through the copy and the two-destination
+    entry points.  Checked against torch's own wrapping int8 arithmetic over every element."""
+    import torch
+    count = (1 << 32) + 4099
+    g = torch.Generator(device="cuda")
+    g.manual_seed(17)
+    big = [torch.randint(-128, 128, (count + 3,), dtype=torch.int8, device="cuda", generator=g) for _ in range(2)]
+    a, b = big[0][3:], big[1][3:]
+    head_before = big[0][:3].clone()
+    want_sum = a + b                     # int8 addition wraps in torch as in the reference
+    want_max = torch.maximum(a, b)
+    comp.set_param("variant", variant)
+    try:
+        out = torch.empty(count + 3, dtype=torch.int8, device="cuda")[3:]
+        comp.comp_reduce_n(comp.INT8, comp.MAX, [a, b], out, count)
+        torch.cuda.synchronize()
+        assert torch.equal(out, want_max)
+        del want_max
+        o1 = torch.zeros(count + 3, dtype=torch.int8, device="cuda")
+        comp.comp_reduce_write_n(comp.INT8, comp.SUM, [a, b], [out, o1[3:]], count)
+        torch.cuda.synchronize()
+        assert torch.equal(out, want_sum) and torch.equal(o1[3:], want_sum) and int(o1[:3].count_nonzero()) == 0
+        del o1
+        comp.comp_copy(a, out, count, use_nontemporal=True)
+        torch.cuda.synchronize()
+        assert torch.equal(out, a)
+        comp.comp_reduce(comp.INT8, comp.SUM, b, count, a)      # in place: a += b
+        torch.cuda.synchronize()
+        assert torch.equal(a, want_sum)
+        assert torch.equal(big[0][:3], head_before)             # the bytes in front of the buffer are untouched
+    finally:
+        comp.set_param("variant", 0)
