@@ -53,17 +53,22 @@ ccl::env_data parse_env() {
     return e;
 }
 
-// the library's float16 mode follows ccl::global_data::env().fp16_impl_type, which a caller may also set by hand
-int bf16_impl_for(const ccl_datatype& dtype) {
-    const ccl::env_data& e = ccl::global_data::env();
-    if (dtype.idx() == ccl::datatype::float16) {
-        int impl = (int)e.fp16_impl_type;
-        if (impl < MI_CCL_FP16_F16C || impl > MI_CCL_FP16_AVX512FP16)
-            fail("float16 reduction needs fp16_impl_type f16c, avx512f or avx512fp16");     // fp16.cpp:41-53 has no other path
-        if (mi_ccl_get_param("fp16_impl") != impl)
-            mi_ccl_set_param("fp16_impl", impl);
-    }
-    return (int)e.bf16_impl_type;
+// The library's float16 mode follows ccl::global_data::env().fp16_impl_type, which a caller may also set by hand.
+// Returns false when that value names no implementation: the reference's dispatch has no branch for it and leaves
+// inout as it was (src/comp/fp16/fp16_intrisics.hpp:204-248), and so do the functions below.
+bool fp16_mode(const ccl_datatype& dtype) {
+    if (dtype.idx() != ccl::datatype::float16)
+        return true;
+    const int impl = (int)ccl::global_data::env().fp16_impl_type;
+    if (impl < MI_CCL_FP16_F16C || impl > MI_CCL_FP16_AVX512FP16)
+        return false;
+    if (mi_ccl_get_param("fp16_impl") != impl)
+        mi_ccl_set_param("fp16_impl", impl);
+    return true;
+}
+
+int bf16_impl() {
+    return (int)ccl::global_data::env().bf16_impl_type;
 }
 
 // ccl::reduction::custom: the callback is host code, so both buffers are staged to the host and the result is
@@ -140,8 +145,10 @@ ccl::status ccl_comp_reduce(ccl_sched* sched, const void* in_buf, size_t in_coun
     // only the 16-bit paths report a count (bf16.cpp:94-96, fp16.cpp:48-50)
     if (out_count && (dtype.idx() == ccl::datatype::bfloat16 || dtype.idx() == ccl::datatype::float16))
         *out_count = in_count;
+    if (!fp16_mode(dtype))
+        return ccl::status::success;        // float16 without an implementation selected: inout stays as it is
     return to_status(mi_ccl_comp_reduce((int)dtype.idx(), (int)reduction, in_buf, in_count, inout_buf,
-                                        bf16_impl_for(dtype), stream_of(sched)),
+                                        bf16_impl(), stream_of(sched)),
                      "ccl_comp_reduce");
 }
 
@@ -163,9 +170,11 @@ ccl::status ccl_comp_batch_reduce(const void* in_buf, const std::vector<size_t>&
     if (out_count && !bf16_keep_precision_mode && offsets.size() > 1 &&
         (dtype.idx() == ccl::datatype::bfloat16 || dtype.idx() == ccl::datatype::float16))
         *out_count = in_count;
+    if (!fp16_mode(dtype))
+        return ccl::status::success;        // every pairwise call of the chain leaves inout as it is
     return to_status(mi_ccl_comp_batch_reduce(in_buf, offsets.data(), offsets.size(), in_count, inout_buf,
                                               (int)dtype.idx(), (int)reduction, bf16_keep_precision_mode,
-                                              bf16_impl_for(dtype), stream_of(sched)),
+                                              bf16_impl(), stream_of(sched)),
                      "ccl_comp_batch_reduce");
 }
 
@@ -182,7 +191,8 @@ void ccl_fp16_reduce(const void* in_buf, size_t in_cnt, void* inout_buf, size_t*
                      ccl_sched* sched) {
     if (out_cnt)
         *out_cnt = in_cnt;                                             // fp16.cpp:48-50
-    bf16_impl_for(ccl_datatype_storage::instance().get(ccl::datatype::float16));
+    if (!fp16_mode(ccl_datatype_storage::instance().get(ccl::datatype::float16)))
+        return;
     to_status(mi_ccl_fp16_reduce(in_buf, in_cnt, inout_buf, (int)reduction_op, stream_of(sched)), "ccl_fp16_reduce");
 }
 
@@ -209,8 +219,9 @@ ccl::status ccl_comp_reduce_n(ccl_sched* sched, const void* own_buf, const std::
     srcs.push_back(own_buf);
     srcs.insert(srcs.end(), peer_bufs.begin(), peer_bufs.end());
     int lp = bf16_keep_precision_mode ? MI_CCL_LP_KEEP_PRECISION : MI_CCL_LP_PAIRWISE;
+    (void)fp16_mode(dtype);     // the device kernels have no "no implementation" state: the library's current mode applies
     return to_status(mi_ccl_comp_reduce_n((int)dtype.idx(), (int)reduction, srcs.data(), (int)srcs.size(), out_buf,
-                                          count, lp, bf16_impl_for(dtype), stream_of(sched)),
+                                          count, lp, bf16_impl(), stream_of(sched)),
                      "ccl_comp_reduce_n");
 }
 
@@ -226,8 +237,9 @@ ccl::status ccl_comp_reduce_write_n(ccl_sched* sched, const void* own_buf, const
     srcs.push_back(own_buf);
     srcs.insert(srcs.end(), peer_bufs.begin(), peer_bufs.end());
     int lp = bf16_keep_precision_mode ? MI_CCL_LP_KEEP_PRECISION : MI_CCL_LP_PAIRWISE;
+    (void)fp16_mode(dtype);
     return to_status(mi_ccl_comp_reduce_write_n((int)dtype.idx(), (int)reduction, srcs.data(), (int)srcs.size(),
                                                 out_bufs.data(), (int)out_bufs.size(), count, lp,
-                                                bf16_impl_for(dtype), stream_of(sched)),
+                                                bf16_impl(), stream_of(sched)),
                      "ccl_comp_reduce_write_n");
 }

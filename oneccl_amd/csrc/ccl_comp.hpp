@@ -84,7 +84,9 @@ typedef enum {
 namespace ccl {
 // The two knobs of the reference's env_data that this path reads (src/common/env/env.cpp:711-720): which
 // CPU implementation's results to reproduce.  Defaults: avx512bf (round to nearest even) and avx512f;
-// CCL_BF16 = scalar | avx512f | avx512bf and CCL_FP16 = f16c | avx512f are read once, like the reference.
+// CCL_BF16 = scalar | avx512f | avx512bf and CCL_FP16 = f16c | avx512f | avx512fp16 are read once, like the reference.
+// A float16 reduce with fp16_impl_type set to a value that names no implementation leaves inout untouched, as the
+// reference's dispatch does (src/comp/fp16/fp16_intrisics.hpp:204-248).
 struct env_data {
     ccl_bf16_impl_type bf16_impl_type = ccl_bf16_avx512bf;
     ccl_fp16_impl_type fp16_impl_type = ccl_fp16_avx512f;

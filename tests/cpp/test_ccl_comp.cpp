@@ -219,6 +219,30 @@ int main() {
         for (int i = 0; i < 22; i++) ok = ok && w[i] == ((uint32_t)h[i] << 16);
         EXPECT(ok, "bf16->fp32 arrays");
     }
+    // float16 implementation knob (fp16_utils.hpp:26-32): avx512f quiets a signalling NaN that min hands back, avx512fp16
+    // keeps it, and a value that names no implementation makes the reduce a no-op, as in the reference (probe values
+    // of the reference library: fp16_intrisics.hpp:204-248 has no else branch)
+    {
+        const ccl_fp16_impl_type saved = ccl::global_data::env().fp16_impl_type;
+        std::vector<uint16_t> in = { 0x3c00, 0x3c00, 0x7c01, 0x4000 }, io = { 0x7c01, 0x4000, 0x3c00, 0x3c00 };
+        struct { ccl_fp16_impl_type impl; uint16_t want[4]; } cases[] = {
+            { ccl_fp16_avx512f, { 0x7e01, 0x3c00, 0x3c00, 0x3c00 } },          // min(in, io): io on NaN, quieted
+            { ccl_fp16_avx512fp16, { 0x7c01, 0x3c00, 0x3c00, 0x3c00 } },       // the same operand, untouched
+            { ccl_fp16_no_compiler_support, { 0x7c01, 0x4000, 0x3c00, 0x3c00 } },   // inout unchanged
+        };
+        for (auto& c : cases) {
+            ccl::global_data::env().fp16_impl_type = c.impl;
+            DevBuf<uint16_t> din(in), dio(io);
+            size_t out_count = 0;
+            ccl_comp_reduce(&sched, din.p, 4, dio.p, &out_count, DT(ccl::datatype::float16), ccl::reduction::min, nullptr);
+            std::vector<uint16_t> got = dio.host();
+            EXPECT(memcmp(got.data(), c.want, 8) == 0 && out_count == 4, "fp16 impl %d: %04x %04x %04x %04x", (int)c.impl, got[0], got[1], got[2], got[3]);
+            std::vector<uint16_t> exp = io;
+            orc_fp16_reduce(in.data(), 4, exp.data(), ORC_MIN, (int)c.impl);
+            EXPECT(memcmp(got.data(), exp.data(), 8) == 0, "fp16 impl %d equals the oracle", (int)c.impl);
+        }
+        ccl::global_data::env().fp16_impl_type = saved;
+    }
     // fusion manager over the HIP backend: 700 small bf16 gradient tensors arrive as individual requests, are fused
     // (tight layout, at most 256 per launch), reduced against 7 peer fusion buffers by ONE 8-input reduce per launch,
     // and unpacked.  Peer j holds the constant c_j everywhere, so the expected tensor does not depend on where the
