@@ -1,8 +1,11 @@
 // N-input elementwise reduce kernels for gfx950 (MI355X), templated on an element-traits class.
 //
-// Every kernel is a pure HBM stream: each lane issues one 128-bit load per input per unrolled step (a
-// wave reads 1 KiB contiguous per input per instruction), folds the inputs in argument order in registers
-// and writes one 128-bit nontemporal store.  There is no cross-lane traffic, no LDS and no MFMA.
+// Every kernel is a pure HBM stream: each lane issues one 128-bit load per input per step (a wave reads 1 KiB
+// contiguous per input per instruction), folds the inputs in argument order in registers and writes one 128-bit
+// nontemporal store per output.  There is no cross-lane traffic and no MFMA.  Two forms exist: a streaming form
+// (reduce_vec_kernel, reduce_multi_kernel), and for large buffers a phased form (reduce_phased_kernel,
+// reduce_multi_phased_kernel) that parks results in LDS and registers so that the whole chip reads for a while and
+// then writes for a while -- HBM loses about a quarter of its bandwidth when reads and writes are interleaved.
 //
 // Arithmetic follows the oneCCL CPU reduction: acc = src0; acc = step(in = src_j, inout = acc), j = 1..N-1
 // (src/comp/comp.cpp:31-58 for the step, src/kernels/kernels.cl:279-282 for the order).
