@@ -3,7 +3,6 @@
 
 #include <hip/hip_runtime.h>
 
-#include "../../include/mi_ccl_comp.h"
 
 namespace {
 
@@ -13,10 +12,6 @@ namespace {
 void check_hip(hipError_t e, const char* what) {
     if (e != hipSuccess)
         fail(std::string(what) + ": " + hipGetErrorString(e));
-}
-void check_rc(int rc, const char* what) {
-    if (rc != MI_CCL_SUCCESS)
-        fail(std::string(what) + ": " + mi_ccl_status_str(rc));
 }
 hipStream_t stream_of(ccl_sched* sched) {
     return (hipStream_t)sched->stream;
