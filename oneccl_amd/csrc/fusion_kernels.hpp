@@ -163,6 +163,14 @@ fusion_reduce_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers
     }
 }
 
+// Items per phase of the phased fused kernel whose results wait in registers on top of the kPhaseU / 2 that wait in
+// LDS (two vectors = 8 registers per item).  A traits class with heavier arithmetic specialises this before its
+// kernels are instantiated; the build fails on any scratch use.
+template <class TR>
+struct FusionPhaseRegs {
+    static constexpr int items(int nt) { return nt <= 8 ? 12 : 0; }     // with more, the slot selection no longer stays in registers
+};
+
 // The same reduce with reads and writes separated in time (see reduce_phased_kernel): each block takes kPhaseU / 2
 // work items per phase (an item is 16 KiB of one tensor = two vectors per lane), keeps their results in LDS, and
 // writes them after the chip-wide barrier.  Item (phase, slot, block) = phase * slots * blocks + slot * blocks + block.
@@ -174,23 +182,27 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                             const FusionItem* items, uint32_t nitems, uint32_t t0, PhaseSync* ps) {
     typedef typename TR::elem_t E;
     constexpr uint32_t ES = sizeof(E);
-    constexpr int S = kPhaseU / 2;
+    constexpr int S = kPhaseU / 2;                      // items per phase whose results wait in LDS
+    constexpr int RI = FusionPhaseRegs<TR>::items(NT);  // ... and in registers (two vectors per lane each)
+    constexpr int SLOTS = S + RI;
     constexpr int NP = NT - 1;
     static_assert(kFusionChunk == 2 * 16 * kPhaseBlock, "an item is two vectors per lane");
-    static_assert(S <= 64, "one descriptor per lane of a wave");
+    static_assert(SLOTS <= 64, "one descriptor per lane of a wave");
+    static_assert(RI <= 12, "the register slots are named one by one below");
     __shared__ u32x4 stage[kPhaseU * kPhaseBlock];
+    u32x4 rs[2 * (RI > 0 ? RI : 1)];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
     bool give_up = false;
     unsigned gen = 0;
     if (tid == 0) gen = MI_ALOAD(&ps->rel.v);
-    const uint64_t per_phase = (uint64_t)S * gridDim.x;
+    const uint64_t per_phase = (uint64_t)SLOTS * gridDim.x;
     for (uint64_t p0 = 0; p0 < nitems; p0 += per_phase) {
         // Lane k of every wave fetches the descriptor of this block's k-th item of the phase, so that the chain
         // item -> tensor tables -> pointers is walked once, for all items at once, instead of once per item.
         uint64_t d_a = 0, d_o = 0, d_poff = 0;
         uint32_t d_nb = 0;      // 0: no item in this slot
-        if (lane < (uint32_t)S) {
+        if (lane < (uint32_t)SLOTS) {
             const uint64_t it = p0 + (uint64_t)lane * gridDim.x + blockIdx.x;
             if (it < nitems) {
                 const FusionItem w = items[it];
@@ -202,7 +214,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                 d_poff = off[w.t] + lo;
             }
         }
-        for (int k = 0; k < S; k++) {
+        for (int k = 0; k < SLOTS; k++) {
             const uint32_t nb = __shfl(d_nb, k, 64);
             if (nb == 0) break;
             const unsigned char* a = (const unsigned char*)(uintptr_t)__shfl(d_a, k, 64);
@@ -235,8 +247,20 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                     res[0] = r0[0];
                     res[1] = r1[0];
                 }
-                stage[(2 * k) * kPhaseBlock + tid] = res[0];
-                stage[(2 * k + 1) * kPhaseBlock + tid] = res[1];
+                if (k < S) {
+                    stage[(2 * k) * kPhaseBlock + tid] = res[0];
+                    stage[(2 * k + 1) * kPhaseBlock + tid] = res[1];
+                }
+                else {
+                    // a register file has no run-time index: the slot is picked by a (wave-uniform) branch
+#define MI_RS_PUT(i) case i: if (i < RI) { rs[2 * (i < RI ? i : 0)] = res[0]; rs[2 * (i < RI ? i : 0) + 1] = res[1]; } break;
+                    switch (k - S) {
+                        MI_RS_PUT(0) MI_RS_PUT(1) MI_RS_PUT(2) MI_RS_PUT(3) MI_RS_PUT(4) MI_RS_PUT(5)
+                        MI_RS_PUT(6) MI_RS_PUT(7) MI_RS_PUT(8) MI_RS_PUT(9) MI_RS_PUT(10) MI_RS_PUT(11)
+                        default: break;
+                    }
+#undef MI_RS_PUT
+                }
                 if (tid < head + tail) {
                     const uint32_t i = (tid < head) ? tid : head + nvec * TR::VEC + (tid - head);
                     typename TR::acc_t r = TR::init(((const E*)a)[i]);
@@ -257,7 +281,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
             }
         }
         phase_barrier(ps, ++gen, give_up);
-        for (int k = 0; k < S; k++) {
+        for (int k = 0; k < SLOTS; k++) {
             const uint32_t nb = __shfl(d_nb, k, 64);
             if (nb == 0) break;
             const unsigned char* a = (const unsigned char*)(uintptr_t)__shfl(d_a, k, 64);
@@ -274,8 +298,22 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                 if (head > nelem) head = nelem;
                 const uint32_t nvec = (nelem - head) / TR::VEC;
                 u32x4* d = (u32x4*)(o + head * ES);
-                if (tid < nvec) st_stream(d + tid, stage[(2 * k) * kPhaseBlock + tid]);
-                if (tid + kPhaseBlock < nvec) st_stream(d + tid + kPhaseBlock, stage[(2 * k + 1) * kPhaseBlock + tid]);
+                u32x4 v0 = { 0, 0, 0, 0 }, v1 = v0;
+                if (k < S) {
+                    v0 = stage[(2 * k) * kPhaseBlock + tid];
+                    v1 = stage[(2 * k + 1) * kPhaseBlock + tid];
+                }
+                else {
+#define MI_RS_GET(i) case i: if (i < RI) { v0 = rs[2 * (i < RI ? i : 0)]; v1 = rs[2 * (i < RI ? i : 0) + 1]; } break;
+                    switch (k - S) {
+                        MI_RS_GET(0) MI_RS_GET(1) MI_RS_GET(2) MI_RS_GET(3) MI_RS_GET(4) MI_RS_GET(5)
+                        MI_RS_GET(6) MI_RS_GET(7) MI_RS_GET(8) MI_RS_GET(9) MI_RS_GET(10) MI_RS_GET(11)
+                        default: break;
+                    }
+#undef MI_RS_GET
+                }
+                if (tid < nvec) st_stream(d + tid, v0);
+                if (tid + kPhaseBlock < nvec) st_stream(d + tid + kPhaseBlock, v1);
             }
         }
         if (p0 + per_phase < nitems) phase_barrier(ps, ++gen, give_up);
