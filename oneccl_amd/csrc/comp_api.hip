@@ -42,7 +42,7 @@ static std::atomic<int> g_waves_per_cu{ 256 };
 static std::atomic<int> g_max_blocks{ 0 };
 static std::atomic<int> g_xcd_chunked{ 0 };
 static std::atomic<int> g_variant{ 0 };
-static std::atomic<long> g_phased_min_bytes{ 320L << 20 };
+static std::atomic<long> g_phased_min_bytes{ 160L << 20 };
 static std::atomic<int> g_fp16_impl{ MI_CCL_FP16_AVX512F };
 static std::atomic<int> g_num_cus[64];
 
@@ -370,9 +370,10 @@ int mi_ccl_comp_copy(const void* in, void* out, size_t bytes, int use_nontempora
         return MI_CCL_INVALID_ARGUMENTS;
     Tuning t = current_tuning();
     const uintptr_t mis = (uintptr_t)out & 15u;
-    // large copies go through the one-input reduce (a copy for plain types), which separates reads from writes
+    // very large copies go through the one-input reduce (a copy for plain types), whose phased form separates
+    // reads from writes; below that the plain copy kernel is as fast
     if (((uintptr_t)in & 15u) == mis && t.sync && t.variant == 0 &&
-        2 * (uint64_t)bytes >= 3 * (uint64_t)t.phased_min_bytes) {
+        2 * (uint64_t)bytes >= 25 * (uint64_t)t.phased_min_bytes) {
         LaunchArgs a;
         const void* srcs[1] = { in };
         a.srcs = srcs;

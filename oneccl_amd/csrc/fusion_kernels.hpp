@@ -344,10 +344,11 @@ inline hipError_t launch_fusion_op(const FusionLaunchArgs& a) {
             out.p[t - t0] = a.out[t];
         }
         hipError_t e = hipSuccess;
-        // large groups: separate reads from writes in time (at most 16 KiB of padding per item is over-counted)
+        // large groups (from 320 MB of traffic by default): separate reads from writes in time (at most 16 KiB of
+        // padding per item is over-counted)
         const uint64_t traffic = (uint64_t)(a.n_peers + 2) * (i1 - i0) * kFusionChunk;
         const bool phased = a.tune.sync && a.tune.num_cus >= kPhaseGroups && a.n_peers >= 1 && a.n_peers <= 7 &&
-                            (a.tune.variant == 8 || (a.tune.variant == 0 && traffic >= (uint64_t)a.tune.phased_min_bytes));
+                            (a.tune.variant == 8 || (a.tune.variant == 0 && traffic >= 2 * (uint64_t)a.tune.phased_min_bytes));
         if (phased) {
             switch (a.n_peers) {
                 case 1: e = launch_fusion_phased<TR, OP, 2>(a, own, out, pp, i0, i1, t0); break;

@@ -6,11 +6,6 @@ template <>
 struct HasUnrollVariants<Bf16KeepTraits<true>> {
     static constexpr bool value = true;
 };
-// the headline kernel: staged as deep as the register file allows without spilling
-template <>
-struct PhaseRegs<Bf16KeepTraits<true>> {
-    static constexpr int fit(int n) { return n <= 4 ? 20 : 28; }
-};
 template hipError_t launch_reduce<Bf16KeepTraits<true>>(const LaunchArgs&);
 template hipError_t launch_fusion_reduce<Bf16KeepTraits<true>>(const FusionLaunchArgs&);
 }  // namespace mi

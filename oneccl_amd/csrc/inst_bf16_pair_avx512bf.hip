@@ -2,11 +2,6 @@
 #include "fusion_kernels.hpp"
 
 namespace mi {
-// seven rounding steps per element make this the heaviest traits class; deeper register staging spills
-template <>
-struct PhaseRegs<Bf16PairwiseTraits<true, true>> {
-    static constexpr int fit(int n) { return n <= 4 ? 20 : 12; }
-};
 // ... and with 7 or 8 inputs the streaming kernel is bound by them, not by loads in flight
 template <>
 struct StreamUnroll<Bf16PairwiseTraits<true, true>> {

@@ -7,6 +7,10 @@ template <>
 struct FusionPhaseRegs<U8Traits> {
     static constexpr int items(int nt) { return nt <= 6 ? 12 : 6; }
 };
+template <>
+struct MultiPhaseRegs<U8Traits> {
+    static constexpr int groups = 5;
+};
 template hipError_t launch_reduce<U8Traits>(const LaunchArgs&);
 template hipError_t launch_fusion_reduce<U8Traits>(const FusionLaunchArgs&);
 }  // namespace mi

@@ -41,7 +41,7 @@ struct Tuning {
     int waves_per_cu;   // 256-thread blocks per CU the grid is capped at (a block loops over tiles beyond that)
     int max_blocks;     // 0 = no cap
     int xcd_chunked;    // 1: each XCD streams one contiguous eighth of the buffer
-    int variant;        // 0 = automatic; 1, 2, 4 = streaming kernel with that unroll depth; 8 = phased kernel
+    int variant;        // 0 = automatic; 1, 2, 4 = streaming kernel (with that unroll depth where compiled); 8 = phased kernel
     int num_cus;
     long phased_min_bytes;   // automatic choice: phased kernel when (N + 1) * bytes per buffer reaches this
     struct PhaseSync* sync;  // device-resident barrier words of the current device (may be null)
@@ -488,15 +488,6 @@ __device__ __forceinline__ void phase_barrier(PhaseSync* ps, unsigned gen, bool&
     __syncthreads();
 }
 
-// Vectors per lane per phase that are staged in registers on top of the kPhaseU staged in LDS, by number of
-// inputs.  A 512-lane block has 256 registers per lane; the in-flight loads (about eight, 4 registers each),
-// addressing and accumulators leave room for roughly this many staged vectors.  A traits class with lighter or
-// heavier arithmetic specialises this before its kernels are instantiated; the build fails on any scratch use.
-template <class TR>
-struct PhaseRegs {
-    static constexpr int fit(int n) { return n <= 4 ? 20 : 22; }
-};
-
 // G vectors per lane at once: all G x N loads are issued before the first is used, so that a lane keeps about
 // eight 128-bit loads in flight whatever N is.  Callers branch around this (a real branch keeps the compiler
 // from hoisting the loads of later steps, which would spill).
@@ -534,61 +525,6 @@ __device__ __forceinline__ void reduce_group_guarded(const u32x4* const (&s)[N],
             }
         }
     }
-}
-
-template <class TR, int OP, int N>
-__global__ void __launch_bounds__(kPhaseBlock)
-reduce_phased_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint32_t tail, PhaseSync* ps) {
-    typedef typename TR::elem_t E;
-    constexpr int G = (N == 1) ? 10 : (N == 2) ? 4 : (N <= 4) ? 2 : 1;       // vectors per lane per step
-    constexpr int R = PhaseRegs<TR>::fit(N) / G * G;           // vectors per lane staged in registers
-    static_assert(kPhaseU % G == 0, "LDS steps must be a multiple of the group size");
-    __shared__ u32x4 stage[kPhaseU * kPhaseBlock];
-    const u32x4* s[N];
-#pragma unroll
-    for (int j = 0; j < N; j++) s[j] = (const u32x4*)((const E*)src.p[j] + head);
-    u32x4* d = (u32x4*)((E*)dst + head);
-    const uint64_t gthreads = (uint64_t)gridDim.x * kPhaseBlock;
-    const uint64_t gtid = (uint64_t)blockIdx.x * kPhaseBlock + threadIdx.x;
-    const uint64_t per_phase = gthreads * (kPhaseU + R);
-    bool give_up = false;
-    unsigned gen = 0;
-    if (threadIdx.x == 0) gen = MI_ALOAD(&ps->rel.v);     // read before this block's first arrival
-    for (uint64_t p0 = 0; p0 < nvec; p0 += per_phase) {
-        u32x4 r[R > 0 ? R : 1];
-#pragma unroll
-        for (int u = 0; u < R; u += G) {
-            uint64_t idx[G];
-            u32x4 out[G];
-#pragma unroll
-            for (int g = 0; g < G; g++) idx[g] = p0 + (uint64_t)(u + g) * gthreads + gtid;
-            reduce_group_guarded<TR, OP, N, G>(s, idx, nvec, out);
-#pragma unroll
-            for (int g = 0; g < G; g++) r[u + g] = out[g];
-        }
-        for (int u = 0; u < kPhaseU; u += G) {
-            uint64_t idx[G];
-            u32x4 out[G];
-#pragma unroll
-            for (int g = 0; g < G; g++) idx[g] = p0 + (uint64_t)(R + u + g) * gthreads + gtid;
-            reduce_group_guarded<TR, OP, N, G>(s, idx, nvec, out);
-#pragma unroll
-            for (int g = 0; g < G; g++) stage[(u + g) * kPhaseBlock + threadIdx.x] = out[g];
-        }
-        phase_barrier(ps, ++gen, give_up);      // all reads of this phase are done
-#pragma unroll
-        for (int u = 0; u < R; u++) {
-            const uint64_t i = p0 + (uint64_t)u * gthreads + gtid;
-            if (i < nvec) st_stream(d + i, r[u]);
-        }
-        for (int u = 0; u < kPhaseU; u++) {
-            const uint64_t i = p0 + (uint64_t)(R + u) * gthreads + gtid;
-            if (i < nvec) st_stream(d + i, stage[u * kPhaseBlock + threadIdx.x]);
-        }
-        // all writes of this phase are issued before the next phase reads; nothing follows the last phase
-        if (p0 + per_phase < nvec) phase_barrier(ps, ++gen, give_up);
-    }
-    if (blockIdx.x == 0 && (head | tail)) reduce_edges<TR, OP>(src, N, dst, head, nvec, tail);
 }
 
 // One element per lane, any alignment of the buffers relative to each other.
@@ -667,37 +603,68 @@ reduce_multi_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uin
     if (blockIdx.x == 0 && (head | tail)) reduce_multi_edges<TR, OP>(src, n, dst, m, head, nvec, tail);
 }
 
-// The phased form of the same: kPhaseU vectors per lane are reduced into LDS while HBM sees only reads, then stored
-// to every destination while it sees only writes.
+// Groups of four result vectors per lane that the phased form below keeps in registers on top of the kPhaseU vectors
+// it keeps in LDS.  A traits class with heavier arithmetic specialises this before its kernels are instantiated; the
+// build fails on any scratch use.
+template <class TR>
+struct MultiPhaseRegs {
+    static constexpr int groups = 6;
+};
+
+// The phased form of the same: kPhaseU vectors per lane in LDS and 4 x MultiPhaseRegs::groups in registers are
+// reduced while HBM sees only reads, then stored to every destination while it sees only writes.  The register
+// groups are unrolled (a register file has no run-time index); the loop over the inputs inside each stays a loop.
 template <class TR, int OP>
 __global__ void __launch_bounds__(kPhaseBlock)
 reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uint64_t nvec, uint32_t tail,
                            PhaseSync* ps) {
     typedef typename TR::elem_t E;
-    constexpr int G = 4;
+    constexpr int G = 4;                                // vectors per lane and input in flight
+    constexpr int RG = MultiPhaseRegs<TR>::groups;
+    constexpr int LG = kPhaseU / G;                     // groups staged in LDS
     static_assert(kPhaseU % G == 0, "LDS steps must be a multiple of the group size");
     __shared__ u32x4 stage[kPhaseU * kPhaseBlock];
     const uint64_t gthreads = (uint64_t)gridDim.x * kPhaseBlock;
     const uint64_t gtid = (uint64_t)blockIdx.x * kPhaseBlock + threadIdx.x;
-    const uint64_t per_phase = gthreads * kPhaseU;
+    const uint64_t per_phase = gthreads * (uint64_t)(G * (RG + LG));
+    auto pos = [&](uint64_t p0, int u) -> uint64_t { return p0 + (uint64_t)u * gthreads + gtid; };   // slot u of this lane
     bool give_up = false;
     unsigned gen = 0;
     if (threadIdx.x == 0) gen = MI_ALOAD(&ps->rel.v);
     for (uint64_t p0 = 0; p0 < nvec; p0 += per_phase) {
-        for (int u = 0; u < kPhaseU; u += G) {
+        u32x4 rs[G * (RG > 0 ? RG : 1)];
+#pragma unroll
+        for (int q = 0; q < RG; q++) {
             uint64_t idx[G];
             u32x4 v[G];
 #pragma unroll
-            for (int g = 0; g < G; g++) idx[g] = p0 + (uint64_t)(u + g) * gthreads + gtid;
+            for (int g = 0; g < G; g++) idx[g] = pos(p0, q * G + g);
+            if (idx[0] < nvec) {
+                reduce_rt_tile<TR, OP, G>(src, n, head, idx, nvec, v);
+#pragma unroll
+                for (int g = 0; g < G; g++) rs[q * G + g] = v[g];
+            }
+        }
+        for (int q = 0; q < LG; q++) {
+            uint64_t idx[G];
+            u32x4 v[G];
+#pragma unroll
+            for (int g = 0; g < G; g++) idx[g] = pos(p0, (RG + q) * G + g);
+            if (idx[0] >= nvec) break;      // slabs grow with q: nothing further for this lane in this phase
             reduce_rt_tile<TR, OP, G>(src, n, head, idx, nvec, v);
 #pragma unroll
-            for (int g = 0; g < G; g++) stage[(u + g) * kPhaseBlock + threadIdx.x] = v[g];
+            for (int g = 0; g < G; g++) stage[(q * G + g) * kPhaseBlock + threadIdx.x] = v[g];
         }
         phase_barrier(ps, ++gen, give_up);
         for (int k = 0; k < m; k++) {
             u32x4* d = (u32x4*)((E*)dst.p[k] + head);
+#pragma unroll
+            for (int u = 0; u < G * RG; u++) {
+                const uint64_t i = pos(p0, u);
+                if (i < nvec) st_stream(d + i, rs[u]);
+            }
             for (int u = 0; u < kPhaseU; u++) {
-                const uint64_t i = p0 + (uint64_t)u * gthreads + gtid;
+                const uint64_t i = pos(p0, G * RG + u);
                 if (i < nvec) st_stream(d + i, stage[u * kPhaseBlock + threadIdx.x]);
             }
         }
@@ -758,27 +725,8 @@ struct StreamUnroll {
 };
 
 template <class TR, int OP, int N>
-inline hipError_t launch_phased(const LaunchArgs& a, uint32_t head, uint64_t nvec, uint32_t tail) {
-    SrcFixed<N> s;
-    for (int j = 0; j < N; j++) s.p[j] = a.srcs[j];
-    // one block per CU, a multiple of the arrival groups; all blocks must be resident together
-    int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
-    hipLaunchKernelGGL((reduce_phased_kernel<TR, OP, N>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.dst, head,
-                       nvec, tail, a.tune.sync);
-    return hipGetLastError();
-}
-
-template <class TR, int OP, int N>
 inline hipError_t launch_fixed_unroll(const LaunchArgs& a, uint32_t head, uint64_t nvec, uint32_t tail) {
     constexpr int kDefault = StreamUnroll<TR>::get(N);
-    {
-        const bool can = a.tune.sync != nullptr && a.tune.num_cus >= kPhaseGroups;
-        // with two or three inputs the streaming kernel holds up longer (less to interleave per write)
-        const uint64_t traffic = (uint64_t)(N + 1) * nvec * 16u;
-        const bool big = traffic >= (uint64_t)a.tune.phased_min_bytes * (N <= 3 ? 3u : 1u);
-        if (can && (a.tune.variant == 8 || (a.tune.variant == 0 && big)))
-            return launch_phased<TR, OP, N>(a, head, nvec, tail);
-    }
     if constexpr (HasUnrollVariants<TR>::value) {
         switch (a.tune.variant) {
             case 1: return launch_fixed<TR, OP, N, 1>(a, head, nvec, tail);
@@ -788,6 +736,18 @@ inline hipError_t launch_fixed_unroll(const LaunchArgs& a, uint32_t head, uint64
         }
     }
     return launch_fixed<TR, OP, N, kDefault>(a, head, nvec, tail);
+}
+
+// The phased form pays for its barriers from a few hundred MB of traffic, later the fewer inputs there are (less to
+// interleave per write).  Measured crossovers against the streaming kernels, in traffic per launch: 150 MB with 5 or
+// more inputs, 240 MB with 4, 0.8 GB with 3, about 4 GB with 1 or 2; 320 MB with more than one destination.
+// Tuning::phased_min_bytes scales them all (default 160 MB); Tuning::variant 8 forces the phased form.
+inline bool wants_phased(const LaunchArgs& a, uint64_t nvec) {
+    if (a.tune.sync == nullptr || a.tune.num_cus < kPhaseGroups) return false;
+    if (a.tune.variant != 0) return a.tune.variant == 8;
+    const uint64_t traffic = (uint64_t)(a.n + a.m) * nvec * 16u;
+    const unsigned halves = a.m > 1 ? 4u : a.n >= 5 ? 2u : a.n == 4 ? 3u : a.n == 3 ? 10u : a.n == 2 ? 60u : 50u;
+    return 2 * traffic >= (uint64_t)a.tune.phased_min_bytes * halves;
 }
 
 template <class TR, int OP>
@@ -812,11 +772,7 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
     if (head > a.count) head = a.count;
     const uint64_t nvec = (a.count - head) / VEC;
     const uint32_t tail = (uint32_t)(a.count - head - nvec * VEC);
-    const bool can = a.tune.sync != nullptr && a.tune.num_cus >= kPhaseGroups;
-    const uint64_t traffic = (uint64_t)(a.n + a.m) * nvec * 16u;
-    // LDS staging only (no register-staged vectors): the phased form pays off later than in the one-output kernel,
-    // from about 512 MB of traffic with the default setting
-    if (can && (a.tune.variant == 8 || (a.tune.variant == 0 && traffic >= (uint64_t)a.tune.phased_min_bytes / 5 * 8))) {
+    if (wants_phased(a, nvec)) {
         int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
                            a.m, (uint32_t)head, nvec, tail, a.tune.sync);
@@ -852,6 +808,7 @@ inline hipError_t launch_op(const LaunchArgs& a) {
     if (head > a.count) head = a.count;
     const uint64_t nvec = (a.count - head) / VEC;
     const uint32_t tail = (uint32_t)(a.count - head - nvec * VEC);
+    if (wants_phased(a, nvec)) return launch_multi_op<TR, OP>(a);         // the phased kernel takes any number of inputs
     switch (a.n) {
         case 1: return launch_fixed_unroll<TR, OP, 1>(a, (uint32_t)head, nvec, tail);
         case 2: return launch_fixed_unroll<TR, OP, 2>(a, (uint32_t)head, nvec, tail);
