@@ -171,7 +171,7 @@ struct FusionPhaseRegs {
     static constexpr int items(int nt) { return nt <= 8 ? 12 : 0; }     // with more, the slot selection no longer stays in registers
 };
 
-// The same reduce with reads and writes separated in time (see reduce_phased_kernel): each block takes kPhaseU / 2
+// The same reduce with reads and writes separated in time (see reduce_multi_phased_kernel): each block takes kPhaseU / 2
 // work items per phase (an item is 16 KiB of one tensor = two vectors per lane), keeps their results in LDS, and
 // writes them after the chip-wide barrier.  Item (phase, slot, block) = phase * slots * blocks + slot * blocks + block.
 // Head/tail elements of tensors that do not start on a 16-byte boundary, and tensors whose streams disagree modulo

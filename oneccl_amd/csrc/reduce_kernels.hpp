@@ -3,8 +3,8 @@
 // Every kernel is a pure HBM stream: each lane issues one 128-bit load per input per step (a wave reads 1 KiB
 // contiguous per input per instruction), folds the inputs in argument order in registers and writes one 128-bit
 // nontemporal store per output.  There is no cross-lane traffic and no MFMA.  Two forms exist: a streaming form
-// (reduce_vec_kernel, reduce_multi_kernel), and for large buffers a phased form (reduce_phased_kernel,
-// reduce_multi_phased_kernel) that parks results in LDS and registers so that the whole chip reads for a while and
+// (reduce_vec_kernel, reduce_multi_kernel), and for large buffers a phased form (reduce_multi_phased_kernel)
+// that parks results in LDS and registers so that the whole chip reads for a while and
 // then writes for a while -- HBM loses about a quarter of its bandwidth when reads and writes are interleaved.
 //
 // Arithmetic follows the oneCCL CPU reduction: acc = src0; acc = step(in = src_j, inout = acc), j = 1..N-1
@@ -435,7 +435,7 @@ reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint
 //
 // HBM on this part loses about a quarter of its bandwidth when reads and writes are interleaved (an
 // 8-read + 1-write stream sustains ~5.5 TB/s where reads alone reach ~7.1 TB/s and writes alone ~6 TB/s).
-// This kernel keeps the two apart in time, chip-wide: one 512-lane block per CU reduces up to 44 vectors per
+// reduce_multi_phased_kernel (further down) keeps the two apart in time, chip-wide: one 512-lane block per CU reduces up to 44 vectors per
 // lane into LDS and registers (read phase: HBM sees only reads), all blocks meet at a barrier, then every block
 // streams its staged results out (write phase: HBM sees only writes), and they meet again.  Each phase boundary
 // costs a few microseconds of idle HBM, so a phase holds as much as the CU can: 160 KiB of LDS plus up to 24
