@@ -739,14 +739,14 @@ inline hipError_t launch_fixed_unroll(const LaunchArgs& a, uint32_t head, uint64
 }
 
 // The phased form pays for its barriers from a few hundred MB of traffic, later the fewer inputs there are (less to
-// interleave per write).  Measured crossovers against the streaming kernels, in traffic per launch: 150 MB with 5 or
-// more inputs, 240 MB with 4, 0.8 GB with 3, about 4 GB with 1 or 2; 320 MB with more than one destination.
+// interleave per write).  Measured crossovers against the streaming kernels, in traffic per launch: 240 MB with 4 or
+// more inputs, 0.8 GB with 3, about 4 GB with 1 or 2; 320 MB with more than one destination.
 // Tuning::phased_min_bytes scales them all (default 160 MB); Tuning::variant 8 forces the phased form.
 inline bool wants_phased(const LaunchArgs& a, uint64_t nvec) {
     if (a.tune.sync == nullptr || a.tune.num_cus < kPhaseGroups) return false;
     if (a.tune.variant != 0) return a.tune.variant == 8;
     const uint64_t traffic = (uint64_t)(a.n + a.m) * nvec * 16u;
-    const unsigned halves = a.m > 1 ? 4u : a.n >= 5 ? 2u : a.n == 4 ? 3u : a.n == 3 ? 10u : a.n == 2 ? 60u : 50u;
+    const unsigned halves = a.m > 1 ? 4u : a.n >= 4 ? 3u : a.n == 3 ? 10u : a.n == 2 ? 60u : 50u;
     return 2 * traffic >= (uint64_t)a.tune.phased_min_bytes * halves;
 }
 
@@ -809,6 +809,10 @@ inline hipError_t launch_op(const LaunchArgs& a) {
     const uint64_t nvec = (a.count - head) / VEC;
     const uint32_t tail = (uint32_t)(a.count - head - nvec * VEC);
     if (wants_phased(a, nvec)) return launch_multi_op<TR, OP>(a);         // the phased kernel takes any number of inputs
+    // five or more inputs in the range between latency-bound and phased (64 to 240 MB of traffic): taking the inputs
+    // one after the other, as the run-time-count streaming kernel does, measures 5-12 % above loading them together
+    if (a.n >= 5 && a.tune.variant == 0 && (uint64_t)(a.n + 1) * nvec * 16u >= (uint64_t)a.tune.phased_min_bytes / 5 * 2)
+        return launch_multi_op<TR, OP>(a);
     switch (a.n) {
         case 1: return launch_fixed_unroll<TR, OP, 1>(a, (uint32_t)head, nvec, tail);
         case 2: return launch_fixed_unroll<TR, OP, 2>(a, (uint32_t)head, nvec, tail);
