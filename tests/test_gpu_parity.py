@@ -225,15 +225,23 @@ def test_copy_and_converters(comp):
                 got = to_host(dd, np.uint8)
                 assert (got[sb:sb + nbytes] == src[sa:sa + nbytes]).all()
                 assert (got[:sb] == 0).all() and (got[sb + nbytes:] == 0).all()
-    # a copy large enough for the phased one-input kernel, with head and tail bytes
+    # a large copy with head and tail bytes, through the plain copy kernel and (with the crossover lowered) through
+    # the phased one-input kernel that copies of several GB take
     nbytes = (800 << 20) + 5
     src_d = torch.randint(-128, 127, (nbytes + 32,), dtype=torch.int8, device="cuda")
-    dst_d = torch.zeros(nbytes + 32, dtype=torch.int8, device="cuda")
-    comp.comp_copy(src_d.data_ptr() + 3, dst_d.data_ptr() + 19, nbytes, use_nontemporal=True)
-    torch.cuda.synchronize()
-    assert torch.equal(dst_d[19:19 + nbytes], src_d[3:3 + nbytes])
-    assert int(dst_d[:19].count_nonzero()) == 0 and int(dst_d[19 + nbytes:].count_nonzero()) == 0
-    del src_d, dst_d
+    for min_bytes in (comp.get_param("phased_min_bytes"), 1 << 20):
+        default = comp.get_param("phased_min_bytes")
+        comp.set_param("phased_min_bytes", min_bytes)
+        try:
+            dst_d = torch.zeros(nbytes + 32, dtype=torch.int8, device="cuda")
+            comp.comp_copy(src_d.data_ptr() + 3, dst_d.data_ptr() + 19, nbytes, use_nontemporal=True)
+            torch.cuda.synchronize()
+        finally:
+            comp.set_param("phased_min_bytes", default)
+        assert torch.equal(dst_d[19:19 + nbytes], src_d[3:3 + nbytes])
+        assert int(dst_d[:19].count_nonzero()) == 0 and int(dst_d[19 + nbytes:].count_nonzero()) == 0
+        del dst_d
+    del src_d
     L = O.lib()
     for count in (1, 5, 16, 22, 1000, 65536 + 7):
         f32 = rng.integers(0, 2**32, count, dtype=np.uint32)
