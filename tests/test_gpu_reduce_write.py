@@ -155,3 +155,27 @@ def test_errors(comp):
     with pytest.raises(comp.CclError):
         comp.comp_reduce_write_n(O.FLOAT32, O.SUM, [a], [a], 64, lp_mode=1)     # keep precision is for bf16
     comp.comp_reduce_write_n(O.FLOAT32, O.SUM, [a], [a, a], 0)                  # count 0: nothing to do
+
+
+def test_automatic_kernel_choice_at_mid_and_large_sizes(comp):
+    """No knob set: sizes on both sides of the crossovers between the per-N streaming kernel, the run-time-count
+    streaming kernel (five and more inputs from 64 MB of traffic) and the phased kernel (from 240 MB with four and
+    more inputs), with buffers that share a misalignment, against the oracle."""
+    import torch
+    rng = np.random.default_rng(77)
+    assert comp.get_param("variant") == 0
+    for dtype, n, count, shift in [(O.BFLOAT16, 8, 3_000_001, 3), (O.BFLOAT16, 8, 5_000_003, 0), (O.BFLOAT16, 6, 9_000_001, 5),
+                                   (O.BFLOAT16, 8, 20_000_003, 1), (O.FLOAT32, 4, 9_000_002, 2), (O.FLOAT32, 4, 16_000_001, 0),
+                                   (O.INT8, 5, 30_000_001, 7), (O.INT8, 5, 50_000_017, 0), (O.FLOAT16, 7, 12_000_005, 4)]:
+        np_t = O.NP_STORAGE[dtype]
+        srcs = make_inputs(rng, dtype, count, O.SUM, n)
+        big = [to_dev(np.concatenate([np.zeros(shift, np_t), s])) for s in srcs]
+        d = [b[shift:] for b in big]
+        obig = torch.zeros(count + shift + 4, dtype=d[0].dtype, device="cuda")
+        keep = 1 if dtype == O.BFLOAT16 else 0
+        comp.comp_reduce_n(dtype, O.SUM, d, obig[shift:], count, lp_mode=keep)
+        torch.cuda.synchronize()
+        want = O.reduce_n(srcs, dtype, O.SUM, keep=keep, threads=8)
+        got = to_host(obig, np_t)
+        assert_same(got[shift:shift + count], want, dtype, f"{O.DTYPE_NAMES[dtype]} n={n} count={count} shift={shift}")
+        assert not got[:shift].view(np.uint8).any() and not got[shift + count:].view(np.uint8).any()
