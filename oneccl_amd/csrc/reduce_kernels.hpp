@@ -303,6 +303,56 @@ struct VecOps<Bf16PairwiseTraits<true, VEC_SEM>> {
     }
 };
 
+// fp16: the accumulator stays in storage format (two halves per dword, in a.v[0..3]).  sum and prod widen, combine
+// and narrow both halves of a dword.  min and max pick each half with one compare and a bit-field insert; the
+// quieting of a NaN they hand back (only the first input can bring one: a NaN `in` is never chosen) does not change
+// any later compare, so it is done once at the end, for both halves of a dword at a time -- a.v[4] says whether a
+// min/max step has happened at all (with one input there is nothing to quiet).
+template <bool NATIVE>
+struct VecOps<Fp16Traits<NATIVE>> {
+    typedef Fp16Traits<NATIVE> TR;
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ Accs<TR> init(u32x4 x) {
+        Accs<TR> a;
+#pragma unroll
+        for (int k = 0; k < 4; k++) a.v[k] = x[k];
+        a.v[4] = 0;
+        return a;
+    }
+    template <int OP>
+    static __device__ __forceinline__ void step(u32x4 x, Accs<TR>& a) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const half2_t in = __builtin_bit_cast(half2_t, (uint32_t)x[k]), io = __builtin_bit_cast(half2_t, a.v[k]);
+            if (OP == OP_SUM || OP == OP_PROD) {
+                const float lo = (OP == OP_SUM) ? ((float)io[0] + (float)in[0]) : ((float)io[0] * (float)in[0]);
+                const float hi = (OP == OP_SUM) ? ((float)io[1] + (float)in[1]) : ((float)io[1] * (float)in[1]);
+                const half2_t r = { (_Float16)lo, (_Float16)hi };
+                a.v[k] = __builtin_bit_cast(uint32_t, r);
+            }
+            else {
+                const bool lo = (OP == OP_MIN) ? (in[0] < io[0]) : (in[0] > io[0]);
+                const bool hi = (OP == OP_MIN) ? (in[1] < io[1]) : (in[1] > io[1]);
+                const uint32_t m = (lo ? 0x0000ffffu : 0u) | (hi ? 0xffff0000u : 0u);
+                a.v[k] = (x[k] & m) | (a.v[k] & ~m);
+            }
+        }
+        if (OP == OP_MIN || OP == OP_MAX) a.v[4] = 1;
+    }
+    static __device__ __forceinline__ u32x4 finish(const Accs<TR>& a) {
+        u32x4 r = { a.v[0], a.v[1], a.v[2], a.v[3] };
+        if (!NATIVE && a.v[4]) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                // a half h is a NaN iff (h & 0x7fff) > 0x7c00 iff (h & 0x7fff) + 0x03ff has bit 15 set
+                const uint32_t nan = ((r[k] & 0x7fff7fffu) + 0x03ff03ffu) & 0x80008000u;
+                r[k] |= nan >> 6;      // the quiet bit, 0x0200, of each NaN half
+            }
+        }
+        return r;
+    }
+};
+
 // bf16 accumulated in fp32 and rounded to nearest even once: element-wise init and step, packed narrowing.
 template <>
 struct VecOps<Bf16KeepTraits<true>> {
