@@ -100,6 +100,7 @@ __global__ void __launch_bounds__(kBlock)
 fusion_reduce_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers, const uint64_t* off,
                      const uint64_t* bytes, const FusionItem* items, uint32_t nitems, uint32_t t0) {
     typedef typename TR::elem_t E;
+    kernel_prologue<TR, OP>();
     constexpr uint32_t ES = sizeof(E);
     const uint32_t tid = threadIdx.x;
     for (uint32_t it = blockIdx.x; it < nitems; it += gridDim.x) {
@@ -181,6 +182,7 @@ __global__ void __launch_bounds__(kPhaseBlock)
 fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, const uint64_t* off, const uint64_t* bytes,
                             const FusionItem* items, uint32_t nitems, uint32_t t0, PhaseSync* ps) {
     typedef typename TR::elem_t E;
+    kernel_prologue<TR, OP>();
     constexpr uint32_t ES = sizeof(E);
     constexpr int S = kPhaseU / 2;                      // items per phase whose results wait in LDS
     constexpr int RI = FusionPhaseRegs<TR>::items(NT);  // ... and in registers (two vectors per lane each)

@@ -252,6 +252,22 @@ struct Accs {
     typename TR::acc_t v[TR::VEC];
 };
 
+// Traits/operation pairs whose kernels run with the wave's fp32 denormal mode set to "inputs kept, results flushed
+// to a signed zero" (MODE.FP_DENORM[1:0] = 1).  That is what the x86 sequence "fp32 add or multiply, then
+// VCVTNEPS2BF16" amounts to: the conversion reads a denormal sum as zero.  With the mode set, the packed conversion
+// needs no per-value denormal test.  Every kernel that uses VecOps<TR>::step<OP> calls kernel_prologue<TR, OP>() first.
+template <class TR, int OP>
+struct FlushF32Results {
+    static constexpr bool value = false;
+};
+template <class TR, int OP>
+__device__ __forceinline__ void kernel_prologue() {
+    if constexpr (FlushF32Results<TR, OP>::value) {
+        // s_setreg hwreg(HW_REG_MODE = 1, offset 4, size 2) <- 1
+        __builtin_amdgcn_s_setreg(1 | (4 << 6) | ((2 - 1) << 11), 1);
+    }
+}
+
 // Vector-level operations on the 128-bit unit a lane moves.  The default walks the VEC elements one by one with
 // the traits' init / step / finish; traits with a cheaper packed form specialise VecOps.
 template <class TR>
@@ -277,6 +293,15 @@ struct VecOps {
     }
 };
 
+template <bool VEC_SEM>
+struct FlushF32Results<Bf16PairwiseTraits<true, VEC_SEM>, OP_SUM> {
+    static constexpr bool value = true;
+};
+template <bool VEC_SEM>
+struct FlushF32Results<Bf16PairwiseTraits<true, VEC_SEM>, OP_PROD> {
+    static constexpr bool value = true;
+};
+
 // bf16 rounded to nearest even after every pair: the accumulator stays in storage format (two bf16 per dword, in
 // a.v[0..3]); both halves of a dword are widened, combined and narrowed together by the packed conversion.
 template <bool VEC_SEM>
@@ -295,7 +320,13 @@ struct VecOps<Bf16PairwiseTraits<true, VEC_SEM>> {
             const uint32_t in = x[k], io = a.v[k];
             const uint32_t lo = f32_step_bits<OP, VEC_SEM>(in << 16, io << 16);
             const uint32_t hi = f32_step_bits<OP, VEC_SEM>(in & 0xffff0000u, io & 0xffff0000u);
-            a.v[k] = bf16_narrow_rne_pack2(lo, hi);
+            if constexpr (FlushF32Results<TR, OP>::value) {     // a denormal sum or product is already a signed zero
+                const f32x2 f = { as_f32(lo), as_f32(hi) };
+                a.v[k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+            }
+            else {
+                a.v[k] = bf16_narrow_rne_pack2(lo, hi);
+            }
         }
     }
     static __device__ __forceinline__ u32x4 finish(const Accs<TR>& a) {
@@ -438,6 +469,7 @@ template <class TR, int OP, int N, int UNROLL>
 __global__ void __launch_bounds__(kBlock)
 reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint32_t tail, int xcd_chunked) {
     typedef typename TR::elem_t E;
+    kernel_prologue<TR, OP>();
     constexpr uint64_t kTile = (uint64_t)kBlock * UNROLL;
     const u32x4* s[N];
 #pragma unroll
@@ -635,6 +667,7 @@ __global__ void __launch_bounds__(kBlock)
 reduce_multi_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uint64_t nvec, uint32_t tail,
                     int xcd_chunked) {
     typedef typename TR::elem_t E;
+    kernel_prologue<TR, OP>();
     constexpr uint64_t kTile = (uint64_t)kBlock * UNROLL;
     const uint64_t ntiles = (nvec + kTile - 1) / kTile;
     for (TileIter it(ntiles, xcd_chunked); it.tile < it.end; it.tile += it.stride) {
@@ -669,6 +702,7 @@ __global__ void __launch_bounds__(kPhaseBlock)
 reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uint64_t nvec, uint32_t tail,
                            PhaseSync* ps) {
     typedef typename TR::elem_t E;
+    kernel_prologue<TR, OP>();
     constexpr int G = 4;                                // vectors per lane and input in flight
     constexpr int RG = MultiPhaseRegs<TR>::groups;
     constexpr int LG = kPhaseU / G;                     // groups staged in LDS

@@ -440,3 +440,51 @@ def test_fp16_native_mode_against_reference_made_vectors(comp, golden, golden_fp
         comp.set_param("fp16_impl", 3)
     with pytest.raises(comp.CclError):
         comp.set_param("fp16_impl", 1)
+
+
+def test_bf16_pairwise_tiny_sums_and_products_through_every_kernel(comp):
+    """Round-after-every-pair bf16 under avx512bf where the fp32 sum or product is a denormal: VCVTNEPS2BF16 reads it
+    as zero (the result is a signed zero), and a value just under the smallest normal must not round up to it.  Every
+    pair of a value set around the bottom of the exponent range (sums) and around the square root of it (products),
+    through the streaming and the phased kernel, the run-time-count kernels (nine inputs; two outputs) and the
+    fused kernel, in both forms."""
+    import torch
+    vals = []
+    for sign in (0, 0x8000):
+        for e in (0, 1, 2, 3, 61, 62, 63, 64, 65, 66):
+            for m in (0, 1, 0x3F, 0x40, 0x7E, 0x7F):
+                vals.append(sign | (e << 7) | m)
+    vals = np.array(vals, dtype=np.uint16)
+    a = np.tile(np.repeat(vals, vals.size), 25)          # in
+    b = np.tile(np.tile(vals, vals.size), 25)            # inout
+    count = a.size
+    zero = np.zeros(count, np.uint16)
+    for op in (O.SUM, O.PROD):
+        want2 = O.reduce_n([b, a], O.BFLOAT16, op)
+        ident = zero if op == O.SUM else np.full(count, 0x3F80, np.uint16)
+        want9 = O.reduce_n([b, a] + [ident] * 7, O.BFLOAT16, op)
+        for variant in (2, 8):
+            comp.set_param("variant", variant)
+            try:
+                da, db = to_dev(a), to_dev(b)
+                comp.comp_reduce(O.BFLOAT16, op, da, count, db)
+                torch.cuda.synchronize()
+                assert (to_host(db, np.uint16) == want2).all(), (op, variant, "pair")
+                db = to_dev(b)
+                di = to_dev(ident)
+                outs = [torch.empty_like(db) for _ in range(2)]
+                comp.comp_reduce_write_n(O.BFLOAT16, op, [db, da] + [di] * 7, outs, count)
+                torch.cuda.synchronize()
+                for o in outs:
+                    assert (to_host(o, np.uint16) == want9).all(), (op, variant, "nine inputs, two outputs")
+                plan = comp.FusionPlan([count // 2, count - count // 2], O.BFLOAT16, 256)
+                fb = torch.zeros(plan.nbytes // 2, dtype=torch.int16, device="cuda")
+                own = [db[:count // 2], db[count // 2:]]
+                plan.pack([da[:count // 2], da[count // 2:]], fb)
+                res = [torch.empty_like(t) for t in own]
+                plan.reduce(op, own, [fb], res)
+                torch.cuda.synchronize()
+                got = np.concatenate([to_host(r, np.uint16) for r in res])
+                assert (got == want2).all(), (op, variant, "fused")
+            finally:
+                comp.set_param("variant", 0)
