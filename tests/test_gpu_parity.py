@@ -354,11 +354,13 @@ def test_phased_kernel_parity(comp, dtype, op, n):
 
 
 def test_randomised_calls_against_oracle(comp):
-    """400 seeded random calls: dtype, op, input count (1..12), element count, 16-bit mode, per-buffer element
-    shifts (shared or mixed misalignment), output aliasing an input or not, kernel choice forced or automatic."""
+    """400 seeded random calls (MI_CCL_FUZZ_CASES / MI_CCL_FUZZ_SEED change that): dtype, op, input count (1..12),
+    1..3 destinations, element count, 16-bit mode, per-buffer element shifts (shared or mixed misalignment), output
+    aliasing an input or not, kernel choice forced or automatic."""
+    import os
     import torch
-    rng = np.random.default_rng(20260101)
-    for case in range(400):
+    rng = np.random.default_rng(int(os.environ.get("MI_CCL_FUZZ_SEED", "20260101")))
+    for case in range(int(os.environ.get("MI_CCL_FUZZ_CASES", "400"))):
         dtype = int(rng.integers(0, 12))
         op = int(rng.integers(0, 4))
         n = int(rng.integers(1, 13))
@@ -384,17 +386,31 @@ def test_randomised_calls_against_oracle(comp):
         else:
             out_holder, out_lo = to_dev(np.zeros(count + 2 * pad, np_t)), pad + shifts[n]
         variant = int(rng.choice([0, 0, 2, 8]))
+        m = int(rng.choice([1, 1, 2, 3]))
+        extra = []       # further destinations: (holder, first element), with the output's shift or one of their own
+        for _ in range(m - 1):
+            sh = shifts[alias if alias >= 0 else n] if same_shift else int(rng.integers(0, 16 // esz + 1))
+            extra.append((to_dev(np.zeros(count + 2 * pad, np_t)), pad + sh))
         comp.set_param("variant", variant)
         try:
-            comp.comp_reduce_n(dtype, op, ptrs, out_holder.data_ptr() + out_lo * esz, count, lp_mode=lp, bf16_impl=impl)
+            out_ptr = out_holder.data_ptr() + out_lo * esz
+            if m == 1:
+                comp.comp_reduce_n(dtype, op, ptrs, out_ptr, count, lp_mode=lp, bf16_impl=impl)
+            else:
+                comp.comp_reduce_write_n(dtype, op, ptrs, [out_ptr] + [h.data_ptr() + lo * esz for h, lo in extra], count,
+                                         lp_mode=lp, bf16_impl=impl)
             torch.cuda.synchronize()
         finally:
             comp.set_param("variant", 0)
         want = O.reduce_n(srcs, dtype, op, keep=keep, quirk_tail=quirk, bf16_impl=impl)
         got = to_host(out_holder, np_t)
-        what = (f"case {case}: dtype={O.DTYPE_NAMES[dtype]} op={O.OP_NAMES[op]} n={n} count={count} lp={lp} impl={impl} "
+        what = (f"case {case}: dtype={O.DTYPE_NAMES[dtype]} op={O.OP_NAMES[op]} n={n} m={m} count={count} lp={lp} impl={impl} "
                 f"shifts={shifts} alias={alias} variant={variant} kind={kind}")
         assert_same(got[out_lo:out_lo + count], want, dtype, what)
+        for h, lo in extra:
+            g2 = to_host(h, np_t)
+            assert_same(g2[lo:lo + count], want, dtype, what + " (further destination)")
+            assert (g2[:lo] == 0).all() and (g2[lo + count:] == 0).all(), what + ": wrote outside a further destination"
         if alias < 0:
             assert (got[:out_lo] == 0).all() and (got[out_lo + count:] == 0).all(), what + ": wrote outside the destination"
         else:
