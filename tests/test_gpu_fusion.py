@@ -146,3 +146,43 @@ def test_fusion_config_bf16_256_tensors(comp):
     with pytest.raises(comp.CclError):
         plan.reduce(O.SUM, d_t, d_peers, outs, lp_mode=comp.LP_KEEP_PRECISION | comp.LP_TAIL_QUIRK)
     plan.close()
+
+
+@pytest.mark.parametrize("dtype,op,n_peers,lp,impl,align", [
+    (O.BFLOAT16, O.SUM, 7, 1, 2, 256), (O.FLOAT16, O.MAX, 1, 0, 2, 256), (O.INT8, O.MIN, 7, 0, 2, 256),
+    (O.FLOAT64, O.PROD, 2, 0, 2, 256), (O.BFLOAT16, O.SUM, 5, 0, 2, 1), (O.INT32, O.SUM, 8, 0, 2, 256),
+    (O.FLOAT32, O.MIN, 4, 0, 2, 16), (O.BFLOAT16, O.PROD, 3, 0, 1, 256)])
+def test_fused_reduce_over_several_phases(comp, dtype, op, n_peers, lp, impl, align):
+    """The phased fused kernel with enough work that every LDS and register slot of a phase is used and a second
+    phase follows (a phase holds 22 items of 16 KiB per block: 92 MB chip-wide), for several element types,
+    operations and peer counts (more than 7 peers take the streaming kernel), against the oracle tensor by tensor."""
+    import torch
+    rng = np.random.default_rng(900 + dtype * 8 + n_peers)
+    esz = O.DTYPE_SIZE[dtype]
+    np_t = O.NP_STORAGE[dtype]
+    k = 37
+    target = 110 << 20                                   # payload bytes
+    w = rng.random(k) ** 3 + 0.01
+    counts = [max(1, int(target * x / w.sum()) // esz + int(rng.integers(0, 7))) for x in w]
+    counts[3] = 5
+    plan = comp.FusionPlan(counts, dtype, align)
+    offs, total = O.fusion_offsets(counts, esz, align)
+    nelem = (total + esz - 1) // esz
+    tensors = [make_inputs(rng, dtype, c, op, 1)[0] for c in counts]
+    peers = [make_inputs(rng, dtype, nelem, op, 1)[0] for _ in range(n_peers)]
+    d_t = [to_dev(t) for t in tensors]
+    d_p = [to_dev(p) for p in peers]
+    outs = [to_dev(np.zeros(c + 4, np_t)) for c in counts]
+    comp.set_param("variant", 8)
+    try:
+        plan.reduce(op, d_t, d_p, outs, lp_mode=lp, bf16_impl=impl)
+        torch.cuda.synchronize()
+    finally:
+        comp.set_param("variant", 0)
+    for i, c in enumerate(counts):
+        o = int(offs[i]) // esz
+        want = O.reduce_n([tensors[i]] + [p[o:o + c] for p in peers], dtype, op, keep=lp, bf16_impl=impl)
+        g = to_host(outs[i], np_t)
+        assert_same(g[:c], want, dtype, f"tensor {i} of {c} elements")
+        assert not g[c:].view(np.uint8).any(), "wrote past the tensor"
+    plan.close()
