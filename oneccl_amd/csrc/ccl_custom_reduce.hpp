@@ -30,10 +30,13 @@ struct src_table {
     const T* p[kMaxSrcs];
 };
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 u32x4_u __attribute__((aligned(1)));      // a 128-bit access that promises no alignment
 
-// 16 bytes per lane and input per step, two steps in flight; buffers aligned to 16 bytes
+// 16 bytes per lane and input per step, two steps in flight, from element `head` on (where dst reaches a 16-byte
+// boundary); the sources may sit at any other alignment
 template <class T, class F>
-__global__ void __launch_bounds__(kBlock) reduce_vec_kernel(src_table<T> src, int n, T* dst, uint64_t nvec, F f) {
+__global__ void __launch_bounds__(kBlock) reduce_vec_kernel(src_table<T> src, int n, T* dst, uint64_t head,
+                                                            uint64_t nvec, F f) {
     constexpr int VEC = 16 / sizeof(T);
     struct alignas(16) pack {
         T v[VEC];
@@ -43,28 +46,30 @@ __global__ void __launch_bounds__(kBlock) reduce_vec_kernel(src_table<T> src, in
     for (uint64_t i0 = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i0 < nvec; i0 += 2 * stride) {
         const uint64_t i1 = i0 + stride;
         const bool two = i1 < nvec;
-        pack a0 = __builtin_bit_cast(pack, __builtin_nontemporal_load((const u32x4*)src.p[0] + i0)), a1 = a0;
-        if (two) a1 = __builtin_bit_cast(pack, __builtin_nontemporal_load((const u32x4*)src.p[0] + i1));
+        pack a0 = __builtin_bit_cast(pack, __builtin_nontemporal_load((const u32x4_u*)(src.p[0] + head) + i0)), a1 = a0;
+        if (two) a1 = __builtin_bit_cast(pack, __builtin_nontemporal_load((const u32x4_u*)(src.p[0] + head) + i1));
         for (int j = 1; j < n; j++) {
-            pack x0 = __builtin_bit_cast(pack, __builtin_nontemporal_load((const u32x4*)src.p[j] + i0)), x1 = x0;
-            if (two) x1 = __builtin_bit_cast(pack, __builtin_nontemporal_load((const u32x4*)src.p[j] + i1));
+            pack x0 = __builtin_bit_cast(pack, __builtin_nontemporal_load((const u32x4_u*)(src.p[j] + head) + i0)), x1 = x0;
+            if (two) x1 = __builtin_bit_cast(pack, __builtin_nontemporal_load((const u32x4_u*)(src.p[j] + head) + i1));
 #pragma unroll
             for (int k = 0; k < VEC; k++) {
                 a0.v[k] = f(x0.v[k], a0.v[k]);
                 a1.v[k] = f(x1.v[k], a1.v[k]);
             }
         }
-        __builtin_nontemporal_store(__builtin_bit_cast(u32x4, a0), (u32x4*)dst + i0);
-        if (two) __builtin_nontemporal_store(__builtin_bit_cast(u32x4, a1), (u32x4*)dst + i1);
+        __builtin_nontemporal_store(__builtin_bit_cast(u32x4, a0), (u32x4_u*)(dst + head) + i0);
+        if (two) __builtin_nontemporal_store(__builtin_bit_cast(u32x4, a1), (u32x4_u*)(dst + head) + i1);
     }
 }
 
-// any alignment: one element per lane; also the count % VEC tail of the vector form (first element `begin`)
+// one element per lane: the elements before the first vector and after the last one (elements [0, head) and
+// [begin, count))
 template <class T, class F>
-__global__ void __launch_bounds__(kBlock) reduce_elem_kernel(src_table<T> src, int n, T* dst, uint64_t begin,
-                                                             uint64_t count, F f) {
+__global__ void __launch_bounds__(kBlock) reduce_elem_kernel(src_table<T> src, int n, T* dst, uint64_t head,
+                                                             uint64_t begin, uint64_t count, F f) {
     const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-    for (uint64_t i = begin + (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < count; i += stride) {
+    for (uint64_t t = (uint64_t)blockIdx.x * kBlock + threadIdx.x; t < head + (count - begin); t += stride) {
+        const uint64_t i = t < head ? t : begin + (t - head);
         T a = src.p[0][i];
         for (int j = 1; j < n; j++) a = f(src.p[j][i], a);
         dst[i] = a;
@@ -93,26 +98,27 @@ ccl::status ccl_custom_reduce_n(ccl_sched* sched, const std::vector<const T*>& s
     if (count == 0) return ccl::status::success;
     if (srcs.empty() || srcs.size() > (size_t)kMaxSrcs || !out) throw ccl::exception("ccl_custom_reduce_n: bad arguments");
     src_table<T> t{};
-    bool aligned = ((uintptr_t)out & 15u) == 0;
     for (size_t j = 0; j < srcs.size(); j++) {
         if (!srcs[j]) throw ccl::exception("ccl_custom_reduce_n: null source");
         t.p[j] = srcs[j];
-        aligned = aligned && ((uintptr_t)srcs[j] & 15u) == 0;
     }
     hipStream_t stream = (hipStream_t)(sched ? sched->stream : nullptr);
     const int n = (int)srcs.size();
     constexpr uint64_t VEC = 16 / sizeof(T);
-    const uint64_t nvec = aligned ? count / VEC : 0;
+    // the vectors start where the output reaches a 16-byte boundary
+    const uintptr_t mis = (uintptr_t)out & 15u;
+    uint64_t head = (mis % sizeof(T)) == 0 ? ((16u - mis) & 15u) / sizeof(T) : 0;
+    if (head > count) head = count;
+    const uint64_t nvec = (count - head) / VEC;
     const uint64_t max_grid = (uint64_t)cu_count() * 8;
     if (nvec) {
         uint64_t blocks = (nvec + 2 * kBlock - 1) / (2 * kBlock);
         hipLaunchKernelGGL((reduce_vec_kernel<T, F>), dim3((unsigned)(blocks < max_grid ? blocks : max_grid)), dim3(kBlock),
-                           0, stream, t, n, out, nvec, f);
+                           0, stream, t, n, out, head, nvec, f);
     }
-    if (nvec * VEC < count) {
-        uint64_t rest = count - nvec * VEC, blocks = (rest + kBlock - 1) / kBlock;
-        hipLaunchKernelGGL((reduce_elem_kernel<T, F>), dim3((unsigned)(blocks < max_grid ? blocks : max_grid)), dim3(kBlock),
-                           0, stream, t, n, out, nvec * VEC, (uint64_t)count, f);
+    if (head + nvec * VEC < count || head) {
+        hipLaunchKernelGGL((reduce_elem_kernel<T, F>), dim3(1), dim3(kBlock), 0, stream, t, n, out, head,
+                           head + nvec * VEC, (uint64_t)count, f);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) throw ccl::exception(std::string("ccl_custom_reduce_n: ") + hipGetErrorString(e));

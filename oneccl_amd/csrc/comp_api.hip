@@ -200,12 +200,13 @@ static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void
 // ---------------------------------------------------------------------------------------------------
 // copy and converter kernels
 
+// Vectors from the output's first 16-byte boundary on; the input is read as loose vectors (any alignment).
 template <bool NT>
 __global__ void __launch_bounds__(kBlock)
 copy_kernel(const unsigned char* in, unsigned char* out, uint32_t head, uint64_t nvec, uint32_t tail) {
     constexpr int UNROLL = 4;
     constexpr uint64_t kTile = (uint64_t)kBlock * UNROLL;
-    const u32x4* s = (const u32x4*)(in + head);
+    const u32x4_u* s = (const u32x4_u*)(in + head);
     u32x4* d = (u32x4*)(out + head);
     const uint64_t ntiles = (nvec + kTile - 1) / kTile;
     for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
@@ -215,7 +216,7 @@ copy_kernel(const unsigned char* in, unsigned char* out, uint32_t head, uint64_t
         for (int u = 0; u < UNROLL; u++) {
             const uint64_t i = base + (uint64_t)u * kBlock;
             if (i < nvec)
-                x[u] = NT ? __builtin_nontemporal_load(s + i) : s[i];
+                x[u] = NT ? ld_loose(s + i) : *(s + i);
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
@@ -233,11 +234,6 @@ copy_kernel(const unsigned char* in, unsigned char* out, uint32_t head, uint64_t
         uint64_t i = (t < head) ? t : (uint64_t)head + nvec * 16 + (t - head);
         out[i] = in[i];
     }
-}
-
-__global__ void __launch_bounds__(kBlock) copy_bytes_kernel(const unsigned char* in, unsigned char* out, uint64_t n) {
-    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) out[i] = in[i];
 }
 
 // fp32 -> bf16, four elements per lane; elements at or beyond rne_limit are truncated
@@ -372,8 +368,7 @@ int mi_ccl_comp_copy(const void* in, void* out, size_t bytes, int use_nontempora
     const uintptr_t mis = (uintptr_t)out & 15u;
     // very large copies go through the one-input reduce (a copy for plain types), whose phased form separates
     // reads from writes; below that the plain copy kernel is as fast
-    if (((uintptr_t)in & 15u) == mis && t.sync && t.variant == 0 &&
-        2 * (uint64_t)bytes >= 25 * (uint64_t)t.phased_min_bytes) {
+    if (t.sync && t.variant == 0 && 2 * (uint64_t)bytes >= 25 * (uint64_t)t.phased_min_bytes) {
         LaunchArgs a;
         const void* srcs[1] = { in };
         a.srcs = srcs;
@@ -384,12 +379,6 @@ int mi_ccl_comp_copy(const void* in, void* out, size_t bytes, int use_nontempora
         a.stream = (hipStream_t)stream;
         a.tune = t;
         return status_of(launch_reduce<U8Traits>(a));
-    }
-    if (((uintptr_t)in & 15u) != mis) {
-        int grid = grid_for((bytes + kBlock - 1) / kBlock, t);
-        hipLaunchKernelGGL(copy_bytes_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream,
-                           (const unsigned char*)in, (unsigned char*)out, (uint64_t)bytes);
-        return status_of(hipGetLastError());
     }
     uint64_t head = mis ? 16u - mis : 0;
     if (head > bytes)

@@ -42,56 +42,36 @@ struct FusionLaunchArgs {
     Tuning tune;
 };
 
-// Copy n <= kFusionChunk bytes with one block.
+// Copy n <= kFusionChunk bytes with one block: vectors from the destination's first 16-byte boundary on, whatever
+// the source's alignment is.
 __device__ __forceinline__ void copy_span(const unsigned char* src, unsigned char* dst, uint32_t n) {
     const uint32_t tid = threadIdx.x;
-    const uint32_t d = (uint32_t)((uintptr_t)src ^ (uintptr_t)dst);
-    if ((d & 15u) == 0) {
-        uint32_t head = (uint32_t)(-(intptr_t)src) & 15u;
-        if (head > n) head = n;
-        const uint32_t nvec = (n - head) >> 4, tail = n - head - (nvec << 4);
-        const u32x4* s = (const u32x4*)(src + head);
-        u32x4* o = (u32x4*)(dst + head);
-        u32x4 x[4];
-#pragma unroll
-        for (int u = 0; u < 4; u++)
-            if (tid + u * kBlock < nvec) x[u] = ld_stream(s + tid + u * kBlock);
-#pragma unroll
-        for (int u = 0; u < 4; u++)
-            if (tid + u * kBlock < nvec) st_stream(o + tid + u * kBlock, x[u]);
-        if (tid < head + tail) {
-            uint32_t i = (tid < head) ? tid : head + (nvec << 4) + (tid - head);
-            dst[i] = src[i];
-        }
-        return;
-    }
-    // source and destination disagree modulo 16: move the widest unit both can be aligned to
-    const uint32_t unit = (d & 1u) ? 1u : (d & 2u) ? 2u : (d & 4u) ? 4u : 8u;
-    uint32_t head = (uint32_t)(-(intptr_t)src) & (unit - 1u);
+    uint32_t head = (uint32_t)(-(intptr_t)dst) & 15u;
     if (head > n) head = n;
-    const uint32_t nu = (n - head) / unit, tail = n - head - nu * unit;
-    if (unit == 8) {
-        const uint64_t* s = (const uint64_t*)(src + head);
-        uint64_t* o = (uint64_t*)(dst + head);
-        for (uint32_t i = tid; i < nu; i += kBlock) o[i] = s[i];
-    }
-    else if (unit == 4) {
-        const uint32_t* s = (const uint32_t*)(src + head);
-        uint32_t* o = (uint32_t*)(dst + head);
-        for (uint32_t i = tid; i < nu; i += kBlock) o[i] = s[i];
-    }
-    else if (unit == 2) {
-        const uint16_t* s = (const uint16_t*)(src + head);
-        uint16_t* o = (uint16_t*)(dst + head);
-        for (uint32_t i = tid; i < nu; i += kBlock) o[i] = s[i];
-    }
-    else {
-        for (uint32_t i = tid; i < nu; i += kBlock) dst[head + i] = src[head + i];
-    }
+    const uint32_t nvec = (n - head) >> 4, tail = n - head - (nvec << 4);
+    const u32x4_u* s = (const u32x4_u*)(src + head);
+    u32x4_u* o = (u32x4_u*)(dst + head);
+    u32x4 x[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+        if (tid + u * kBlock < nvec) x[u] = ld_loose(s + tid + u * kBlock);
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+        if (tid + u * kBlock < nvec) st_loose(o + tid + u * kBlock, x[u]);
     if (tid < head + tail) {
-        uint32_t i = (tid < head) ? tid : head + nu * unit + (tid - head);
+        uint32_t i = (tid < head) ? tid : head + (nvec << 4) + (tid - head);
         dst[i] = src[i];
     }
+}
+
+// Elements of a tensor chunk before its output's first 16-byte boundary, where its vectors start (none when the
+// output is not even aligned to its element size).  Inputs that disagree with the output modulo 16 bytes -- the peers'
+// copies of a tensor behind an odd-sized one in a tightly packed fusion buffer -- are read as loose vectors; aligning
+// the peers and storing loose vectors instead measures 6 % slower.
+template <uint32_t ES>
+__device__ __forceinline__ uint32_t fusion_head(const void* out) {
+    const uint32_t mis = (uint32_t)(uintptr_t)out & 15u;
+    return (mis % ES) == 0 ? ((16u - mis) & 15u) / ES : 0;
 }
 
 // out_t[i] = own_t[i] OP peer_0[off_t + i] OP ... : one pass, same arithmetic as reduce_multi_kernel
@@ -111,54 +91,41 @@ fusion_reduce_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers
         const unsigned char* a = (const unsigned char*)own.p[w.t - t0] + lo;
         unsigned char* o = (unsigned char*)out.p[w.t - t0] + lo;
         const uint64_t poff = off[w.t] + lo;
-        // all streams congruent modulo 16?
-        uint32_t mis = (uint32_t)(uintptr_t)a & 15u;
-        bool same = (((uint32_t)(uintptr_t)o & 15u) == mis);
-        for (int j = 0; j < n_peers; j++)
-            same = same && ((((uint32_t)(uintptr_t)peers.p[j] + (uint32_t)poff) & 15u) == mis);
         const uint32_t nelem = nb / ES;
-        if (same) {
-            uint32_t head = mis ? (16u - mis) / ES : 0;
+        {
+            uint32_t head = fusion_head<ES>(o);
             if (head > nelem) head = nelem;
             const uint32_t nvec = (nelem - head) / TR::VEC, tail = nelem - head - nvec * TR::VEC;
             Accs<TR> acc[4];
-            const u32x4* s0 = (const u32x4*)(a + head * ES);
+            const u32x4_u* s0 = (const u32x4_u*)(a + head * ES);
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 const uint32_t i = tid + u * kBlock;
-                acc[u] = vec_init<TR>((i < nvec) ? ld_stream(s0 + i) : u32x4{ 0, 0, 0, 0 });
+                acc[u] = vec_init<TR>((i < nvec) ? ld_loose(s0 + i) : u32x4{ 0, 0, 0, 0 });
             }
             for (int j = 0; j < n_peers; j++) {
-                const u32x4* sj = (const u32x4*)((const unsigned char*)peers.p[j] + poff + head * ES);
+                const u32x4_u* sj = (const u32x4_u*)((const unsigned char*)peers.p[j] + poff + head * ES);
                 u32x4 x[4];
 #pragma unroll
                 for (int u = 0; u < 4; u++) {
                     const uint32_t i = tid + u * kBlock;
-                    x[u] = (i < nvec) ? ld_stream(sj + i) : u32x4{ 0, 0, 0, 0 };
+                    x[u] = (i < nvec) ? ld_loose(sj + i) : u32x4{ 0, 0, 0, 0 };
                 }
 #pragma unroll
                 for (int u = 0; u < 4; u++) vec_step<TR, OP>(x[u], acc[u]);
             }
-            u32x4* d = (u32x4*)(o + head * ES);
+            u32x4_u* d = (u32x4_u*)(o + head * ES);
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 const uint32_t i = tid + u * kBlock;
-                if (i < nvec) st_stream(d + i, vec_finish<TR>(acc[u]));
+                if (i < nvec) st_loose(d + i, vec_finish<TR>(acc[u]));
             }
             if (tid < head + tail) {
                 const uint32_t i = (tid < head) ? tid : head + nvec * TR::VEC + (tid - head);
-                typename TR::acc_t r = TR::init(((const E*)a)[i]);
+                typename TR::acc_t r = TR::init(ld_elem<E>(a, i));
                 for (int j = 0; j < n_peers; j++)
-                    r = TR::template step<OP>(((const E*)((const unsigned char*)peers.p[j] + poff))[i], r);
-                ((E*)o)[i] = TR::finish(r);
-            }
-        }
-        else {
-            for (uint32_t i = tid; i < nelem; i += kBlock) {
-                typename TR::acc_t r = TR::init(((const E*)a)[i]);
-                for (int j = 0; j < n_peers; j++)
-                    r = TR::template step<OP>(((const E*)((const unsigned char*)peers.p[j] + poff))[i], r);
-                ((E*)o)[i] = TR::finish(r);
+                    r = TR::template step<OP>(ld_elem<E>((const unsigned char*)peers.p[j] + poff, i), r);
+                st_elem<E>(o, i, TR::finish(r));
             }
         }
     }
@@ -175,8 +142,8 @@ struct FusionPhaseRegs {
 // The same reduce with reads and writes separated in time (see reduce_multi_phased_kernel): each block takes kPhaseU / 2
 // work items per phase (an item is 16 KiB of one tensor = two vectors per lane), keeps their results in LDS, and
 // writes them after the chip-wide barrier.  Item (phase, slot, block) = phase * slots * blocks + slot * blocks + block.
-// Head/tail elements of tensors that do not start on a 16-byte boundary, and tensors whose streams disagree modulo
-// 16 bytes, are written directly (they are a few bytes, or a rare layout).  NT = 1 + number of peers.
+// Head/tail elements of chunks whose output does not start on a 16-byte boundary are written directly (they are a
+// few bytes).  NT = 1 + number of peers.
 template <class TR, int OP, int NT>
 __global__ void __launch_bounds__(kPhaseBlock)
 fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, const uint64_t* off, const uint64_t* bytes,
@@ -204,6 +171,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
         // item -> tensor tables -> pointers is walked once, for all items at once, instead of once per item.
         uint64_t d_a = 0, d_o = 0, d_poff = 0;
         uint32_t d_nb = 0;      // 0: no item in this slot
+        uint32_t d_head = 0;    // elements before the item's first vector
         if (lane < (uint32_t)SLOTS) {
             const uint64_t it = p0 + (uint64_t)lane * gridDim.x + blockIdx.x;
             if (it < nitems) {
@@ -214,6 +182,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                 d_a = (uint64_t)(uintptr_t)own.p[w.t - t0] + lo;
                 d_o = (uint64_t)(uintptr_t)out.p[w.t - t0] + lo;
                 d_poff = off[w.t] + lo;
+                d_head = fusion_head<ES>((const void*)(uintptr_t)d_o);
             }
         }
         for (int k = 0; k < SLOTS; k++) {
@@ -222,20 +191,15 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
             const unsigned char* a = (const unsigned char*)(uintptr_t)__shfl(d_a, k, 64);
             unsigned char* o = (unsigned char*)(uintptr_t)__shfl(d_o, k, 64);
             const uint64_t poff = __shfl(d_poff, k, 64);
-            const uint32_t mis = (uint32_t)(uintptr_t)a & 15u;
-            bool same = (((uint32_t)(uintptr_t)o & 15u) == mis);
-#pragma unroll
-            for (int j = 0; j < NP; j++)
-                same = same && ((((uint32_t)(uintptr_t)peers.p[j] + (uint32_t)poff) & 15u) == mis);
             const uint32_t nelem = nb / ES;
-            if (same) {
-                uint32_t head = mis ? (16u - mis) / ES : 0;
+            {
+                uint32_t head = __shfl(d_head, k, 64);
                 if (head > nelem) head = nelem;
                 const uint32_t nvec = (nelem - head) / TR::VEC, tail = nelem - head - nvec * TR::VEC;
-                const u32x4* s[NT];
-                s[0] = (const u32x4*)(a + head * ES);
+                const u32x4_u* s[NT];
+                s[0] = (const u32x4_u*)(a + head * ES);
 #pragma unroll
-                for (int j = 0; j < NP; j++) s[j + 1] = (const u32x4*)((const unsigned char*)peers.p[j] + poff + head * ES);
+                for (int j = 0; j < NP; j++) s[j + 1] = (const u32x4_u*)((const unsigned char*)peers.p[j] + poff + head * ES);
                 const uint64_t idx[2] = { tid, tid + (uint32_t)kPhaseBlock };
                 u32x4 res[2];
                 if constexpr (TR::VEC * NT <= 64) {
@@ -265,20 +229,11 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                 }
                 if (tid < head + tail) {
                     const uint32_t i = (tid < head) ? tid : head + nvec * TR::VEC + (tid - head);
-                    typename TR::acc_t r = TR::init(((const E*)a)[i]);
+                    typename TR::acc_t r = TR::init(ld_elem<E>(a, i));
 #pragma unroll
                     for (int j = 0; j < NP; j++)
-                        r = TR::template step<OP>(((const E*)((const unsigned char*)peers.p[j] + poff))[i], r);
-                    ((E*)o)[i] = TR::finish(r);
-                }
-            }
-            else {
-                for (uint32_t i = tid; i < nelem; i += kPhaseBlock) {
-                    typename TR::acc_t r = TR::init(((const E*)a)[i]);
-#pragma unroll
-                    for (int j = 0; j < NP; j++)
-                        r = TR::template step<OP>(((const E*)((const unsigned char*)peers.p[j] + poff))[i], r);
-                    ((E*)o)[i] = TR::finish(r);
+                        r = TR::template step<OP>(ld_elem<E>((const unsigned char*)peers.p[j] + poff, i), r);
+                    st_elem<E>(o, i, TR::finish(r));
                 }
             }
         }
@@ -286,20 +241,13 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
         for (int k = 0; k < SLOTS; k++) {
             const uint32_t nb = __shfl(d_nb, k, 64);
             if (nb == 0) break;
-            const unsigned char* a = (const unsigned char*)(uintptr_t)__shfl(d_a, k, 64);
             unsigned char* o = (unsigned char*)(uintptr_t)__shfl(d_o, k, 64);
-            const uint64_t poff = __shfl(d_poff, k, 64);
-            const uint32_t mis = (uint32_t)(uintptr_t)a & 15u;
-            bool same = (((uint32_t)(uintptr_t)o & 15u) == mis);
-#pragma unroll
-            for (int j = 0; j < NP; j++)
-                same = same && ((((uint32_t)(uintptr_t)peers.p[j] + (uint32_t)poff) & 15u) == mis);
-            if (same) {
+            {
                 const uint32_t nelem = nb / ES;
-                uint32_t head = mis ? (16u - mis) / ES : 0;
+                uint32_t head = __shfl(d_head, k, 64);
                 if (head > nelem) head = nelem;
                 const uint32_t nvec = (nelem - head) / TR::VEC;
-                u32x4* d = (u32x4*)(o + head * ES);
+                u32x4_u* d = (u32x4_u*)(o + head * ES);
                 u32x4 v0 = { 0, 0, 0, 0 }, v1 = v0;
                 if (k < S) {
                     v0 = stage[(2 * k) * kPhaseBlock + tid];
@@ -314,8 +262,8 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                     }
 #undef MI_RS_GET
                 }
-                if (tid < nvec) st_stream(d + tid, v0);
-                if (tid + kPhaseBlock < nvec) st_stream(d + tid + kPhaseBlock, v1);
+                if (tid < nvec) st_loose(d + tid, v0);
+                if (tid + kPhaseBlock < nvec) st_loose(d + tid + kPhaseBlock, v1);
             }
         }
         if (p0 + per_phase < nitems) phase_barrier(ps, ++gen, give_up);

@@ -426,8 +426,26 @@ __device__ __forceinline__ u32x4 vec_finish(const Accs<TR>& a) {
     return VecOps<TR>::finish(a);
 }
 
-__device__ __forceinline__ u32x4 ld_stream(const u32x4* p) { return __builtin_nontemporal_load(p); }
-__device__ __forceinline__ void st_stream(u32x4* p, u32x4 v) { __builtin_nontemporal_store(v, p); }
+// Streaming 128-bit accesses through pointers that promise no alignment (the instruction is the same one).  The
+// memory pipeline takes a vector access at any byte address (a wave's 1 KiB then touches one cache line more), so
+// buffers that disagree modulo 16 bytes -- tensors behind an odd-sized one in a tightly packed fusion buffer, a
+// peer's chunk at an odd offset -- still move as vectors.  The host starts the vectors on a 16-byte boundary of as
+// many buffers as it can.
+typedef u32x4 u32x4_u __attribute__((aligned(1)));
+__device__ __forceinline__ u32x4 ld_loose(const u32x4_u* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void st_loose(u32x4_u* p, u32x4 v) { __builtin_nontemporal_store(v, p); }
+template <class E>
+struct __attribute__((packed)) LooseElem {
+    E v;
+};
+template <class E>
+__device__ __forceinline__ E ld_elem(const void* p, uint64_t i) {
+    return ((const LooseElem<E>*)p)[i].v;
+}
+template <class E>
+__device__ __forceinline__ void st_elem(void* p, uint64_t i, E x) {
+    ((LooseElem<E>*)p)[i].v = x;
+}
 
 // The count % VEC elements after the last full vector and the elements before the first aligned one:
 // at most 2*(VEC-1) <= 30 elements, one per lane of the first wave of block 0.
@@ -438,9 +456,9 @@ __device__ __forceinline__ void reduce_edges(const SRC& src, int n, void* dst, u
     uint32_t t = threadIdx.x;
     if (t < head + tail) {
         uint64_t i = (t < head) ? t : (uint64_t)head + nvec * TR::VEC + (t - head);
-        typename TR::acc_t a = TR::init(((const E*)src.p[0])[i]);
-        for (int j = 1; j < n; j++) a = TR::template step<OP>(((const E*)src.p[j])[i], a);
-        ((E*)dst)[i] = TR::finish(a);
+        typename TR::acc_t a = TR::init(ld_elem<E>(src.p[0], i));
+        for (int j = 1; j < n; j++) a = TR::template step<OP>(ld_elem<E>(src.p[j], i), a);
+        st_elem<E>(dst, i, TR::finish(a));
     }
 }
 
@@ -471,10 +489,10 @@ reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr uint64_t kTile = (uint64_t)kBlock * UNROLL;
-    const u32x4* s[N];
+    const u32x4_u* s[N];
 #pragma unroll
-    for (int j = 0; j < N; j++) s[j] = (const u32x4*)((const E*)src.p[j] + head);
-    u32x4* d = (u32x4*)((E*)dst + head);
+    for (int j = 0; j < N; j++) s[j] = (const u32x4_u*)((const unsigned char*)src.p[j] + head * sizeof(E));
+    u32x4_u* d = (u32x4_u*)((unsigned char*)dst + head * sizeof(E));
     const uint64_t ntiles = (nvec + kTile - 1) / kTile;
 
     for (TileIter it(ntiles, xcd_chunked); it.tile < it.end; it.tile += it.stride) {
@@ -484,13 +502,13 @@ reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint
 #pragma unroll
             for (int j = 0; j < N; j++)
 #pragma unroll
-                for (int u = 0; u < UNROLL; u++) x[j][u] = ld_stream(s[j] + base + (uint64_t)u * kBlock);
+                for (int u = 0; u < UNROLL; u++) x[j][u] = ld_loose(s[j] + base + (uint64_t)u * kBlock);
 #pragma unroll
             for (int u = 0; u < UNROLL; u++) {
                 Accs<TR> a = vec_init<TR>(x[0][u]);
 #pragma unroll
                 for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j][u], a);
-                st_stream(d + base + (uint64_t)u * kBlock, vec_finish<TR>(a));
+                st_loose(d + base + (uint64_t)u * kBlock, vec_finish<TR>(a));
             }
         }
         else {
@@ -500,11 +518,11 @@ reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint
                 if (i < nvec) {
                     u32x4 x[N];
 #pragma unroll
-                    for (int j = 0; j < N; j++) x[j] = ld_stream(s[j] + i);
+                    for (int j = 0; j < N; j++) x[j] = ld_loose(s[j] + i);
                     Accs<TR> a = vec_init<TR>(x[0]);
 #pragma unroll
                     for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j], a);
-                    st_stream(d + i, vec_finish<TR>(a));
+                    st_loose(d + i, vec_finish<TR>(a));
                 }
             }
         }
@@ -574,12 +592,12 @@ __device__ __forceinline__ void phase_barrier(PhaseSync* ps, unsigned gen, bool&
 // eight 128-bit loads in flight whatever N is.  Callers branch around this (a real branch keeps the compiler
 // from hoisting the loads of later steps, which would spill).
 template <class TR, int OP, int N, int G>
-__device__ __forceinline__ void reduce_group(const u32x4* const (&s)[N], const uint64_t (&idx)[G], u32x4 (&out)[G]) {
+__device__ __forceinline__ void reduce_group(const u32x4_u* const (&s)[N], const uint64_t (&idx)[G], u32x4 (&out)[G]) {
     u32x4 x[G][N];
 #pragma unroll
     for (int g = 0; g < G; g++)
 #pragma unroll
-        for (int j = 0; j < N; j++) x[g][j] = ld_stream(s[j] + idx[g]);
+        for (int j = 0; j < N; j++) x[g][j] = ld_loose(s[j] + idx[g]);
 #pragma unroll
     for (int g = 0; g < G; g++) {
         Accs<TR> a = vec_init<TR>(x[g][0]);
@@ -591,7 +609,7 @@ __device__ __forceinline__ void reduce_group(const u32x4* const (&s)[N], const u
 
 // the same for a group that may reach past the end of the buffer: slots at or beyond nvec are left alone
 template <class TR, int OP, int N, int G>
-__device__ __forceinline__ void reduce_group_guarded(const u32x4* const (&s)[N], const uint64_t (&idx)[G],
+__device__ __forceinline__ void reduce_group_guarded(const u32x4_u* const (&s)[N], const uint64_t (&idx)[G],
                                                      uint64_t nvec, u32x4 (&out)[G]) {
     if (idx[G - 1] < nvec) {
         reduce_group<TR, OP, N, G>(s, idx, out);
@@ -609,19 +627,6 @@ __device__ __forceinline__ void reduce_group_guarded(const u32x4* const (&s)[N],
     }
 }
 
-// One element per lane, any alignment of the buffers relative to each other.
-template <class TR, int OP>
-__global__ void __launch_bounds__(kBlock)
-reduce_elem_kernel(SrcTable src, int n, void* dst, uint64_t count) {
-    typedef typename TR::elem_t E;
-    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < count; i += stride) {
-        typename TR::acc_t a = TR::init(((const E*)src.p[0])[i]);
-        for (int j = 1; j < n; j++) a = TR::template step<OP>(((const E*)src.p[j])[i], a);
-        ((E*)dst)[i] = TR::finish(a);
-    }
-}
-
 // ---------------------------------------------------------------------------------------------------
 // Run-time counts of inputs (up to 64) and destinations (up to 16): the reduced vector is stored to each of m buffers (the reference's allreduce_kernel stores
 // to the own and to the peer's output, kernels.cl:190-217; with one input this is write_monolithic_kernel_N,
@@ -633,14 +638,14 @@ __device__ __forceinline__ void reduce_rt_tile(const SrcTable& src, int n, uint3
                                                uint64_t nvec, u32x4 (&out)[UNROLL]) {
     typedef typename TR::elem_t E;
     Accs<TR> a[UNROLL];
-    const u32x4* s0 = (const u32x4*)((const E*)src.p[0] + head);
+    const u32x4_u* s0 = (const u32x4_u*)((const unsigned char*)src.p[0] + head * sizeof(E));
 #pragma unroll
-    for (int u = 0; u < UNROLL; u++) a[u] = vec_init<TR>((idx[u] < nvec) ? ld_stream(s0 + idx[u]) : u32x4{ 0, 0, 0, 0 });
+    for (int u = 0; u < UNROLL; u++) a[u] = vec_init<TR>((idx[u] < nvec) ? ld_loose(s0 + idx[u]) : u32x4{ 0, 0, 0, 0 });
     for (int j = 1; j < n; j++) {
-        const u32x4* sj = (const u32x4*)((const E*)src.p[j] + head);
+        const u32x4_u* sj = (const u32x4_u*)((const unsigned char*)src.p[j] + head * sizeof(E));
         u32x4 x[UNROLL];
 #pragma unroll
-        for (int u = 0; u < UNROLL; u++) x[u] = (idx[u] < nvec) ? ld_stream(sj + idx[u]) : u32x4{ 0, 0, 0, 0 };
+        for (int u = 0; u < UNROLL; u++) x[u] = (idx[u] < nvec) ? ld_loose(sj + idx[u]) : u32x4{ 0, 0, 0, 0 };
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) vec_step<TR, OP>(x[u], a[u]);
     }
@@ -655,10 +660,10 @@ __device__ __forceinline__ void reduce_multi_edges(const SrcTable& src, int n, c
     uint32_t t = threadIdx.x;
     if (t < head + tail) {
         uint64_t i = (t < head) ? t : (uint64_t)head + nvec * TR::VEC + (t - head);
-        typename TR::acc_t a = TR::init(((const E*)src.p[0])[i]);
-        for (int j = 1; j < n; j++) a = TR::template step<OP>(((const E*)src.p[j])[i], a);
+        typename TR::acc_t a = TR::init(ld_elem<E>(src.p[0], i));
+        for (int j = 1; j < n; j++) a = TR::template step<OP>(ld_elem<E>(src.p[j], i), a);
         const E r = TR::finish(a);
-        for (int k = 0; k < m; k++) ((E*)dst.p[k])[i] = r;
+        for (int k = 0; k < m; k++) st_elem<E>(dst.p[k], i, r);
     }
 }
 
@@ -677,10 +682,10 @@ reduce_multi_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uin
         for (int u = 0; u < UNROLL; u++) idx[u] = it.tile * kTile + threadIdx.x + (uint64_t)u * kBlock;
         reduce_rt_tile<TR, OP, UNROLL>(src, n, head, idx, nvec, v);
         for (int k = 0; k < m; k++) {
-            u32x4* d = (u32x4*)((E*)dst.p[k] + head);
+            u32x4_u* d = (u32x4_u*)((unsigned char*)dst.p[k] + head * sizeof(E));
 #pragma unroll
             for (int u = 0; u < UNROLL; u++)
-                if (idx[u] < nvec) st_stream(d + idx[u], v[u]);
+                if (idx[u] < nvec) st_loose(d + idx[u], v[u]);
         }
     }
     if (blockIdx.x == 0 && (head | tail)) reduce_multi_edges<TR, OP>(src, n, dst, m, head, nvec, tail);
@@ -741,33 +746,20 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
         }
         phase_barrier(ps, ++gen, give_up);
         for (int k = 0; k < m; k++) {
-            u32x4* d = (u32x4*)((E*)dst.p[k] + head);
+            u32x4_u* d = (u32x4_u*)((unsigned char*)dst.p[k] + head * sizeof(E));
 #pragma unroll
             for (int u = 0; u < G * RG; u++) {
                 const uint64_t i = pos(p0, u);
-                if (i < nvec) st_stream(d + i, rs[u]);
+                if (i < nvec) st_loose(d + i, rs[u]);
             }
             for (int u = 0; u < kPhaseU; u++) {
                 const uint64_t i = pos(p0, G * RG + u);
-                if (i < nvec) st_stream(d + i, stage[u * kPhaseBlock + threadIdx.x]);
+                if (i < nvec) st_loose(d + i, stage[u * kPhaseBlock + threadIdx.x]);
             }
         }
         if (p0 + per_phase < nvec) phase_barrier(ps, ++gen, give_up);
     }
     if (blockIdx.x == 0 && (head | tail)) reduce_multi_edges<TR, OP>(src, n, dst, m, head, nvec, tail);
-}
-
-template <class TR, int OP>
-__global__ void __launch_bounds__(kBlock)
-reduce_multi_elem_kernel(SrcTable src, int n, DstTable dst, int m, uint64_t count) {
-    typedef typename TR::elem_t E;
-    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < count; i += stride) {
-        typename TR::acc_t a = TR::init(((const E*)src.p[0])[i]);
-        for (int j = 1; j < n; j++) a = TR::template step<OP>(((const E*)src.p[j])[i], a);
-        const E r = TR::finish(a);
-        for (int k = 0; k < m; k++) ((E*)dst.p[k])[i] = r;
-    }
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -834,6 +826,21 @@ inline bool wants_phased(const LaunchArgs& a, uint64_t nvec) {
     return 2 * traffic >= (uint64_t)a.tune.phased_min_bytes * halves;
 }
 
+// Elements before the first vector: the vectors start on a 16-byte boundary of as many buffers as possible (of the
+// first destination among equals; eight aligned inputs and a loose output measure 6.6 TB/s where the reverse measures
+// 5.2).  The buffers that disagree are read and written as loose vectors.  No head when that boundary is not a
+// multiple of the element size.
+template <class E>
+inline uint64_t vector_head(const LaunchArgs& a) {
+    int votes[16] = { 0 };
+    for (int j = 0; j < a.n; j++) votes[(uintptr_t)a.srcs[j] & 15u]++;
+    for (int k = 0; k < a.m; k++) votes[(uintptr_t)(a.dsts ? a.dsts[k] : a.dst) & 15u]++;
+    uintptr_t mis = (uintptr_t)(a.dsts ? a.dsts[0] : a.dst) & 15u;
+    for (uintptr_t c = 0; c < 16; c++)
+        if (votes[c] > votes[mis]) mis = c;
+    return (mis % sizeof(E)) == 0 ? ((16u - mis) & 15u) / sizeof(E) : 0;
+}
+
 template <class TR, int OP>
 inline hipError_t launch_multi_op(const LaunchArgs& a) {
     typedef typename TR::elem_t E;
@@ -842,17 +849,7 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
     DstTable d;
     for (int j = 0; j < a.n; j++) s.p[j] = a.srcs[j];
     for (int k = 0; k < a.m; k++) d.p[k] = a.dsts ? a.dsts[k] : a.dst;
-    const uintptr_t mis = (uintptr_t)d.p[0] & 15u;
-    bool same = true;
-    for (int j = 0; j < a.n; j++) same = same && (((uintptr_t)a.srcs[j] & 15u) == mis);
-    for (int k = 0; k < a.m; k++) same = same && (((uintptr_t)d.p[k] & 15u) == mis);
-    if (!same || (mis % sizeof(E)) != 0) {
-        int grid = grid_for((a.count + kBlock - 1) / kBlock, a.tune);
-        hipLaunchKernelGGL((reduce_multi_elem_kernel<TR, OP>), dim3(grid), dim3(kBlock), 0, a.stream, s, a.n, d, a.m,
-                           (uint64_t)a.count);
-        return hipGetLastError();
-    }
-    uint64_t head = mis ? (16u - mis) / sizeof(E) : 0;
+    uint64_t head = vector_head<E>(a);
     if (head > a.count) head = a.count;
     const uint64_t nvec = (a.count - head) / VEC;
     const uint32_t tail = (uint32_t)(a.count - head - nvec * VEC);
@@ -875,20 +872,7 @@ inline hipError_t launch_op(const LaunchArgs& a) {
     typedef typename TR::elem_t E;
     constexpr uint32_t VEC = TR::VEC;
     if (a.m > 1 || a.n > kMaxFixedN) return launch_multi_op<TR, OP>(a);     // run-time counts of inputs and outputs
-    // common misalignment of all buffers to 16 bytes, in elements; mixed misalignment -> element kernel
-    const uintptr_t mis = (uintptr_t)a.dst & 15u;
-    bool same = true;
-    for (int j = 0; j < a.n; j++) same = same && (((uintptr_t)a.srcs[j] & 15u) == mis);
-    if (!same || (mis % sizeof(E)) != 0) {
-        SrcTable s;
-        for (int j = 0; j < a.n; j++) s.p[j] = a.srcs[j];
-        uint64_t blocks = (a.count + kBlock - 1) / kBlock;
-        int grid = grid_for(blocks, a.tune);
-        hipLaunchKernelGGL((reduce_elem_kernel<TR, OP>), dim3(grid), dim3(kBlock), 0, a.stream, s, a.n, a.dst,
-                           (uint64_t)a.count);
-        return hipGetLastError();
-    }
-    uint64_t head = mis ? (16u - mis) / sizeof(E) : 0;
+    uint64_t head = vector_head<E>(a);
     if (head > a.count) head = a.count;
     const uint64_t nvec = (a.count - head) / VEC;
     const uint32_t tail = (uint32_t)(a.count - head - nvec * VEC);

@@ -84,6 +84,7 @@ static uint16_t bf16(float v) { uint32_t u; memcpy(&u, &v, 4); return orc_bf16_n
 struct absmax { __device__ float operator()(float in, float inout) const { return fmaxf(fabsf(in), fabsf(inout)); } };
 struct val_idx { float v; int32_t i; };
 struct argmax { __device__ val_idx operator()(val_idx in, val_idx inout) const { return (in.v > inout.v || (in.v == inout.v && in.i < inout.i)) ? in : inout; } };
+struct xor_u16 { __device__ uint16_t operator()(uint16_t in, uint16_t inout) const { return (uint16_t)(in ^ inout); } };
 struct sat_add_u8 { __device__ uint8_t operator()(uint8_t in, uint8_t inout) const { unsigned s = (unsigned)in + inout; return (uint8_t)(s > 255 ? 255 : s); } };
 
 static const char* g_match_seen = nullptr; static size_t g_offset_seen = 0;
@@ -321,6 +322,19 @@ int main() {
         ccl_custom_reduce_n<uint8_t>(&sched, { du.p + 1, dv.p + 1, dv.p + 1 }, du.p + 1, 1000, sat_add_u8{});
         std::vector<uint8_t> gu = du.host();
         EXPECT(gu[0] == 200 && gu[1] == 255 && gu[1000] == 255, "saturating byte add, in place, odd alignment");
+
+        // sources and output at different offsets from a 16-byte boundary (loose vector reads)
+        {
+            const size_t cnt = 50021;
+            std::vector<uint16_t> x(cnt + 16), y(cnt + 16);
+            for (size_t i = 0; i < x.size(); i++) { x[i] = (uint16_t)(i * 31 + 7); y[i] = (uint16_t)(i * 17 + 3); }
+            DevBuf<uint16_t> dx(x), dy(y), dz(cnt + 16);
+            ccl_custom_reduce_n<uint16_t>(&sched, { dx.p + 1, dy.p + 6 }, dz.p + 3, cnt, xor_u16{});
+            std::vector<uint16_t> gz = dz.host();
+            ok = gz[2] == 0 && gz[3 + cnt] == 0;
+            for (size_t i = 0; i < cnt; i++) ok = ok && gz[3 + i] == (uint16_t)(x[1 + i] ^ y[6 + i]);
+            EXPECT(ok, "16-bit xor with every buffer at its own alignment");
+        }
     }
 
     CK(hipStreamDestroy(stream));

@@ -156,8 +156,8 @@ def test_recorded_probe_values_on_gpu(comp, probes):
 
 @pytest.mark.parametrize("dtype", [O.INT8, O.INT16, O.FLOAT32, O.FLOAT64, O.BFLOAT16, O.FLOAT16])
 def test_misaligned_and_inplace(comp, dtype):
-    """Buffers that share a misalignment modulo 16 bytes (head/tail lanes), buffers that do not (element
-    kernel), in-place output, output aliasing a later input."""
+    """Buffers that share a misalignment modulo 16 bytes (head/tail lanes), buffers that do not (loose vector
+    accesses), in-place output, output aliasing a later input."""
     import torch
     rng = np.random.default_rng(77 + dtype)
     esz = O.DTYPE_SIZE[dtype]
@@ -349,6 +349,56 @@ def test_phased_kernel_parity(comp, dtype, op, n):
             got = to_host(out, O.NP_STORAGE[dtype])
             assert_same(got[shift:], want, dtype, f"phased count={count} shift={shift}")
             assert (got[:shift] == 0).all()
+    finally:
+        comp.set_param("variant", 0)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 8])
+@pytest.mark.parametrize("dtype,op,n,m", [(O.BFLOAT16, O.SUM, 8, 1), (O.INT8, O.MAX, 5, 1), (O.FLOAT16, O.MIN, 3, 2),
+                                          (O.FLOAT64, O.SUM, 2, 1), (O.INT32, O.PROD, 11, 3), (O.UINT16, O.SUM, 1, 2)])
+def test_buffers_that_disagree_modulo_16_bytes(comp, variant, dtype, op, n, m):
+    """Every input and destination at its own offset from a 16-byte boundary, through each kernel form (default
+    choice, streaming, phased) and at sizes from less than a vector to several phases: the vectors start on a
+    boundary of the most common alignment, every other buffer is accessed as loose vectors, nothing outside the
+    destinations is written."""
+    import torch
+    rng = np.random.default_rng(4000 + 16 * dtype + n)
+    esz = O.DTYPE_SIZE[dtype]
+    np_t = O.NP_STORAGE[dtype]
+    per16 = 16 // esz
+    pad = 64
+    keep = 1 if dtype == O.BFLOAT16 else 0
+    comp.set_param("variant", variant)
+    try:
+        for count in (1, per16 - 1, per16 + 1, 1000, 70_001, 3_000_017):
+            srcs = make_inputs(rng, dtype, count, op, n)
+            want = O.reduce_n(srcs, dtype, op, keep=keep, threads=16)
+            for trial in range(3):
+                # trial 0: all different where possible; 1: inputs agree, destinations do not; 2: random
+                if trial == 0:
+                    sh = [(j + 1) % per16 for j in range(n + m)]
+                elif trial == 1:
+                    sh = [3 % per16] * n + [(5 + k) % per16 for k in range(m)]
+                else:
+                    sh = [int(x) for x in rng.integers(0, per16, n + m)]
+                big = []
+                for s_, k in zip(srcs, sh[:n]):
+                    h = np.zeros(count + 2 * pad, np_t)
+                    h[pad + k:pad + k + count] = s_
+                    big.append(to_dev(h))
+                outs = [to_dev(np.zeros(count + 2 * pad, np_t)) for _ in range(m)]
+                sp = [b_.data_ptr() + (pad + k) * esz for b_, k in zip(big, sh[:n])]
+                dp = [o_.data_ptr() + (pad + k) * esz for o_, k in zip(outs, sh[n:])]
+                if m == 1:
+                    comp.comp_reduce_n(dtype, op, sp, dp[0], count, lp_mode=keep)
+                else:
+                    comp.comp_reduce_write_n(dtype, op, sp, dp, count, lp_mode=keep)
+                torch.cuda.synchronize()
+                for o_, k in zip(outs, sh[n:]):
+                    g = to_host(o_, np_t)
+                    assert_same(g[pad + k:pad + k + count], want, dtype, f"count={count} shifts={sh}")
+                    assert not g[:pad + k].view(np.uint8).any() and not g[pad + k + count:].view(np.uint8).any(), \
+                        f"wrote outside a destination: count={count} shifts={sh}"
     finally:
         comp.set_param("variant", 0)
 

@@ -67,7 +67,7 @@ def test_one_input_is_a_byte_copy_for_every_dtype(comp):
 @pytest.mark.parametrize("variant", [2, 8])
 def test_destination_aliases_a_source_and_misaligned_buffers(comp, variant):
     """In place (destination k is source j, as allreduce_kernel's output may be its input), buffers that share a
-    misalignment to 16 bytes (vector path with head and tail) and buffers that do not (element path)."""
+    misalignment to 16 bytes (vector path with head and tail) and buffers that do not (loose vector accesses)."""
     import torch
     rng = np.random.default_rng(12)
     comp.set_param("variant", variant)
