@@ -8,8 +8,11 @@
       7 peer fusion buffers: pack + reduce + unpack, and the fused single pass
 
   types  every datatype x op at 512 MiB per buffer, 8 and 4 inputs
+  align  buffers that disagree modulo 16 bytes: 8-input bf16 sum at 64 MiB per buffer with every input at its own
+         alignment, and with only the output off; the reference's tight fusion layout (alignment 1) of 400 odd-sized
+         tensors: pack, unpack and the fused reduce
 
-    python bench_configs.py [--out results/configs.json] [--skip c3,types]
+    python bench_configs.py [--out results/configs.json] [--skip c3,types,align]
 
 Writes a JSON file and prints a markdown table.  Bytes are algorithmic: (N + 1) x chunk for a reduce, 2 x payload
 for pack and unpack.  Buffers of 64 MiB rotate over several sets so that the 256 MB Infinity Cache cannot hold them.
@@ -119,6 +122,35 @@ def main():
                     cells.append(f"{opn} {gbs:,.0f}")
                 rows.append(f"| {label}, {nin} inputs, 512 MiB per buffer | {(nin + 1) * size:,} | | {' / '.join(cells)} | | GB/s per op |")
                 del ss, oo
+    # ---- buffers at different offsets from a 16-byte boundary
+    if "align" not in args.skip:
+        na = 33_554_432
+        sets = [[torch.empty(na + 64, dtype=torch.bfloat16, device="cuda").normal_(0, 1) for _ in range(9)] for _ in range(6)]
+        for label, shifts in (("all aligned", [0] * 9), ("every input at its own alignment", [1, 2, 3, 4, 5, 6, 7, 0, 0]),
+                              ("only the output off by 6 bytes", [0] * 8 + [3])):
+            ptrs = [[t.data_ptr() + 2 * sh for t, sh in zip(s_, shifts)] for s_ in sets]
+            us = timed(torch, lambda i: comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, ptrs[i % 6][:8], ptrs[i % 6][8], na,
+                                                          lp_mode=comp.LP_KEEP_PRECISION), 64, 16)
+            add(f"align: bf16 sum, 8 inputs, 64 MiB, {label}", us, 9 * na * 2, "6 rotating buffer sets")
+        del sets
+        rng = np.random.default_rng(1)
+        for label, odd in (("even", 0), ("odd", 1)):
+            counts = [int(c) // 8 * 8 + odd for c in np.exp(rng.uniform(np.log(2048), np.log(4 << 20), 400))]
+            payload = sum(counts) * 2
+            plan = comp.FusionPlan(counts, comp.BFLOAT16, 1)
+            nelem = plan.nbytes // 2 + 8
+            tens = [torch.empty(c, dtype=torch.bfloat16, device="cuda").normal_(0, 0.02) for c in counts]
+            outs = [torch.empty_like(t) for t in tens]
+            fb = torch.empty(nelem, dtype=torch.bfloat16, device="cuda")
+            peers = [torch.empty(nelem, dtype=torch.bfloat16, device="cuda").normal_(0, 0.02) for _ in range(7)]
+            us = timed(torch, lambda i: plan.pack(tens, fb), 20, 5)
+            add(f"align: pack, 400 {label}-sized bf16 tensors, tight layout, payload {payload:,} B", us, 2 * payload)
+            us = timed(torch, lambda i: plan.unpack(fb, outs), 20, 5)
+            add(f"align: unpack, {label}-sized", us, 2 * payload)
+            us = timed(torch, lambda i: plan.reduce(comp.SUM, tens, peers, outs, lp_mode=comp.LP_KEEP_PRECISION), 20, 5)
+            add(f"align: fused reduce against 7 peers, {label}-sized", us, 9 * payload)
+            plan.close()
+            del tens, outs, fb, peers
     # ---- C4
     rng = np.random.default_rng(4)
     counts = [int(round(math.exp(rng.uniform(math.log(2048), math.log(2_097_152))))) for _ in range(256)]
