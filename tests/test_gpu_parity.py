@@ -225,23 +225,15 @@ def test_copy_and_converters(comp):
                 got = to_host(dd, np.uint8)
                 assert (got[sb:sb + nbytes] == src[sa:sa + nbytes]).all()
                 assert (got[:sb] == 0).all() and (got[sb + nbytes:] == 0).all()
-    # a large copy with head and tail bytes, through the plain copy kernel and (with the crossover lowered) through
-    # the phased one-input kernel that copies of several GB take
-    nbytes = (800 << 20) + 5
+    # a large copy with head and tail bytes (one 4 KiB tile per block: a few hundred thousand blocks)
+    nbytes = (2400 << 20) + 5
     src_d = torch.randint(-128, 127, (nbytes + 32,), dtype=torch.int8, device="cuda")
-    for min_bytes in (comp.get_param("phased_min_bytes"), 1 << 20):
-        default = comp.get_param("phased_min_bytes")
-        comp.set_param("phased_min_bytes", min_bytes)
-        try:
-            dst_d = torch.zeros(nbytes + 32, dtype=torch.int8, device="cuda")
-            comp.comp_copy(src_d.data_ptr() + 3, dst_d.data_ptr() + 19, nbytes, use_nontemporal=True)
-            torch.cuda.synchronize()
-        finally:
-            comp.set_param("phased_min_bytes", default)
-        assert torch.equal(dst_d[19:19 + nbytes], src_d[3:3 + nbytes])
-        assert int(dst_d[:19].count_nonzero()) == 0 and int(dst_d[19 + nbytes:].count_nonzero()) == 0
-        del dst_d
-    del src_d
+    dst_d = torch.zeros(nbytes + 32, dtype=torch.int8, device="cuda")
+    comp.comp_copy(src_d.data_ptr() + 3, dst_d.data_ptr() + 19, nbytes, use_nontemporal=True)
+    torch.cuda.synchronize()
+    assert torch.equal(dst_d[19:19 + nbytes], src_d[3:3 + nbytes])
+    assert int(dst_d[:19].count_nonzero()) == 0 and int(dst_d[19 + nbytes:].count_nonzero()) == 0
+    del dst_d, src_d
     L = O.lib()
     for count in (1, 5, 16, 22, 1000, 65536 + 7):
         f32 = rng.integers(0, 2**32, count, dtype=np.uint32)
@@ -260,6 +252,27 @@ def test_copy_and_converters(comp):
         comp.convert_bf16_to_fp32_arrays(to_dev(h), d, count)
         torch.cuda.synchronize()
         assert (to_host(d, np.uint32) == (h.astype(np.uint32) << 16)).all()
+    # the two arrays at different offsets from a 16-byte boundary (the input is read as loose vectors), sizes from
+    # less than one group of eight to many blocks; nothing outside the output is written
+    for count in (3, 8, 29, 70_001, 3_000_019):
+        for si, so in ((0, 0), (1, 0), (0, 1), (3, 5), (2, 7)):
+            f32 = rng.integers(0, 2**32, count + 16, dtype=np.uint32)
+            for impl in (1, 2):
+                want = np.empty(count, np.uint16)
+                L.orc_convert_fp32_to_bf16_arrays(f32[si:].ctypes.data, want.ctypes.data, count, impl)
+                d, src_d = to_dev(np.zeros(count + 16, np.uint16)), to_dev(f32)
+                comp.convert_fp32_to_bf16_arrays(src_d.data_ptr() + 4 * si, d.data_ptr() + 2 * so, count, bf16_impl=impl)
+                torch.cuda.synchronize()
+                got = to_host(d, np.uint16)
+                assert (got[so:so + count] == want).all(), (count, si, so, impl)
+                assert not got[:so].any() and not got[so + count:].any(), (count, si, so, impl)
+            h = rng.integers(0, 65536, count + 16, dtype=np.uint16)
+            d, src_d = to_dev(np.zeros(count + 16, np.uint32)), to_dev(h)
+            comp.convert_bf16_to_fp32_arrays(src_d.data_ptr() + 2 * si, d.data_ptr() + 4 * so, count)
+            torch.cuda.synchronize()
+            got = to_host(d, np.uint32)
+            assert (got[so:so + count] == (h[si:si + count].astype(np.uint32) << 16)).all(), (count, si, so)
+            assert not got[:so].any() and not got[so + count:].any(), (count, si, so)
 
 
 def test_bf16_narrowing_exhaustive_on_gpu(comp):
