@@ -88,9 +88,23 @@ def cpu_baseline(torch, comp, w, bufs, sample_elems):
     # acc / narrow (ccl_comp_batch_reduce keep-precision), or the pairwise chain for plain types
     buf = np.concatenate(host)
     offs = np.arange(w["n"], dtype=np.uint64) * np.uint64(s)
-    tmp = np.empty(s, np.float32)
-    acc = np.empty(s, np.float32)
+    tmp = np.zeros(s, np.float32)       # touched before the clock starts
+    acc = np.zeros(s, np.float32)
     L = O.lib()
+    R = O.ref()
+    # (0) the same pass structure with the conversions done by the reference's own AVX-512 helpers (oracle/_ref,
+    # compiled from the reference's sources where the library was built), when the host CPU has AVX512-BF16
+    ref_keep = None
+    if (dt == O.BFLOAT16 and w["keep"] and R is not None and hasattr(R, "ref_batch_reduce_keep_sum")
+            and (O.ref_cpu_support() & 3) == 3):
+        buf2 = buf.copy()
+        t0 = time.perf_counter()
+        rc = R.ref_batch_reduce_keep_sum(buf2.ctypes.data, offs.ctypes.data, w["n"], s, buf2.ctypes.data,
+                                         tmp.ctypes.data, acc.ctypes.data, O.BF16_AVX512BF)
+        t1 = time.perf_counter()
+        assert rc == 0
+        ref_keep = (algo_bytes / (t1 - t0) / 1e9, buf2[:s].copy())
+        del buf2
     t0 = time.perf_counter()
     rc = L.orc_comp_batch_reduce(buf.ctypes.data, offs.ctypes.data, w["n"], s, buf.ctypes.data, dt, O.SUM,
                                  1 if w["keep"] else 0, tmp.ctypes.data, acc.ctypes.data, O.BF16_AVX512BF,
@@ -107,12 +121,38 @@ def cpu_baseline(torch, comp, w, bufs, sample_elems):
     t1 = time.perf_counter()
     multi = algo_bytes / (t1 - t0) / 1e9
     assert (out.view(np.uint8) == ref_out.view(np.uint8)).all(), "oracle forms disagree"
+    # (iii) the reference's own AVX-512 code (oracle/_ref, compiled from the reference's sources where the library
+    # was built): its bf16 reduce rounds after every input, so this times the pairwise mode of the same reduction --
+    # 2^31 elements per call at most, one thread
+    ref_leg = None
+    if dt == O.BFLOAT16 and R is not None and (O.ref_cpu_support() & 3) == 3 and s < 2**31 - 1 and w["n"] >= 2:
+        acc16 = host[0].copy()
+        t0 = time.perf_counter()
+        for j in range(1, w["n"]):
+            assert R.ref_bf16_reduce(host[j].ctypes.data, s, acc16.ctypes.data, O.SUM, O.BF16_AVX512BF) == 0
+        t1 = time.perf_counter()
+        want = O.reduce_n(host, dt, O.SUM, keep=0, threads=W)
+        assert (acc16 == want).all(), "the reference's code and the oracle disagree on the pairwise sum"
+        ref_leg = dict(value=round(algo_bytes / (t1 - t0) / 1e9, 3), unit="GB/s", cores=1, kind="reference",
+                       sample=f"the same sample through ccl_bf16_reduce_impl_avx512bf, {w['n'] - 1} in-place pairwise "
+                              f"calls (rounds after every input, unlike the measured mode); equal to the oracle's "
+                              f"pairwise result")
+    sample = (f"first {s} elements of each of the {w['n']} buffers of the same workload "
+              f"({algo_bytes / 1e9:.2f} GB algorithmic), reference pass structure "
+              f"(ccl_comp_batch_reduce: widen / fp32 add / narrow), 1 thread = CCL_WORKER_COUNT=1")
+    if ref_keep is not None:
+        assert (ref_keep[1] == ref_out).all(), "the reference's helpers and the oracle disagree"
+        return dict(value=round(ref_keep[0], 3), unit="GB/s", cores=1, kind="reference",
+                    sample=sample + "; conversions by the reference's own ccl_bf16_load_as_fp32 / "
+                           "ccl_fp32_store_as_bf16_avx512bf compiled from its sources, results equal to the oracle's; "
+                           f"scalar C port of the same passes: {one:.2f} GB/s; {W}-thread partitioned single-pass "
+                           f"port: {multi:.2f} GB/s",
+                    port=dict(value=round(one, 3), cores=1), multi_thread=dict(value=round(multi, 3), cores=W),
+                    **({"reference_pairwise": ref_leg} if ref_leg else {})), out, s
     return dict(value=round(one, 3), unit="GB/s", cores=1, kind="port",
-                sample=f"first {s} elements of each of the {w['n']} buffers of the same workload "
-                       f"({algo_bytes / 1e9:.2f} GB algorithmic), reference pass structure "
-                       f"(ccl_comp_batch_reduce: widen / fp32 add / narrow), 1 thread = CCL_WORKER_COUNT=1; "
-                       f"{W}-thread partitioned single-pass port: {multi:.2f} GB/s",
-                multi_thread=dict(value=round(multi, 3), cores=W)), out, s
+                sample=sample + f"; {W}-thread partitioned single-pass port: {multi:.2f} GB/s",
+                multi_thread=dict(value=round(multi, 3), cores=W),
+                **({"reference_pairwise": ref_leg} if ref_leg else {})), out, s
 
 
 def main():

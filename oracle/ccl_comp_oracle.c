@@ -22,7 +22,10 @@
  *   orc_comp_reduce plain types     IEEE single op per pair / two's-complement wrap: numpy closed forms,
  *                                   min/max truth table recorded from the reference library
  *   orc_convert_*_arrays tail       recorded probe values of the reference library (tail truncation)
- *   orc_comp_batch_reduce           composition; recorded probe values (1+3*2^-8 -> 3f82 body / 3f81 tail)
+ *   orc_comp_batch_reduce           composition; recorded probe values (1+3*2^-8 -> 3f82 body / 3f81 tail); the
+ *                                   keep-precision sum against the reference's own 16-wide converters called in
+ *                                   the reference's pass order (oracle/_ref, ref_batch_reduce_keep_sum) on random
+ *                                   bit patterns and gradient-like values, 1..9 slices
  *   orc_fusion_*                    pack/unpack round trip, offsets closed form
  *   orc_reduce_write_n              composition of orc_reduce_n (pinned above) and memcpy: every destination equals
  *                                   orc_reduce_n's output; closed forms of the reference's functional tests

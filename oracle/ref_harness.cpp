@@ -6,7 +6,8 @@
  * copied; the output goes to oracle/_ref/ only.
  *
  * What this reaches: ccl_bf16_reduce_impl_{avx512f,avx512bf} (bf16_intrisics.hpp:106-114),
- * ccl_bf16_load_as_fp32 / ccl_fp32_store_as_bf16_{avx512f,avx512bf} (:62-76),
+ * ccl_bf16_load_as_fp32 / ccl_fp32_store_as_bf16_{avx512f,avx512bf} (:62-76), singly and in the loop of the
+ * keep-precision batch reduce,
  * ccl_fp16_reduce_impl_{256,512} (fp16_intrisics.hpp:186-196).
  * What it cannot reach: the dispatchers in comp.cpp / bf16.cpp / fp16.cpp need ccl::global_data, the
  * logger and the datatype storage, i.e. the whole library, whose build needs cmake and the prebuilt
@@ -96,6 +97,38 @@ REF_TARGET_BF16 int ref_fp32_store_as_bf16_16(const void* src, void* dst, int im
         return 0;
     }
     return -1;
+}
+
+/* The keep-precision batch reduce (sum) with the reference's pass structure (src/comp/comp.cpp:202-249: widen the own
+ * slice into acc; per further slice widen into tmp and add tmp into acc in fp32; narrow acc once), its conversions done
+ * by the reference's own 16-wide helpers exactly as its array converters call them (src/comp/bf16/bf16.cpp:130-169)
+ * and the fp32 add by a plain loop built for the baseline x86-64 target, as the reference's CCL_REDUCE loop is
+ * (comp.cpp:31-58).  Slices are in_buf + 2 * offsets[i]; inout is slice 0.  count must be a multiple of 16 (the
+ * scalar tail converters live in bf16.cpp, which is not part of this build).  For timing the reference's CPU path. */
+__attribute__((noinline)) static void ref_add_f32(const float* in, float* inout, size_t count) {
+    for (size_t i = 0; i < count; i++) inout[i] = in[i] + inout[i];
+}
+REF_TARGET_BF16 __attribute__((noinline)) static void ref_widen(const void* bf16, float* f32, size_t count) {
+    for (size_t i = 0; i < count; i += 16) ccl_bf16_load_as_fp32((const char*)bf16 + 2 * i, f32 + i);
+}
+REF_TARGET_BF16 __attribute__((noinline)) static void ref_narrow(const float* f32, void* bf16, size_t count, int impl) {
+    if (impl == 2)
+        for (size_t i = 0; i < count; i += 16) ccl_fp32_store_as_bf16_avx512bf(f32 + i, (char*)bf16 + 2 * i);
+    else
+        for (size_t i = 0; i < count; i += 16) ccl_fp32_store_as_bf16_avx512f(f32 + i, (char*)bf16 + 2 * i);
+}
+int ref_batch_reduce_keep_sum(const void* in_buf, const size_t* offsets, size_t n, size_t count, void* inout,
+                              float* tmp, float* acc, int impl) {
+    int cpu = ref_cpu_support();
+    if (!(cpu & 1) || (impl == 2 && !(cpu & 2)) || (impl != 1 && impl != 2) || (count % 16) != 0 || n < 1)
+        return -1;
+    ref_widen(inout, acc, count);
+    for (size_t i = 1; i < n; i++) {
+        ref_widen((const char*)in_buf + 2 * offsets[i], tmp, count);
+        ref_add_f32(tmp, acc, count);
+    }
+    ref_narrow(acc, inout, count, impl);
+    return 0;
 }
 
 /* impl: 2 = f16c (8 per iteration, memcpy'd tail), 3 = avx512f (16 per iteration, masked tail),

@@ -91,6 +91,9 @@ def ref():
         R.ref_fp16_reduce.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int]
         R.ref_bf16_load_as_fp32_16.argtypes = [C.c_void_p, C.c_void_p]
         R.ref_fp32_store_as_bf16_16.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
+        if hasattr(R, "ref_batch_reduce_keep_sum"):
+            R.ref_batch_reduce_keep_sum.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p,
+                                                    C.c_void_p, C.c_void_p, C.c_int]
         _ref = R
     return _ref
 

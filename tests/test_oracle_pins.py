@@ -427,6 +427,37 @@ def test_against_reference_code_random(fam, dtype, impls):
 
 
 @needs_ref
+@pytest.mark.parametrize("impl", [1, 2])
+def test_keep_precision_batch_reduce_against_the_reference_helpers_in_its_pass_structure(impl):
+    """orc_comp_batch_reduce (keep-precision sum) against the reference's own 16-wide converters called in the
+    reference's pass order (widen own into acc; per slice widen into tmp, fp32 add; narrow once), on random bit
+    patterns (NaNs, infinities, denormals included) and on gradient-like values, 1..9 slices."""
+    R = O.ref()
+    if not hasattr(R, "ref_batch_reduce_keep_sum"):
+        pytest.skip("oracle/_ref predates ref_batch_reduce_keep_sum: rebuild it (make -C oracle ref)")
+    rng = np.random.default_rng(314 + impl)
+    L = O.lib()
+    for n in (1, 2, 5, 8, 9):
+        for count in (16, 4096, 100_000 - 100_000 % 16):
+            for kind in ("bits", "normal"):
+                if kind == "bits":
+                    buf = rng.integers(0, 65536, n * count, dtype=np.uint16)
+                else:
+                    buf = (rng.standard_normal(n * count).astype(np.float32) * 1e-3).view(np.uint32)
+                    buf = (buf >> 16).astype(np.uint16)
+                offs = np.arange(n, dtype=np.uint64) * np.uint64(count)
+                tmp, acc = np.empty(count, np.float32), np.empty(count, np.float32)
+                want = buf.copy()
+                assert R.ref_batch_reduce_keep_sum(want.ctypes.data, offs.ctypes.data, n, count, want.ctypes.data,
+                                                   tmp.ctypes.data, acc.ctypes.data, impl) == 0
+                got = buf.copy()
+                assert L.orc_comp_batch_reduce(got.ctypes.data, offs.ctypes.data, n, count, got.ctypes.data, O.BFLOAT16,
+                                               O.SUM, 1, tmp.ctypes.data, acc.ctypes.data, impl, O.FP16_AVX512F) == 0
+                assert O.same_bits_or_both_nan(got[:count], want[:count], O.BFLOAT16).all(), (n, count, kind)
+                assert (got[count:] == buf[count:]).all()
+
+
+@needs_ref
 def test_against_reference_code_every_bf16_pair_sampled():
     """All 65536 bf16 values against 64 partners (sum, RNE): 4M pairs through the reference code."""
     R = O.ref()
