@@ -293,44 +293,62 @@ struct VecOps {
     }
 };
 
-template <bool VEC_SEM>
-struct FlushF32Results<Bf16PairwiseTraits<true, VEC_SEM>, OP_SUM> {
-    static constexpr bool value = true;
-};
-template <bool VEC_SEM>
-struct FlushF32Results<Bf16PairwiseTraits<true, VEC_SEM>, OP_PROD> {
+// every operation of the avx512bf pairwise reduce ends in VCVTNEPS2BF16, which reads a denormal as zero
+template <bool VEC_SEM, int OP>
+struct FlushF32Results<Bf16PairwiseTraits<true, VEC_SEM>, OP> {
     static constexpr bool value = true;
 };
 
-// bf16 rounded to nearest even after every pair: the accumulator stays in storage format (two bf16 per dword, in
-// a.v[0..3]); both halves of a dword are widened, combined and narrowed together by the packed conversion.
+// x as the hardware hands it back from an fp32 operation: with the wave in the mode above a denormal becomes a
+// signed zero and a signalling NaN its quiet form, every other value is unchanged -- for a value that is a widened
+// bf16, exactly what VCVTNEPS2BF16 followed by widening gives.  (An instruction the compiler cannot fold away: it
+// knows nothing of the mode.)
+__device__ __forceinline__ uint32_t f32_through_alu(uint32_t x) {
+    uint32_t r;
+    asm("v_mul_f32 %0, 1.0, %1" : "=v"(r) : "v"(x));
+    return r;
+}
+
+// bf16 rounded to nearest even after every pair.  The accumulator is carried widened (eight fp32 values whose low
+// halves are zero), so a step widens only the new input: sum and prod round the pair of results with the packed
+// conversion and widen it again; min and max select on the widened values and pass the selected one through the
+// ALU, which is all the rounding step does to a value that already is a bf16.  With one input nothing is touched.
 template <bool VEC_SEM>
 struct VecOps<Bf16PairwiseTraits<true, VEC_SEM>> {
     typedef Bf16PairwiseTraits<true, VEC_SEM> TR;
     static __device__ __forceinline__ Accs<TR> init(u32x4 x) {
         Accs<TR> a;
 #pragma unroll
-        for (int k = 0; k < 4; k++) a.v[k] = x[k];
+        for (int k = 0; k < 4; k++) {
+            a.v[2 * k] = x[k] << 16;
+            a.v[2 * k + 1] = x[k] & 0xffff0000u;
+        }
         return a;
     }
     template <int OP>
     static __device__ __forceinline__ void step(u32x4 x, Accs<TR>& a) {
+        static_assert(FlushF32Results<TR, OP>::value, "the kernels of this traits class set the wave's denormal mode");
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            const uint32_t in = x[k], io = a.v[k];
-            const uint32_t lo = f32_step_bits<OP, VEC_SEM>(in << 16, io << 16);
-            const uint32_t hi = f32_step_bits<OP, VEC_SEM>(in & 0xffff0000u, io & 0xffff0000u);
-            if constexpr (FlushF32Results<TR, OP>::value) {     // a denormal sum or product is already a signed zero
+            const uint32_t lo = f32_step_bits<OP, VEC_SEM>(x[k] << 16, a.v[2 * k]);
+            const uint32_t hi = f32_step_bits<OP, VEC_SEM>(x[k] & 0xffff0000u, a.v[2 * k + 1]);
+            if (OP == OP_SUM || OP == OP_PROD) {    // a denormal sum or product is already a signed zero
                 const f32x2 f = { as_f32(lo), as_f32(hi) };
-                a.v[k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+                const uint32_t r = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+                a.v[2 * k] = r << 16;
+                a.v[2 * k + 1] = r & 0xffff0000u;
             }
             else {
-                a.v[k] = bf16_narrow_rne_pack2(lo, hi);
+                a.v[2 * k] = f32_through_alu(lo);
+                a.v[2 * k + 1] = f32_through_alu(hi);
             }
         }
     }
     static __device__ __forceinline__ u32x4 finish(const Accs<TR>& a) {
-        return u32x4{ a.v[0], a.v[1], a.v[2], a.v[3] };
+        u32x4 r;
+#pragma unroll
+        for (int k = 0; k < 4; k++) r[k] = (a.v[2 * k] >> 16) | (a.v[2 * k + 1] & 0xffff0000u);
+        return r;
     }
 };
 

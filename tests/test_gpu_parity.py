@@ -521,26 +521,28 @@ def test_fp16_native_mode_against_reference_made_vectors(comp, golden, golden_fp
         comp.set_param("fp16_impl", 1)
 
 
-def test_bf16_pairwise_tiny_sums_and_products_through_every_kernel(comp):
+def test_bf16_pairwise_tiny_and_special_values_through_every_kernel(comp):
     """Round-after-every-pair bf16 under avx512bf where the fp32 sum or product is a denormal: VCVTNEPS2BF16 reads it
     as zero (the result is a signed zero), and a value just under the smallest normal must not round up to it.  Every
     pair of a value set around the bottom of the exponent range (sums) and around the square root of it (products),
     through the streaming and the phased kernel, the run-time-count kernels (nine inputs; two outputs) and the
-    fused kernel, in both forms."""
+    fused kernel, in both forms.  min and max hand back one operand, which the same instruction turns into a signed
+    zero when it is a denormal and quiets when it is a signalling NaN: the same value set plus infinities and NaNs,
+    bit for bit."""
     import torch
     vals = []
     for sign in (0, 0x8000):
         for e in (0, 1, 2, 3, 61, 62, 63, 64, 65, 66):
             for m in (0, 1, 0x3F, 0x40, 0x7E, 0x7F):
                 vals.append(sign | (e << 7) | m)
-    vals = np.array(vals, dtype=np.uint16)
-    a = np.tile(np.repeat(vals, vals.size), 25)          # in
-    b = np.tile(np.tile(vals, vals.size), 25)            # inout
-    count = a.size
-    zero = np.zeros(count, np.uint16)
-    for op in (O.SUM, O.PROD):
+    specials = [0x7F80, 0xFF80, 0x7FC0, 0xFFC0, 0x7F81, 0xFF81, 0x7FBF, 0x7FFF, 0xFFFF, 0x7F7F, 0xFF7F, 0x3F80, 0xBF80]
+    for op in (O.SUM, O.PROD, O.MIN, O.MAX):
+        v = np.array(vals + (specials if op in (O.MIN, O.MAX) else []), dtype=np.uint16)
+        a = np.tile(np.repeat(v, v.size), 25)          # in
+        b = np.tile(np.tile(v, v.size), 25)            # inout
+        count = a.size
         want2 = O.reduce_n([b, a], O.BFLOAT16, op)
-        ident = zero if op == O.SUM else np.full(count, 0x3F80, np.uint16)
+        ident = np.full(count, {O.SUM: 0, O.PROD: 0x3F80, O.MIN: 0x7F80, O.MAX: 0xFF80}[op], np.uint16)
         want9 = O.reduce_n([b, a] + [ident] * 7, O.BFLOAT16, op)
         for variant in (2, 8):
             comp.set_param("variant", variant)
