@@ -12,7 +12,9 @@
          alignment, and with only the output off; the reference's tight fusion layout (alignment 1) of 400 odd-sized
          tensors: pack, unpack and the fused reduce
 
-    python bench_configs.py [--out results/configs.json] [--skip c3,types,align]
+  copy   ccl_comp_copy at 64 MiB, 512 MiB and 3 GiB, and the bf16 <-> fp32 array converters at 2^28 elements
+
+    python bench_configs.py [--out results/configs.json] [--skip c3,types,align,copy]
 
 Writes a JSON file and prints a markdown table.  Bytes are algorithmic: (N + 1) x chunk for a reduce, 2 x payload
 for pack and unpack.  Buffers of 64 MiB rotate over several sets so that the 256 MB Infinity Cache cannot hold them.
@@ -151,6 +153,24 @@ def main():
             add(f"align: fused reduce against 7 peers, {label}-sized", us, 9 * payload)
             plan.close()
             del tens, outs, fb, peers
+    # ---- copies and converters
+    if "copy" not in args.skip:
+        for mib in (64, 512, 3072):
+            nb = mib << 20
+            nsets = 4 if mib == 64 else 1
+            src = [torch.empty(nb, dtype=torch.uint8, device="cuda").random_(0, 255) for _ in range(nsets)]
+            dst = [torch.empty(nb, dtype=torch.uint8, device="cuda") for _ in range(nsets)]
+            us = timed(torch, lambda i: comp.comp_copy(src[i % nsets], dst[i % nsets], nb, use_nontemporal=True), 20, 5)
+            add(f"copy, {mib} MiB", us, 2 * nb, f"{nsets} set(s)")
+            del src, dst
+        nc = 1 << 28
+        f32 = torch.empty(nc, dtype=torch.float32, device="cuda").normal_()
+        b16 = torch.empty(nc, dtype=torch.bfloat16, device="cuda")
+        us = timed(torch, lambda i: comp.convert_fp32_to_bf16_arrays(f32, b16, nc), 20, 5)
+        add("convert fp32 -> bf16 (round to nearest even), 2^28 elements", us, 6 * nc)
+        us = timed(torch, lambda i: comp.convert_bf16_to_fp32_arrays(b16, f32, nc), 20, 5)
+        add("convert bf16 -> fp32, 2^28 elements", us, 6 * nc)
+        del f32, b16
     # ---- C4
     rng = np.random.default_rng(4)
     counts = [int(round(math.exp(rng.uniform(math.log(2048), math.log(2_097_152))))) for _ in range(256)]
