@@ -202,17 +202,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                 for (int j = 0; j < NP; j++) s[j + 1] = (const u32x4_u*)((const unsigned char*)peers.p[j] + poff + head * ES);
                 const uint64_t idx[2] = { tid, tid + (uint32_t)kPhaseBlock };
                 u32x4 res[2];
-                if constexpr (TR::VEC * NT <= 64) {
-                    reduce_group_guarded<TR, OP, NT, 2>(s, idx, nvec, res);
-                }
-                else {      // 16 one-byte elements x 7-8 inputs: both vectors at once would not fit the registers
-                    const uint64_t i0[1] = { idx[0] }, i1[1] = { idx[1] };
-                    u32x4 r0[1], r1[1];
-                    reduce_group_guarded<TR, OP, NT, 1>(s, i0, nvec, r0);
-                    reduce_group_guarded<TR, OP, NT, 1>(s, i1, nvec, r1);
-                    res[0] = r0[0];
-                    res[1] = r1[0];
-                }
+                reduce_group_guarded<TR, OP, NT, 2>(s, idx, nvec, res);
                 if (k < S) {
                     stage[(2 * k) * kPhaseBlock + tid] = res[0];
                     stage[(2 * k + 1) * kPhaseBlock + tid] = res[1];

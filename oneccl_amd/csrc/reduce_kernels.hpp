@@ -352,6 +352,45 @@ struct VecOps<Bf16PairwiseTraits<true, VEC_SEM>> {
     }
 };
 
+// One-byte integers: the accumulator stays in storage format (four bytes per dword, in a.v[0..3]) and every byte is
+// combined by one instruction that reads byte k of both operands and writes byte k of the accumulator, leaving the
+// other three alone (the sub-dword addressing of the gfx9 vector ALU).  Sixteen instructions per vector and step
+// where extracting, combining and re-inserting bytes takes the compiler about sixty.  The low byte of a 16-bit sum
+// or product of sign- or zero-extended bytes is the wrapped 8-bit result; min and max compare the extended bytes.
+#define MI_BYTE_OP(INSTR, S0, S1, K)                                                                              \
+    asm(INSTR " %0, " S0 ", " S1 " dst_sel:BYTE_" #K " dst_unused:UNUSED_PRESERVE src0_sel:BYTE_" #K              \
+              " src1_sel:BYTE_" #K                                                                                 \
+        : "+v"(acc)                                                                                                \
+        : "v"(in))
+#define MI_BYTE_OP4(INSTR, S0, S1) \
+    MI_BYTE_OP(INSTR, S0, S1, 0); MI_BYTE_OP(INSTR, S0, S1, 1); MI_BYTE_OP(INSTR, S0, S1, 2); MI_BYTE_OP(INSTR, S0, S1, 3)
+template <bool SIGNED, int OP>
+__device__ __forceinline__ uint32_t bytes_step(uint32_t in, uint32_t acc) {
+    if (OP == OP_SUM) { MI_BYTE_OP4("v_add_u16_sdwa", "%1", "%0"); }
+    else if (OP == OP_PROD) { MI_BYTE_OP4("v_mul_lo_u16_sdwa", "%1", "%0"); }
+    else if (OP == OP_MIN && SIGNED) { MI_BYTE_OP4("v_min_i16_sdwa", "sext(%1)", "sext(%0)"); }
+    else if (OP == OP_MIN) { MI_BYTE_OP4("v_min_u16_sdwa", "%1", "%0"); }
+    else if (SIGNED) { MI_BYTE_OP4("v_max_i16_sdwa", "sext(%1)", "sext(%0)"); }
+    else { MI_BYTE_OP4("v_max_u16_sdwa", "%1", "%0"); }
+    return acc;
+}
+#undef MI_BYTE_OP4
+#undef MI_BYTE_OP
+template <class T>
+struct VecOps<PlainTraits<T, uint8_t>> {
+    typedef PlainTraits<T, uint8_t> TR;
+    static_assert(sizeof(Accs<TR>) == 16, "sixteen one-byte accumulators are the vector itself");
+    static __device__ __forceinline__ Accs<TR> init(u32x4 x) { return __builtin_bit_cast(Accs<TR>, x); }
+    template <int OP>
+    static __device__ __forceinline__ void step(u32x4 x, Accs<TR>& a) {
+        u32x4 acc = __builtin_bit_cast(u32x4, a);
+#pragma unroll
+        for (int k = 0; k < 4; k++) acc[k] = bytes_step<((T)-1 < (T)0), OP>(x[k], acc[k]);
+        a = __builtin_bit_cast(Accs<TR>, acc);
+    }
+    static __device__ __forceinline__ u32x4 finish(const Accs<TR>& a) { return __builtin_bit_cast(u32x4, a); }
+};
+
 // fp16: the accumulator stays in storage format (two halves per dword, in a.v[0..3]).  sum and prod widen, combine
 // and narrow both halves of a dword.  min and max pick each half with one compare and a bit-field insert; the
 // quieting of a NaN they hand back (only the first input can bring one: a NaN `in` is never chosen) does not change

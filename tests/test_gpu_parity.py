@@ -521,6 +521,56 @@ def test_fp16_native_mode_against_reference_made_vectors(comp, golden, golden_fp
         comp.set_param("fp16_impl", 1)
 
 
+@pytest.mark.parametrize("dtype", [O.INT8, O.UINT8])
+def test_one_byte_integers_every_pair_of_values_through_every_kernel(comp, dtype):
+    """All 65,536 (in, inout) pairs of one-byte values for the four operations (wrapping sum and product, signed or
+    unsigned min and max), through the streaming kernel, the phased kernel, the run-time-count kernels (nine inputs,
+    two outputs) and the fused kernel in both forms: the byte-lane instructions of the vector path against the
+    oracle."""
+    import torch
+    np_t = O.NP_STORAGE[dtype]
+    allv = np.arange(256, dtype=np.uint8).view(np_t)
+    a = np.tile(np.repeat(allv, 256), 3)         # in
+    b = np.tile(np.tile(allv, 256), 3)           # inout
+    count = a.size
+    rng = np.random.default_rng(8 + dtype)
+    extra = [rng.integers(0, 256, count, dtype=np.uint8).view(np_t) for _ in range(7)]
+    for op in range(4):
+        want2 = O.reduce_n([b, a], dtype, op)
+        want9 = O.reduce_n([b, a] + extra, dtype, op)
+        for variant in (2, 8):
+            comp.set_param("variant", variant)
+            try:
+                da, db = to_dev(a), to_dev(b)
+                comp.comp_reduce(dtype, op, da, count, db)
+                torch.cuda.synchronize()
+                assert (to_host(db, np_t) == want2).all(), (op, variant, "pair")
+                db = to_dev(b)
+                de = [to_dev(e) for e in extra]
+                outs = [torch.empty_like(db) for _ in range(2)]
+                comp.comp_reduce_write_n(dtype, op, [db, da] + de, outs, count)
+                torch.cuda.synchronize()
+                for o in outs:
+                    assert (to_host(o, np_t) == want9).all(), (op, variant, "nine inputs, two outputs")
+                h = count // 2 + 5
+                plan = comp.FusionPlan([h, count - h], dtype, 1)
+                peers = []
+                for src in [a] + extra:
+                    fb = torch.zeros(plan.nbytes, dtype=db.dtype, device="cuda")
+                    d_ = to_dev(src)
+                    plan.pack([d_[:h], d_[h:]], fb)
+                    peers.append(fb)
+                own = [db[:h], db[h:]]
+                for npeers, want in ((1, want2), (8, want9)):
+                    res = [torch.empty_like(t) for t in own]
+                    plan.reduce(op, own, peers[:npeers], res)
+                    torch.cuda.synchronize()
+                    got = np.concatenate([to_host(r, np_t) for r in res])
+                    assert (got == want).all(), (op, variant, "fused", npeers)
+            finally:
+                comp.set_param("variant", 0)
+
+
 def test_bf16_pairwise_tiny_and_special_values_through_every_kernel(comp):
     """Round-after-every-pair bf16 under avx512bf where the fp32 sum or product is a denormal: VCVTNEPS2BF16 reads it
     as zero (the result is a signed zero), and a value just under the smallest normal must not round up to it.  Every
