@@ -48,7 +48,7 @@ WORKLOADS = {
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two runs), each scaled by what the
 # same counter reads for a plain copy of known size (x2.0000 and x1.0000); the summary is kept under profiles/.
 MEASURED_TRAFFIC_BYTES = {"c5_bf16": (15_684_420 + 1_963_194) * 1024,
-                          "rw_8to8_bf16": (8_388_971 + 8_396_410) * 1024, "write_1to7_bf16": (1_048_873 + 7_346_091) * 1024}
+                          "rw_8to8_bf16": (8_388_986 + 8_396_252) * 1024, "write_1to7_bf16": (1_048_613 + 7_341_101) * 1024}
 
 
 def make_buffers(torch, w, seed):

@@ -136,6 +136,9 @@ static hipError_t dispatch(int dtype, bool keep, int bf16_impl, const LaunchArgs
     }
 }
 
+static int launch_copy(const void* in, void* out, size_t bytes, bool nontemporal, hipStream_t stream);
+static int launch_broadcast(const void* in, void* const* dsts, int m, size_t bytes, hipStream_t stream);
+
 static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void* const* dsts, int m, size_t count,
                          int lp_mode, int bf16_impl, void* stream) {
     if (count == 0)
@@ -162,6 +165,14 @@ static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void
     for (int j = 0; j < n; j++)
         if (!srcs[j] || ((uintptr_t)srcs[j] % esz) != 0)
             return MI_CCL_INVALID_ARGUMENTS;
+
+    // one input, rounded after every pair: a chain of zero pairwise steps hands the input back as it is, whatever
+    // the type -- a copy to one buffer or a broadcast to several
+    if (n == 1 && !keep && current_tuning().variant == 0) {
+        if (m == 1)
+            return dsts[0] == srcs[0] ? MI_CCL_SUCCESS : launch_copy(srcs[0], dsts[0], count * esz, true, (hipStream_t)stream);
+        return launch_broadcast(srcs[0], dsts, m, count * esz, (hipStream_t)stream);
+    }
 
     LaunchArgs a;
     a.srcs = srcs;
@@ -218,6 +229,33 @@ copy_kernel(const unsigned char* in, unsigned char* out, uint32_t head, uint64_t
         uint32_t t = threadIdx.x;
         uint64_t i = (t < head) ? t : (uint64_t)head + nvec * 16 + (t - head);
         out[i] = in[i];
+    }
+}
+
+// One buffer written to m buffers (the shape of write_monolithic_kernel_N, kernels.cl:423-560).  A wave does one load
+// and one store, like the copy; a block serves one destination.  The source is taken in sections of kBcastSect
+// 4 KiB tiles: all tiles of a section go to the first destination, then all of them to the second, and so on, so
+// that every destination sees one ascending stream of writes while the section is re-read from the L2 caches (a
+// tile is always handled on the same XCD: sections are a multiple of eight tiles, and blocks go to the XCDs
+// round-robin).  Sections of 4 to 24 MiB measure 6.4-6.5 TB/s for 1 -> 7 at 1 GiB; 32 MiB no longer fits (4.2), and
+// a wave that stores its vector to all seven destinations itself measures 5.5.
+constexpr uint32_t kBcastSect = 4096;       // tiles of kBlock vectors per section: 16 MiB
+
+__global__ void __launch_bounds__(kBlock)
+broadcast_kernel(const unsigned char* in, DstTable d, int m, uint32_t head, uint64_t nvec, uint32_t tail, uint32_t sect_tiles) {
+    const uint32_t per = sect_tiles * (uint32_t)m;          // blocks per section
+    const uint32_t sect = blockIdx.x / per, r = blockIdx.x - sect * per;
+    const uint32_t k = r / sect_tiles, t = r - k * sect_tiles;
+    const uint64_t i = ((uint64_t)sect * sect_tiles + t) * kBlock + threadIdx.x;
+    if (i < nvec) {
+        const u32x4 v = *((const u32x4_u*)(in + head) + i);         // cached: the other destinations read it again
+        st_loose((u32x4_u*)((unsigned char*)d.p[k] + head) + i, v);
+    }
+    if (blockIdx.x == 0 && threadIdx.x < head + tail) {
+        const uint32_t e = threadIdx.x;
+        const uint64_t b = (e < head) ? e : (uint64_t)head + nvec * 16 + (e - head);
+        const unsigned char x = in[b];
+        for (int q = 0; q < m; q++) ((unsigned char*)d.p[q])[b] = x;
     }
 }
 
@@ -418,11 +456,10 @@ int mi_ccl_comp_batch_reduce(const void* in_buf, const size_t* offsets, size_t n
     return reduce_n_impl(dtype, op, srcs, (int)n_offsets, &inout, 1, count, lp, bf16_impl, stream);
 }
 
-int mi_ccl_comp_copy(const void* in, void* out, size_t bytes, int use_nontemporal, void* stream) {
-    if (bytes == 0)
-        return MI_CCL_SUCCESS;
-    if (!in || !out)
-        return MI_CCL_INVALID_ARGUMENTS;
+} /* extern "C" */
+
+namespace mi {
+static int launch_copy(const void* in, void* out, size_t bytes, bool nontemporal, hipStream_t stream) {
     const uintptr_t mis = (uintptr_t)out & 15u;
     uint64_t head = mis ? 16u - mis : 0;
     if (head > bytes)
@@ -433,13 +470,48 @@ int mi_ccl_comp_copy(const void* in, void* out, size_t bytes, int use_nontempora
     if (blocks > 0x7fffffffu)
         blocks = 0x7fffffffu;      // beyond 8 TiB the kernel strides
     const unsigned grid = (unsigned)(blocks ? blocks : 1);
-    if (use_nontemporal)
-        hipLaunchKernelGGL(copy_kernel<true>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream,
-                           (const unsigned char*)in, (unsigned char*)out, (uint32_t)head, nvec, tail);
+    if (nontemporal)
+        hipLaunchKernelGGL(copy_kernel<true>, dim3(grid), dim3(kBlock), 0, stream, (const unsigned char*)in,
+                           (unsigned char*)out, (uint32_t)head, nvec, tail);
     else
-        hipLaunchKernelGGL(copy_kernel<false>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream,
-                           (const unsigned char*)in, (unsigned char*)out, (uint32_t)head, nvec, tail);
+        hipLaunchKernelGGL(copy_kernel<false>, dim3(grid), dim3(kBlock), 0, stream, (const unsigned char*)in,
+                           (unsigned char*)out, (uint32_t)head, nvec, tail);
     return status_of(hipGetLastError());
+}
+
+// m >= 2 destinations; the vectors start where the first destination reaches a 16-byte boundary
+static int launch_broadcast(const void* in, void* const* dsts, int m, size_t bytes, hipStream_t stream) {
+    DstTable d;
+    for (int k = 0; k < kMaxDsts; k++) d.p[k] = dsts[k < m ? k : 0];
+    const uintptr_t mis = (uintptr_t)dsts[0] & 15u;
+    uint64_t head = mis ? 16u - mis : 0;
+    if (head > bytes)
+        head = bytes;
+    const uint64_t nvec = (bytes - head) / 16;
+    const uint32_t tail = (uint32_t)(bytes - head - nvec * 16);
+    uint64_t tiles = (nvec + kBlock - 1) / kBlock;
+    if (tiles == 0)
+        tiles = 1;
+    const uint32_t sect_tiles = tiles < kBcastSect ? (uint32_t)((tiles + 7) & ~7ull) : kBcastSect;
+    const uint64_t sects = (tiles + sect_tiles - 1) / sect_tiles;
+    const uint64_t blocks = sects * sect_tiles * (uint64_t)m;
+    if (blocks > 0x7fffffffu)
+        return MI_CCL_INVALID_ARGUMENTS;       // more than 8 TiB of destinations
+    hipLaunchKernelGGL(broadcast_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, (const unsigned char*)in, d, m,
+                       (uint32_t)head, nvec, tail, sect_tiles);
+    return status_of(hipGetLastError());
+}
+
+}  // namespace mi
+
+extern "C" {
+
+int mi_ccl_comp_copy(const void* in, void* out, size_t bytes, int use_nontemporal, void* stream) {
+    if (bytes == 0)
+        return MI_CCL_SUCCESS;
+    if (!in || !out)
+        return MI_CCL_INVALID_ARGUMENTS;
+    return launch_copy(in, out, bytes, use_nontemporal != 0, (hipStream_t)stream);
 }
 
 int mi_ccl_convert_fp32_to_bf16_arrays(const void* fp32_buf, void* bf16_buf, size_t count, int bf16_impl,

@@ -64,6 +64,44 @@ def test_one_input_is_a_byte_copy_for_every_dtype(comp):
             assert (o.cpu().numpy() == src).all(), O.DTYPE_NAMES[dtype]
 
 
+def test_broadcast_sections_alignments_and_aliasing(comp):
+    """One input to m buffers by the sectioned broadcast kernel (and to one buffer by the copy kernel): sizes below
+    one tile, around the 16 MiB section and over several sections, 1 to 16 destinations, the source and every
+    destination at its own offset from a 16-byte boundary, one destination being the source itself; nothing outside
+    the destinations is written."""
+    import torch
+    rng = np.random.default_rng(12)
+    pad = 64
+    sect = 16 << 20
+    for nbytes, ms in ((1, (1, 2, 16)), (15, (2,)), (4095, (1, 3)), (100_003, (1, 2, 7)), (sect - 16, (2,)),
+                       (sect + 4096 + 5, (1, 3)), (3 * sect + 12_345, (2, 7)), (200_000_001, (5,))):
+        src = rng.integers(0, 256, nbytes + 2 * pad, dtype=np.uint8)
+        d = torch.from_numpy(src.copy()).cuda()
+        for m in ms:
+            for trial in range(2):
+                sh = [int(x) for x in rng.integers(0, 16, m + 1)] if trial else [0] * (m + 1)
+                outs = [torch.zeros(nbytes + 2 * pad, dtype=torch.uint8, device="cuda") for _ in range(m)]
+                comp.comp_reduce_write_n(O.UINT8, O.SUM, [d.data_ptr() + pad + sh[0]],
+                                         [o.data_ptr() + pad + k for o, k in zip(outs, sh[1:])], nbytes)
+                torch.cuda.synchronize()
+                want = src[pad + sh[0]:pad + sh[0] + nbytes]
+                for o, k in zip(outs, sh[1:]):
+                    g = o.cpu().numpy()
+                    assert (g[pad + k:pad + k + nbytes] == want).all(), (nbytes, m, sh)
+                    assert not g[:pad + k].any() and not g[pad + k + nbytes:].any(), (nbytes, m, sh)
+                del outs
+        # the source among the destinations, with a wider type
+        if nbytes % 4 == 0 or nbytes > 1000:
+            cnt = nbytes // 4
+            d32 = torch.from_numpy(src[:cnt * 4].copy()).cuda()
+            o1, o2 = torch.zeros_like(d32), torch.zeros_like(d32)
+            comp.comp_reduce_write_n(O.FLOAT32, O.MAX, [d32], [o1, d32, o2], cnt)
+            torch.cuda.synchronize()
+            for o in (o1, d32, o2):
+                assert (o.cpu().numpy() == src[:cnt * 4]).all(), (nbytes, "aliased")
+        del d
+
+
 @pytest.mark.parametrize("variant", [2, 8])
 def test_destination_aliases_a_source_and_misaligned_buffers(comp, variant):
     """In place (destination k is source j, as allreduce_kernel's output may be its input), buffers that share a
