@@ -168,7 +168,8 @@ static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void
 
     // one input, rounded after every pair: a chain of zero pairwise steps hands the input back as it is, whatever
     // the type -- a copy to one buffer or a broadcast to several
-    if (n == 1 && !keep && current_tuning().variant == 0) {
+    const Tuning tune = current_tuning();
+    if (n == 1 && !keep && tune.variant == 0) {
         if (m == 1)
             return dsts[0] == srcs[0] ? MI_CCL_SUCCESS : launch_copy(srcs[0], dsts[0], count * esz, true, (hipStream_t)stream);
         return launch_broadcast(srcs[0], dsts, m, count * esz, (hipStream_t)stream);
@@ -183,7 +184,7 @@ static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void
     a.count = count;
     a.op = op;
     a.stream = (hipStream_t)stream;
-    a.tune = current_tuning();
+    a.tune = tune;
 
     // keep-precision under avx512bf: the reference narrows the last count % 16 elements by truncation
     // (src/comp/bf16/bf16.cpp:144-148).  Those <= 15 elements get a launch of the truncating traits.
