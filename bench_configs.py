@@ -170,6 +170,12 @@ def main():
         add("convert fp32 -> bf16 (round to nearest even), 2^28 elements", us, 6 * nc)
         us = timed(torch, lambda i: comp.convert_bf16_to_fp32_arrays(b16, f32, nc), 20, 5)
         add("convert bf16 -> fp32, 2^28 elements", us, 6 * nc)
+        f16 = torch.empty(nc, dtype=torch.float16, device="cuda")
+        us = timed(torch, lambda i: comp.convert_fp32_to_fp16_arrays(f32, f16, nc), 20, 5)
+        add("convert fp32 -> fp16, 2^28 elements", us, 6 * nc)
+        us = timed(torch, lambda i: comp.convert_fp16_to_fp32_arrays(f16, f32, nc), 20, 5)
+        add("convert fp16 -> fp32, 2^28 elements", us, 6 * nc)
+        del f16
         del f32, b16
     # ---- C4
     rng = np.random.default_rng(4)

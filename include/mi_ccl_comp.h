@@ -138,6 +138,14 @@ int mi_ccl_convert_fp32_to_bf16_arrays(const void* fp32_buf, void* bf16_buf, siz
                                        void* stream);
 int mi_ccl_convert_bf16_to_fp32_arrays(const void* bf16_buf, void* fp32_buf, size_t count, void* stream);
 
+/* The reference's fp16 converters, ccl_convert_fp32_to_fp16 / ccl_convert_fp16_to_fp32 (src/comp/fp16/fp16.cpp:55-61),
+ * convert one vector of eight values (VCVTPS2PH round-to-nearest-even / VCVTPH2PS); these convert count values with
+ * the same result per value (subnormals kept, overflow to infinity, a signalling NaN quieted keeping the top of its
+ * payload).  The single-vector ccl_convert_fp32_to_bf16 / ccl_convert_bf16_to_fp32 (bf16.cpp:113-127) are the bf16
+ * array converters above with count = 16. */
+int mi_ccl_convert_fp32_to_fp16_arrays(const void* fp32_buf, void* fp16_buf, size_t count, void* stream);
+int mi_ccl_convert_fp16_to_fp32_arrays(const void* fp16_buf, void* fp32_buf, size_t count, void* stream);
+
 /* ---- fusion buffer ------------------------------------------------------------------------------ */
 
 /* Byte offset of each of k tensors in a fusion buffer: running offset in queue order, every start

@@ -25,7 +25,8 @@ EXPORTS = [
     "mi_ccl_datatype_size", "mi_ccl_datatype_name", "mi_ccl_reduction_to_str", "mi_ccl_status_str",
     "mi_ccl_kernel_name", "mi_ccl_comp_reduce", "mi_ccl_bf16_reduce", "mi_ccl_fp16_reduce",
     "mi_ccl_comp_reduce_n", "mi_ccl_comp_reduce_write_n", "mi_ccl_comp_batch_reduce", "mi_ccl_comp_copy",
-    "mi_ccl_convert_fp32_to_bf16_arrays", "mi_ccl_convert_bf16_to_fp32_arrays", "mi_ccl_fusion_offsets",
+    "mi_ccl_convert_fp32_to_bf16_arrays", "mi_ccl_convert_bf16_to_fp32_arrays",
+    "mi_ccl_convert_fp32_to_fp16_arrays", "mi_ccl_convert_fp16_to_fp32_arrays", "mi_ccl_fusion_offsets",
     "mi_ccl_fusion_plan_create", "mi_ccl_fusion_plan_destroy", "mi_ccl_fusion_plan_bytes",
     "mi_ccl_fusion_plan_offset", "mi_ccl_fusion_pack", "mi_ccl_fusion_unpack", "mi_ccl_fusion_reduce",
     "mi_ccl_set_param", "mi_ccl_get_param",
@@ -66,6 +67,8 @@ def lib():
     L.mi_ccl_comp_copy.argtypes = [vp, vp, sz, i, vp]
     L.mi_ccl_convert_fp32_to_bf16_arrays.argtypes = [vp, vp, sz, i, vp]
     L.mi_ccl_convert_bf16_to_fp32_arrays.argtypes = [vp, vp, sz, vp]
+    L.mi_ccl_convert_fp32_to_fp16_arrays.argtypes = [vp, vp, sz, vp]
+    L.mi_ccl_convert_fp16_to_fp32_arrays.argtypes = [vp, vp, sz, vp]
     L.mi_ccl_fusion_offsets.argtypes = [vp, sz, sz, sz, vp, vp]
     L.mi_ccl_fusion_plan_create.argtypes = [vp, sz, i, sz, C.POINTER(vp)]
     L.mi_ccl_fusion_plan_destroy.argtypes = [vp]
@@ -176,6 +179,16 @@ def comp_copy(inp, out, nbytes, use_nontemporal=False, stream=None):
 def convert_fp32_to_bf16_arrays(fp32_buf, bf16_buf, count, bf16_impl=BF16_AVX512BF, stream=None):
     _check(lib().mi_ccl_convert_fp32_to_bf16_arrays(_ptr(fp32_buf), _ptr(bf16_buf), count, bf16_impl,
                                                     _stream(stream)), "mi_ccl_convert_fp32_to_bf16_arrays")
+
+
+def convert_fp32_to_fp16_arrays(fp32_buf, fp16_buf, count, stream=None):
+    _check(lib().mi_ccl_convert_fp32_to_fp16_arrays(_ptr(fp32_buf), _ptr(fp16_buf), count, _stream(stream)),
+           "mi_ccl_convert_fp32_to_fp16_arrays")
+
+
+def convert_fp16_to_fp32_arrays(fp16_buf, fp32_buf, count, stream=None):
+    _check(lib().mi_ccl_convert_fp16_to_fp32_arrays(_ptr(fp16_buf), _ptr(fp32_buf), count, _stream(stream)),
+           "mi_ccl_convert_fp16_to_fp32_arrays")
 
 
 def convert_bf16_to_fp32_arrays(bf16_buf, fp32_buf, count, stream=None):

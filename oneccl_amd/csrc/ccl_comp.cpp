@@ -207,6 +207,34 @@ void ccl_convert_bf16_to_fp32_arrays(void* bf16_buf, float* fp32_buf, size_t cou
               "ccl_convert_bf16_to_fp32_arrays");
 }
 
+void ccl_convert_fp32_to_bf16(const void* src, void* dst, ccl_sched* sched) {
+    // bf16.cpp:113-123: the avx512bf store when that implementation is selected, the truncating one otherwise
+    const int impl = ccl::global_data::env().bf16_impl_type == ccl_bf16_avx512bf ? MI_CCL_BF16_AVX512BF : MI_CCL_BF16_AVX512F;
+    to_status(mi_ccl_convert_fp32_to_bf16_arrays(src, dst, 16, impl, stream_of(sched)), "ccl_convert_fp32_to_bf16");
+}
+
+void ccl_convert_bf16_to_fp32(const void* src, void* dst, ccl_sched* sched) {
+    to_status(mi_ccl_convert_bf16_to_fp32_arrays(src, dst, 16, stream_of(sched)), "ccl_convert_bf16_to_fp32");
+}
+
+void ccl_convert_fp32_to_fp16(const void* src, void* dst, ccl_sched* sched) {
+    to_status(mi_ccl_convert_fp32_to_fp16_arrays(src, dst, 8, stream_of(sched)), "ccl_convert_fp32_to_fp16");
+}
+
+void ccl_convert_fp16_to_fp32(const void* src, void* dst, ccl_sched* sched) {
+    to_status(mi_ccl_convert_fp16_to_fp32_arrays(src, dst, 8, stream_of(sched)), "ccl_convert_fp16_to_fp32");
+}
+
+void ccl_convert_fp32_to_fp16_arrays(const void* fp32_buf, void* fp16_buf, size_t count, ccl_sched* sched) {
+    to_status(mi_ccl_convert_fp32_to_fp16_arrays(fp32_buf, fp16_buf, count, stream_of(sched)),
+              "ccl_convert_fp32_to_fp16_arrays");
+}
+
+void ccl_convert_fp16_to_fp32_arrays(const void* fp16_buf, float* fp32_buf, size_t count, ccl_sched* sched) {
+    to_status(mi_ccl_convert_fp16_to_fp32_arrays(fp16_buf, fp32_buf, count, stream_of(sched)),
+              "ccl_convert_fp16_to_fp32_arrays");
+}
+
 ccl::status ccl_comp_reduce_n(ccl_sched* sched, const void* own_buf, const std::vector<const void*>& peer_bufs,
                               size_t count, void* out_buf, const ccl_datatype& dtype, ccl::reduction reduction,
                               int bf16_keep_precision_mode) {

@@ -168,6 +168,15 @@ void ccl_fp16_reduce(const void* in_buf, size_t in_cnt, void* inout_buf, size_t*
                      ccl_sched* sched = nullptr);
 void ccl_convert_fp32_to_bf16_arrays(void* fp32_buf, void* bf16_buf, size_t count, ccl_sched* sched = nullptr);
 void ccl_convert_bf16_to_fp32_arrays(void* bf16_buf, float* fp32_buf, size_t count, ccl_sched* sched = nullptr);
+// One vector of 16 (bf16.cpp:113-127) or 8 (fp16.cpp:55-61) values, as the reference's functions of these names
+// convert; the bf16 narrowing follows CCL_BF16 (avx512bf rounds to nearest even, anything else truncates).
+void ccl_convert_fp32_to_bf16(const void* src, void* dst, ccl_sched* sched = nullptr);
+void ccl_convert_bf16_to_fp32(const void* src, void* dst, ccl_sched* sched = nullptr);
+void ccl_convert_fp32_to_fp16(const void* src, void* dst, ccl_sched* sched = nullptr);
+void ccl_convert_fp16_to_fp32(const void* src, void* dst, ccl_sched* sched = nullptr);
+// count values at a time (no counterpart of these names in the reference; same result per value)
+void ccl_convert_fp32_to_fp16_arrays(const void* fp32_buf, void* fp16_buf, size_t count, ccl_sched* sched = nullptr);
+void ccl_convert_fp16_to_fp32_arrays(const void* fp16_buf, float* fp32_buf, size_t count, ccl_sched* sched = nullptr);
 
 // The N-input local reduce of the device path (reduce_monolithic_kernel_N and friends, src/kernels/kernels.cl:269-421):
 // out = own OP peers[0] OP peers[1] ..., own first, peers in argument order.  keep_precision as in batch reduce.

@@ -349,6 +349,51 @@ bf16_to_f32_kernel(const uint16_t* in, uint32_t* out, uint32_t head, uint64_t nq
     }
 }
 
+// fp32 <-> fp16 with the same shapes (the reference converts one vector of eight with VCVTPS2PH imm 0 / VCVTPH2PS,
+// src/comp/fp16/fp16.cpp:55-61): the hardware conversions round to nearest even, keep subnormals and quiet a
+// signalling NaN keeping the top of its payload, as the x86 instructions do.
+__global__ void __launch_bounds__(kBlock)
+f32_to_f16_kernel(const uint32_t* in, uint16_t* out, uint32_t head, uint64_t noct, uint32_t tail) {
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    const u32x4_u* s = (const u32x4_u*)(in + head);
+    u32x4_u* d = (u32x4_u*)(out + head);
+    const uint64_t o = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (o < noct) {
+        const u32x4 x0 = ld_loose(s + 2 * o), x1 = ld_loose(s + 2 * o + 1);
+        u32x4 r;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const u32x4& x = (k < 2) ? x0 : x1;
+            const half2_t h = { (_Float16)as_f32(x[(2 * k) & 3]), (_Float16)as_f32(x[(2 * k + 1) & 3]) };
+            r[k] = __builtin_bit_cast(uint32_t, h);
+        }
+        st_loose(d + o, r);
+    }
+    if (blockIdx.x == 0 && threadIdx.x < head + tail) {
+        const uint32_t t = threadIdx.x;
+        const uint64_t i = (t < head) ? t : (uint64_t)head + noct * 8 + (t - head);
+        out[i] = __builtin_bit_cast(uint16_t, (_Float16)as_f32(in[i]));
+    }
+}
+
+__global__ void __launch_bounds__(kBlock)
+f16_to_f32_kernel(const uint16_t* in, uint32_t* out, uint32_t head, uint64_t nquad, uint32_t tail) {
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    const u32x2_u* s = (const u32x2_u*)(in + head);
+    u32x4_u* d = (u32x4_u*)(out + head);
+    const uint64_t q = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (q < nquad) {
+        const u32x2 x = __builtin_nontemporal_load(s + q);
+        const half2_t a = __builtin_bit_cast(half2_t, (uint32_t)x[0]), b = __builtin_bit_cast(half2_t, (uint32_t)x[1]);
+        st_loose(d + q, u32x4{ as_u32((float)a[0]), as_u32((float)a[1]), as_u32((float)b[0]), as_u32((float)b[1]) });
+    }
+    if (blockIdx.x == 0 && threadIdx.x < head + tail) {
+        const uint32_t t = threadIdx.x;
+        const uint64_t i = (t < head) ? t : (uint64_t)head + nquad * 4 + (t - head);
+        out[i] = as_u32((float)__builtin_bit_cast(_Float16, in[i]));
+    }
+}
+
 // launch geometry of the two converters: `out_elem` bytes per element of the output array, `per` elements per group,
 // `unroll` groups per lane
 struct CvtShape {
@@ -546,6 +591,32 @@ int mi_ccl_convert_bf16_to_fp32_arrays(const void* bf16_buf, void* fp32_buf, siz
     const CvtShape c = cvt_shape(fp32_buf, 4, count, 4, kWidenUnroll);
     hipLaunchKernelGGL(bf16_to_f32_kernel, dim3(c.grid), dim3(kBlock), 0, (hipStream_t)stream,
                        (const uint16_t*)bf16_buf, (uint32_t*)fp32_buf, c.head, c.ngroup, c.tail);
+    return status_of(hipGetLastError());
+}
+
+int mi_ccl_convert_fp32_to_fp16_arrays(const void* fp32_buf, void* fp16_buf, size_t count, void* stream) {
+    if (count == 0)
+        return MI_CCL_SUCCESS;
+    if (!fp32_buf || !fp16_buf || ((uintptr_t)fp32_buf & 3u) || ((uintptr_t)fp16_buf & 1u))
+        return MI_CCL_INVALID_ARGUMENTS;
+    if (count / 8 / kBlock >= 0x7fffffffu)
+        return MI_CCL_INVALID_ARGUMENTS;
+    const CvtShape c = cvt_shape(fp16_buf, 2, count, 8, 1);
+    hipLaunchKernelGGL(f32_to_f16_kernel, dim3(c.grid), dim3(kBlock), 0, (hipStream_t)stream, (const uint32_t*)fp32_buf,
+                       (uint16_t*)fp16_buf, c.head, c.ngroup, c.tail);
+    return status_of(hipGetLastError());
+}
+
+int mi_ccl_convert_fp16_to_fp32_arrays(const void* fp16_buf, void* fp32_buf, size_t count, void* stream) {
+    if (count == 0)
+        return MI_CCL_SUCCESS;
+    if (!fp32_buf || !fp16_buf || ((uintptr_t)fp32_buf & 3u) || ((uintptr_t)fp16_buf & 1u))
+        return MI_CCL_INVALID_ARGUMENTS;
+    if (count / 4 / kBlock >= 0x7fffffffu)
+        return MI_CCL_INVALID_ARGUMENTS;
+    const CvtShape c = cvt_shape(fp32_buf, 4, count, 4, 1);
+    hipLaunchKernelGGL(f16_to_f32_kernel, dim3(c.grid), dim3(kBlock), 0, (hipStream_t)stream, (const uint16_t*)fp16_buf,
+                       (uint32_t*)fp32_buf, c.head, c.ngroup, c.tail);
     return status_of(hipGetLastError());
 }
 

@@ -22,6 +22,7 @@
  *   orc_comp_reduce plain types     IEEE single op per pair / two's-complement wrap: numpy closed forms,
  *                                   min/max truth table recorded from the reference library
  *   orc_convert_*_arrays tail       recorded probe values of the reference library (tail truncation)
+ *   orc_convert_fp32_to_fp16_arrays / fp16_to_fp32: loops over orc_fp16_narrow / orc_fp16_widen (pinned above)
  *   orc_comp_batch_reduce           composition; recorded probe values (1+3*2^-8 -> 3f82 body / 3f81 tail); the
  *                                   keep-precision sum against the reference's own 16-wide converters called in
  *                                   the reference's pass order (oracle/_ref, ref_batch_reduce_keep_sum) on random
@@ -302,6 +303,19 @@ void orc_convert_bf16_to_fp32_arrays(const void* bf16_buf, void* fp32_buf, size_
     uint32_t* dst = (uint32_t*)fp32_buf;
     (void)bf16_impl;
     for (size_t i = 0; i < count; i++) dst[i] = orc_bf16_widen(src[i]);
+}
+
+/* ccl_convert_fp32_to_fp16 / ccl_convert_fp16_to_fp32, fp16.cpp:55-61: the reference converts one vector of eight
+ * values with VCVTPS2PH (imm 0: round to nearest even) / VCVTPH2PS; here for count values. */
+void orc_convert_fp32_to_fp16_arrays(const void* fp32_buf, void* fp16_buf, size_t count) {
+    const uint32_t* src = (const uint32_t*)fp32_buf;
+    uint16_t* dst = (uint16_t*)fp16_buf;
+    for (size_t i = 0; i < count; i++) dst[i] = orc_fp16_narrow(src[i]);
+}
+void orc_convert_fp16_to_fp32_arrays(const void* fp16_buf, void* fp32_buf, size_t count) {
+    const uint16_t* src = (const uint16_t*)fp16_buf;
+    uint32_t* dst = (uint32_t*)fp32_buf;
+    for (size_t i = 0; i < count; i++) dst[i] = orc_fp16_widen(src[i]);
 }
 
 /* ------------------------------------------------------------------------------------------ */

@@ -47,6 +47,8 @@ uint16_t orc_fp16_narrow(uint32_t u);         /* fp16_intrisics.hpp:103 (VCVTPS2
 /* array converters with the scalar truncating tail, bf16.cpp:130-169 */
 void orc_convert_fp32_to_bf16_arrays(const void* fp32_buf, void* bf16_buf, size_t count, int bf16_impl);
 void orc_convert_bf16_to_fp32_arrays(const void* bf16_buf, void* fp32_buf, size_t count, int bf16_impl);
+void orc_convert_fp32_to_fp16_arrays(const void* fp32_buf, void* fp16_buf, size_t count);   /* fp16.cpp:55-57, per value */
+void orc_convert_fp16_to_fp32_arrays(const void* fp16_buf, void* fp32_buf, size_t count);   /* fp16.cpp:59-61 */
 
 /* pairwise in-place primitives */
 void orc_bf16_reduce(const void* in, size_t count, void* inout, int op, int bf16_impl); /* bf16.cpp:87-110 */

@@ -218,6 +218,33 @@ int main() {
         bool ok = true;
         for (int i = 0; i < 22; i++) ok = ok && w[i] == ((uint32_t)h[i] << 16);
         EXPECT(ok, "bf16->fp32 arrays");
+        // the single-vector converters of the reference: 16 values (bf16), 8 values (fp16); the value after the vector
+        // stays untouched
+        std::vector<uint32_t> v(17, 0x3f808000u);
+        v[1] = 0x007fffffu; v[2] = 0x7f800001u; v[3] = 0x477fe000u; v[4] = 0x33000000u; v[5] = 0x38800000u; v[6] = 0xc77ff000u;
+        DevBuf<uint32_t> dv(v); DevBuf<uint16_t> d16(std::vector<uint16_t>(17, 0xabcd));
+        ccl_convert_fp32_to_bf16(dv.p, d16.p, &sched);
+        std::vector<uint16_t> g16 = d16.host(), w16(16);
+        const int impl = (int)ccl::global_data::env().bf16_impl_type;
+        orc_convert_fp32_to_bf16_arrays(v.data(), w16.data(), 16, impl == ORC_BF16_AVX512BF ? ORC_BF16_AVX512BF : ORC_BF16_AVX512F);
+        EXPECT(memcmp(g16.data(), w16.data(), 32) == 0 && g16[16] == 0xabcd, "ccl_convert_fp32_to_bf16 (16 values)");
+        DevBuf<uint32_t> d32(std::vector<uint32_t>(17, 0xabcdabcdu));
+        ccl_convert_bf16_to_fp32(d16.p, d32.p, &sched);
+        std::vector<uint32_t> g32 = d32.host();
+        ok = g32[16] == 0xabcdabcdu;
+        for (int i = 0; i < 16; i++) ok = ok && g32[i] == ((uint32_t)g16[i] << 16);
+        EXPECT(ok, "ccl_convert_bf16_to_fp32 (16 values)");
+        DevBuf<uint16_t> dh16(std::vector<uint16_t>(9, 0xabcd));
+        ccl_convert_fp32_to_fp16(dv.p, dh16.p, &sched);
+        std::vector<uint16_t> gh = dh16.host(), wh(8);
+        orc_convert_fp32_to_fp16_arrays(v.data(), wh.data(), 8);
+        EXPECT(memcmp(gh.data(), wh.data(), 16) == 0 && gh[8] == 0xabcd, "ccl_convert_fp32_to_fp16 (8 values): %04x %04x %04x %04x %04x %04x %04x",
+               gh[0], gh[1], gh[2], gh[3], gh[4], gh[5], gh[6]);
+        DevBuf<uint32_t> dback(std::vector<uint32_t>(9, 0xabcdabcdu));
+        ccl_convert_fp16_to_fp32(dh16.p, dback.p, &sched);
+        std::vector<uint32_t> gb = dback.host(), wb(8);
+        orc_convert_fp16_to_fp32_arrays(gh.data(), wb.data(), 8);
+        EXPECT(memcmp(gb.data(), wb.data(), 32) == 0 && gb[8] == 0xabcdabcdu, "ccl_convert_fp16_to_fp32 (8 values)");
     }
     // float16 implementation knob (fp16_utils.hpp:26-32): avx512f quiets a signalling NaN that min hands back, avx512fp16
     // keeps it, and a value that names no implementation makes the reduce a no-op, as in the reference (probe values

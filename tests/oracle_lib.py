@@ -61,6 +61,8 @@ def lib():
             getattr(L, f).argtypes = [C.c_uint32]
         L.orc_convert_fp32_to_bf16_arrays.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
         L.orc_convert_bf16_to_fp32_arrays.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        L.orc_convert_fp32_to_fp16_arrays.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        L.orc_convert_fp16_to_fp32_arrays.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         L.orc_bf16_reduce.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int]
         L.orc_fp16_reduce.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int]
         L.orc_comp_reduce.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]

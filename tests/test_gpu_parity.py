@@ -275,6 +275,52 @@ def test_copy_and_converters(comp):
             assert not got[:so].any() and not got[so + count:].any(), (count, si, so)
 
 
+def test_fp16_converters_exhaustive_on_gpu(comp):
+    """fp32 -> fp16 for all 2^32 patterns and fp16 -> fp32 for all 2^16, against the oracle (itself exhaustively equal
+    to VCVTPS2PH imm 0 / VCVTPH2PS, which the reference's ccl_convert_fp32_to_fp16 / ccl_convert_fp16_to_fp32 are);
+    then both directions with the two arrays at different alignments and odd counts."""
+    import torch
+    L = O.lib()
+    chunk = 1 << 27
+    d_out = torch.empty(chunk, dtype=torch.int16, device="cuda")
+    want = np.empty(chunk, np.uint16)
+    for c in range(0, 1 << 32, chunk):
+        x = torch.arange(c, c + chunk, dtype=torch.int64, device="cuda")
+        src = torch.where(x >= 2**31, x - 2**32, x).to(torch.int32)
+        comp.convert_fp32_to_fp16_arrays(src, d_out, chunk)
+        torch.cuda.synchronize()
+        host = np.arange(c, c + chunk, dtype=np.uint64).astype(np.uint32)
+        L.orc_convert_fp32_to_fp16_arrays(host.ctypes.data, want.ctypes.data, chunk)
+        got = to_host(d_out, np.uint16)
+        assert (got == want).all(), hex(c + int(np.flatnonzero(got != want)[0]))
+    h = np.arange(65536, dtype=np.uint16)
+    w = np.empty(65536, np.uint32)
+    L.orc_convert_fp16_to_fp32_arrays(h.ctypes.data, w.ctypes.data, 65536)
+    d = to_dev(np.zeros(65536, np.uint32))
+    comp.convert_fp16_to_fp32_arrays(to_dev(h), d, 65536)
+    torch.cuda.synchronize()
+    assert (to_host(d, np.uint32) == w).all()
+    rng = np.random.default_rng(23)
+    for count in (1, 7, 8, 29, 70_001):
+        for si, so in ((0, 0), (1, 3), (3, 6)):
+            f32 = rng.integers(0, 2**32, count + 16, dtype=np.uint32)
+            want = np.empty(count, np.uint16)
+            L.orc_convert_fp32_to_fp16_arrays(f32[si:].ctypes.data, want.ctypes.data, count)
+            d, src_d = to_dev(np.zeros(count + 16, np.uint16)), to_dev(f32)
+            comp.convert_fp32_to_fp16_arrays(src_d.data_ptr() + 4 * si, d.data_ptr() + 2 * so, count)
+            torch.cuda.synchronize()
+            got = to_host(d, np.uint16)
+            assert (got[so:so + count] == want).all() and not got[:so].any() and not got[so + count:].any(), (count, si, so)
+            h16 = rng.integers(0, 65536, count + 16, dtype=np.uint16)
+            want32 = np.empty(count, np.uint32)
+            L.orc_convert_fp16_to_fp32_arrays(h16[si:].ctypes.data, want32.ctypes.data, count)
+            d, src_d = to_dev(np.zeros(count + 16, np.uint32)), to_dev(h16)
+            comp.convert_fp16_to_fp32_arrays(src_d.data_ptr() + 2 * si, d.data_ptr() + 4 * so, count)
+            torch.cuda.synchronize()
+            got = to_host(d, np.uint32)
+            assert (got[so:so + count] == want32).all() and not got[:so].any() and not got[so + count:].any(), (count, si, so)
+
+
 def test_bf16_narrowing_exhaustive_on_gpu(comp):
     """All 2^32 fp32 patterns through the GPU's round-to-nearest-even narrowing vs the oracle (itself
     exhaustively equal to VCVTNEPS2BF16).  The kernel converts pairs with the packed hardware conversion, so every

@@ -192,6 +192,28 @@ def test_fp16_converters_vs_numpy_float16():
     assert (got16[finite] == want16[finite]).all()
 
 
+def test_fp16_array_converters_are_the_per_value_converters():
+    """orc_convert_fp32_to_fp16_arrays / orc_convert_fp16_to_fp32_arrays loop over the pinned per-value functions;
+    checked against them and, for finite values, against numpy's independent float16 casts."""
+    rng = np.random.default_rng(17)
+    u = np.concatenate([rng.integers(0, 2**32, 50_000, dtype=np.uint32),
+                        np.array([0, 0x80000000, 1, 0x33000000, 0x33000001, 0x387FFFFF, 0x38800000, 0x477FEFFF, 0x477FF000,
+                                  0x7F800000, 0xFF800000, 0x7F800001, 0x7FC00000, 0xFFFFFFFF], np.uint32)])
+    out = np.empty(u.size, np.uint16)
+    L.orc_convert_fp32_to_fp16_arrays(u.ctypes.data, out.ctypes.data, u.size)
+    assert (out == np.array([L.orc_fp16_narrow(int(x)) for x in u], np.uint16)).all()
+    f = u.view(np.float32)
+    fin = ~np.isnan(f)
+    with np.errstate(over="ignore", invalid="ignore"):
+        assert (out[fin] == f.astype(np.float16).view(np.uint16)[fin]).all()
+    nan_in = ~fin
+    assert ((out[nan_in] & 0x7C00) == 0x7C00).all() and ((out[nan_in] & 0x0200) != 0).all()      # NaN stays NaN, quiet
+    h = np.arange(65536, dtype=np.uint16)
+    w = np.empty(65536, np.uint32)
+    L.orc_convert_fp16_to_fp32_arrays(h.ctypes.data, w.ctypes.data, 65536)
+    assert (w == np.array([L.orc_fp16_widen(int(x)) for x in h], np.uint32)).all()
+
+
 # ----------------------------------------------------------------------------------------------
 # closed forms for the plain types
 
