@@ -28,26 +28,25 @@ void check_hip(hipError_t e, const char* what) {
         fail(std::string(what) + ": " + hipGetErrorString(e));
 }
 
+// the reference's env_2_enum (src/common/env/env_parser.hpp): the value must be one of the table's names
+template <class E>
+bool enum_by_name(const std::map<E, std::string>& names, const char* v, E& out) {
+    for (const auto& kv : names)
+        if (kv.second == v) {
+            out = kv.first;
+            return true;
+        }
+    return false;
+}
+
 ccl::env_data parse_env() {
     ccl::env_data e;
     if (const char* v = getenv("CCL_BF16")) {      // env.cpp:711-713
-        if (!strcmp(v, "scalar"))
-            e.bf16_impl_type = ccl_bf16_scalar;
-        else if (!strcmp(v, "avx512f"))
-            e.bf16_impl_type = ccl_bf16_avx512f;
-        else if (!strcmp(v, "avx512bf"))
-            e.bf16_impl_type = ccl_bf16_avx512bf;
-        else
+        if (!enum_by_name(bf16_impl_names, v, e.bf16_impl_type))
             fail(std::string("unexpected CCL_BF16 value: ") + v);
     }
     if (const char* v = getenv("CCL_FP16")) {      // env.cpp:715-720; f16c and avx512f give the same bits
-        if (!strcmp(v, "f16c"))
-            e.fp16_impl_type = ccl_fp16_f16c;
-        else if (!strcmp(v, "avx512f"))
-            e.fp16_impl_type = ccl_fp16_avx512f;
-        else if (!strcmp(v, "avx512fp16"))
-            e.fp16_impl_type = ccl_fp16_avx512fp16;
-        else
+        if (!enum_by_name(fp16_env_impl_names, v, e.fp16_impl_type))
             fail(std::string("unsupported FP16 impl type: ") + v);
     }
     return e;
@@ -124,6 +123,26 @@ const std::string& ccl_datatype_storage::name(const ccl_datatype& dtype) const {
 
 const char* ccl_reduction_to_str(ccl::reduction type) {
     return mi_ccl_reduction_to_str((int)type);
+}
+
+const std::map<ccl_bf16_impl_type, std::string> bf16_impl_names = { { ccl_bf16_scalar, "scalar" },
+                                                                   { ccl_bf16_avx512f, "avx512f" },
+                                                                   { ccl_bf16_avx512bf, "avx512bf" } };
+const std::map<ccl_fp16_impl_type, std::string> fp16_impl_names = { { ccl_fp16_no_compiler_support, "no_compiler_support" },
+                                                                   { ccl_fp16_no_hardware_support, "no_hardware_support" },
+                                                                   { ccl_fp16_f16c, "f16c" },
+                                                                   { ccl_fp16_avx512f, "avx512f" },
+                                                                   { ccl_fp16_avx512fp16, "avx512fp16" } };
+const std::map<ccl_fp16_impl_type, std::string> fp16_env_impl_names = { { ccl_fp16_f16c, "f16c" },
+                                                                       { ccl_fp16_avx512f, "avx512f" },
+                                                                       { ccl_fp16_avx512fp16, "avx512fp16" } };
+
+std::set<ccl_bf16_impl_type> ccl_bf16_get_impl_types() {
+    return { ccl_bf16_scalar, ccl_bf16_avx512f, ccl_bf16_avx512bf };
+}
+
+std::set<ccl_fp16_impl_type> ccl_fp16_get_impl_types() {
+    return { ccl_fp16_f16c, ccl_fp16_avx512f, ccl_fp16_avx512fp16 };
 }
 
 ccl::status ccl_comp_copy(const void* in_buf, void* out_buf, size_t bytes, bool use_nontemporal, ccl_sched* sched) {

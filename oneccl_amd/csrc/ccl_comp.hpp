@@ -18,7 +18,9 @@
 #include <stdint.h>
 
 #include <exception>
+#include <map>
 #include <memory>
+#include <set>
 #include <string>
 #include <vector>
 
@@ -80,6 +82,15 @@ typedef enum { ccl_bf16_scalar = 0, ccl_bf16_avx512f, ccl_bf16_avx512bf } ccl_bf
 typedef enum {
     ccl_fp16_no_compiler_support = 0, ccl_fp16_no_hardware_support, ccl_fp16_f16c, ccl_fp16_avx512f, ccl_fp16_avx512fp16
 } ccl_fp16_impl_type;
+
+// Names as the reference prints and parses them (bf16.cpp:26-30, fp16.cpp:25-37) and the implementations a process
+// may choose (bf16_utils.hpp:30-72, fp16_utils.hpp:37-80 ask the CPU; here every implementation's arithmetic is in
+// the kernels, so all of them are on offer).
+extern const std::map<ccl_bf16_impl_type, std::string> bf16_impl_names;
+extern const std::map<ccl_fp16_impl_type, std::string> fp16_impl_names;
+extern const std::map<ccl_fp16_impl_type, std::string> fp16_env_impl_names;
+std::set<ccl_bf16_impl_type> ccl_bf16_get_impl_types();
+std::set<ccl_fp16_impl_type> ccl_fp16_get_impl_types();
 
 namespace ccl {
 // The two knobs of the reference's env_data that this path reads (src/common/env/env.cpp:711-720): which

@@ -197,6 +197,17 @@ int main() {
         EXPECT(!strcmp(ccl_reduction_to_str(ccl::reduction::custom), "custom") && !strcmp(ccl_reduction_to_str((ccl::reduction)9), "unknown"), "reduction names");
         EXPECT(DT(ccl::datatype::bfloat16).size() == 2 && ccl_datatype_storage::instance().name(DT(ccl::datatype::uint64)) == "uint64", "datatype table");
     }
+    // implementation names and the implementations on offer (bf16.cpp:26-30, fp16.cpp:25-37, *_utils.hpp)
+    {
+        EXPECT(bf16_impl_names.at(ccl_bf16_scalar) == "scalar" && bf16_impl_names.at(ccl_bf16_avx512f) == "avx512f" &&
+               bf16_impl_names.at(ccl_bf16_avx512bf) == "avx512bf" && bf16_impl_names.size() == 3, "bf16 implementation names");
+        EXPECT(fp16_impl_names.at(ccl_fp16_no_compiler_support) == "no_compiler_support" && fp16_impl_names.at(ccl_fp16_f16c) == "f16c" &&
+               fp16_impl_names.at(ccl_fp16_avx512fp16) == "avx512fp16" && fp16_impl_names.size() == 5 && fp16_env_impl_names.size() == 3 &&
+               fp16_env_impl_names.count(ccl_fp16_no_hardware_support) == 0, "fp16 implementation names");
+        EXPECT(ccl_bf16_get_impl_types().count(ccl_bf16_avx512bf) == 1 && ccl_bf16_get_impl_types().size() == 3, "bf16 implementations on offer");
+        EXPECT(ccl_fp16_get_impl_types().count(ccl_fp16_avx512fp16) == 1 && ccl_fp16_get_impl_types().count(ccl_fp16_no_compiler_support) == 0,
+               "fp16 implementations on offer");
+    }
     // copy and array converters
     {
         std::vector<uint8_t> src(100003);
