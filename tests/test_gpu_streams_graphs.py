@@ -50,6 +50,60 @@ def test_graph_capture_and_replay(comp, variant):
         comp.set_param("variant", 0)
 
 
+def test_graph_of_copy_broadcast_converters_and_fused_reduce(comp):
+    """A pipeline of the other kernels in one captured graph -- widen bf16 to fp32, copy, narrow back, broadcast to
+    three buffers, fused reduce of two tensors against two peer fusion buffers -- replayed four times with eager work
+    in between; every replay equals the eager result and the oracle."""
+    import torch
+    rng = np.random.default_rng(5)
+    count = 1_000_003
+    src = O.bf16_from_f32(rng.standard_normal(count).astype(np.float32))
+    d_src = to_dev(src)
+    f32 = torch.zeros(count, dtype=torch.int32, device="cuda")
+    f32b = torch.zeros_like(f32)
+    back = torch.zeros_like(d_src)
+    outs = [torch.zeros_like(d_src) for _ in range(3)]
+    counts = [400_001, count - 400_001]
+    plan = comp.FusionPlan(counts, comp.BFLOAT16, 1)
+    peers_h = [O.bf16_from_f32(rng.standard_normal(plan.nbytes // 2).astype(np.float32)) for _ in range(2)]
+    peers = [to_dev(p_) for p_ in peers_h]
+    res = [torch.zeros(c, dtype=d_src.dtype, device="cuda") for c in counts]
+
+    def pipeline():
+        comp.convert_bf16_to_fp32_arrays(d_src, f32, count)
+        comp.comp_copy(f32, f32b, 4 * count, use_nontemporal=True)
+        comp.convert_fp32_to_bf16_arrays(f32b, back, count)
+        comp.comp_reduce_write_n(comp.BFLOAT16, comp.SUM, [back], outs, count)
+        plan.reduce(comp.SUM, [outs[2][:counts[0]], outs[2][counts[0]:]], peers, res, lp_mode=comp.LP_KEEP_PRECISION)
+
+    offs, _ = O.fusion_offsets(counts, 2, 1)
+    want_res = []
+    for t, c in enumerate(counts):
+        lo = sum(counts[:t])
+        o = offs[t] // 2
+        want_res.append(O.reduce_n([src[lo:lo + c]] + [p_[o:o + c] for p_ in peers_h], O.BFLOAT16, O.SUM, keep=1))
+
+    def check(tag):
+        torch.cuda.synchronize()
+        for o_ in outs:
+            assert (to_host(o_, np.uint16) == src).all(), tag      # widening and narrowing back is exact
+        for r_, w_ in zip(res, want_res):
+            assert (to_host(r_, np.uint16) == w_).all(), tag
+
+    pipeline()
+    check("eager")
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        pipeline()
+    for rep in range(4):
+        for t_ in outs + res + [back]:
+            t_.fill_(0)
+        torch.cuda.synchronize()
+        g.replay()
+        check(f"replay {rep}")
+    plan.close()
+
+
 def test_two_phased_reduces_overlapping_on_two_streams(comp):
     import torch
     rng = np.random.default_rng(11)
