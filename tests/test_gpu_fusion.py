@@ -109,6 +109,51 @@ def test_pack_reduce_unpack_and_fused(comp, align, dtype):
     plan.close()
 
 
+@pytest.mark.parametrize("dtype,op", [(O.FLOAT16, O.MAX), (O.BFLOAT16, O.SUM), (O.INT32, O.PROD)])
+def test_fused_reduce_peer_count_limits_and_errors(comp, dtype, op):
+    """No peers at all (every tensor comes back as it is -- or, for bf16 with fp32 accumulate, as widening and
+    rounding once leave it), one peer, the maximum of 16, and the argument errors: 17 peers, a null tensor."""
+    import torch
+    rng = np.random.default_rng(70 + dtype)
+    counts = [1, 4095, 4096, 4097, 20_000, 0, 33_333]
+    np_t = O.NP_STORAGE[dtype]
+    esz = O.DTYPE_SIZE[dtype]
+    keep = 1 if dtype == O.BFLOAT16 else 0
+    lp = comp.LP_KEEP_PRECISION if keep else comp.LP_PAIRWISE
+    plan = comp.FusionPlan(counts, dtype, 1)
+    offs, total = O.fusion_offsets(counts, esz, 1)
+    nelem = total // esz
+    tensors = [make_inputs(rng, dtype, c, op, 1, "bits" if dtype != O.INT32 else "config")[0] if c else np.zeros(0, np_t) for c in counts]
+    peers = [make_inputs(rng, dtype, nelem, op, 1)[0] for _ in range(16)]
+    d_t = [to_dev(t if t.size else np.zeros(1, np_t)) for t in tensors]
+    d_peers = [to_dev(p_) for p_ in peers]
+    for n_peers in (0, 1, 16):
+        for variant in (0, 8):
+            comp.set_param("variant", variant)
+            try:
+                outs = [to_dev(np.zeros(c + 3, np_t)) for c in counts]
+                plan.reduce(op, d_t, d_peers[:n_peers], outs, lp_mode=lp)
+                torch.cuda.synchronize()
+            finally:
+                comp.set_param("variant", 0)
+            for i, c in enumerate(counts):
+                o = int(offs[i]) // esz
+                want = O.reduce_n([tensors[i]] + [p_[o:o + c] for p_ in peers[:n_peers]], dtype, op, keep=keep) if c else tensors[i]
+                g = to_host(outs[i], np_t)
+                assert_same(g[:c], want, dtype, f"peers={n_peers} variant={variant} tensor {i}")
+                assert not g[c:].view(np.uint8).any()
+    outs = [to_dev(np.zeros(c + 3, np_t)) for c in counts]
+    with pytest.raises(comp.CclError):
+        plan.reduce(op, d_t, d_peers + [d_peers[0]], outs, lp_mode=lp)          # 17 peers
+    with pytest.raises(comp.CclError):
+        plan.reduce(op, [0] + d_t[1:], d_peers[:2], outs, lp_mode=lp)             # a null tensor with a non-zero count
+    with pytest.raises(comp.CclError):
+        plan.reduce(4, d_t, d_peers[:2], outs, lp_mode=lp)                         # custom has no device form here
+    torch.cuda.synchronize()
+    assert all(not to_host(o_, np_t).view(np.uint8).any() for o_ in outs), "a rejected call wrote something"
+    plan.close()
+
+
 def test_fusion_config_bf16_256_tensors(comp):
     """The benchmark's fusion configuration at reduced element counts: 256 bf16 gradient tensors, counts
     log-uniform, N(0, 0.02) values, 256-byte aligned offsets, 8-input sum against 7 peer fusion buffers."""
