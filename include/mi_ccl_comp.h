@@ -186,7 +186,8 @@ int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* ow
  * at; default 256, i.e. one tile per block up to 65,536 blocks), "max_blocks" (cap on the grid; 0 = no cap), "xcd_chunked" (0/1: give each of the 8 XCDs one
  * contiguous share of the buffer), "variant" (kernel form: 0 = chosen by size and shape; 1, 2, 4 = the streaming
  * kernels with that many vectors per lane where a type has them; 8 = the phased kernels at any size; a non-zero value
- * also keeps one-input calls and pack/unpack on their general kernels -- for tests and measurements),
+ * also keeps one-input calls on the general reduce kernels instead of the copy and broadcast kernels -- for tests and
+ * measurements),
  * "phased_min_bytes" (scales the sizes from which the phased kernels are used; default 160 MB), "num_cus" (read
  * only), and "fp16_impl" (enum mi_ccl_fp16_impl above).
  * Returns invalid_arguments for an unknown name or out-of-range value. */
