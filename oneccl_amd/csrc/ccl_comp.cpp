@@ -105,20 +105,55 @@ ccl_datatype_storage::ccl_datatype_storage() {
     }
 }
 
-const ccl_datatype_storage& ccl_datatype_storage::instance() {
+ccl_datatype_storage& ccl_datatype_storage::instance() {
     static ccl_datatype_storage s;
     return s;
 }
 
+bool ccl_datatype_storage::is_predefined_datatype(ccl::datatype idx) {
+    return (int)idx >= (int)ccl::datatype::int8 && (int)idx <= (int)ccl::datatype::last_predefined;
+}
+
 const ccl_datatype& ccl_datatype_storage::get(ccl::datatype idx) const {
-    int i = (int)idx;
-    if (i < 0 || i >= 12)
-        fail("unexpected datatype " + std::to_string(i));
-    return table[i];
+    if (is_predefined_datatype(idx))
+        return table[(int)idx];
+    std::lock_guard<std::mutex> lock(guard);
+    auto it = custom_table.find((int)idx);
+    if (it == custom_table.end())
+        fail("unexpected datatype " + std::to_string((int)idx));
+    return it->second.first;
 }
 
 const std::string& ccl_datatype_storage::name(const ccl_datatype& dtype) const {
-    return names[(int)get(dtype.idx()).idx()];
+    if (is_predefined_datatype(dtype.idx()))
+        return names[(int)dtype.idx()];
+    std::lock_guard<std::mutex> lock(guard);
+    auto it = custom_table.find((int)dtype.idx());
+    if (it == custom_table.end())
+        fail("unexpected datatype " + std::to_string((int)dtype.idx()));
+    return it->second.second;
+}
+
+ccl::datatype ccl_datatype_storage::create_by_datatype_size(size_t datatype_size) {
+    if (datatype_size == 0)
+        fail("non-positive datatype size 0");
+    std::lock_guard<std::mutex> lock(guard);
+    while (custom_table.count(custom_idx) || is_predefined_datatype((ccl::datatype)custom_idx)) {
+        custom_idx++;
+        if (custom_idx < (int)ccl::datatype::int8)        // wrapped around
+            custom_idx = (int)ccl::datatype::int8;
+    }
+    const ccl::datatype idx = (ccl::datatype)custom_idx;
+    custom_table[custom_idx] = std::make_pair(ccl_datatype(idx, datatype_size), "DTYPE_" + std::to_string(custom_idx));
+    return idx;
+}
+
+void ccl_datatype_storage::free(ccl::datatype idx) {
+    if (is_predefined_datatype(idx))
+        fail("attempt to free predefined datatype idx " + std::to_string((int)idx));
+    std::lock_guard<std::mutex> lock(guard);
+    if (!custom_table.erase((int)idx))
+        fail("attempt to free non-existing datatype idx " + std::to_string((int)idx));
 }
 
 const char* ccl_reduction_to_str(ccl::reduction type) {

@@ -20,6 +20,7 @@
 #include <exception>
 #include <map>
 #include <memory>
+#include <mutex>
 #include <set>
 #include <string>
 #include <vector>
@@ -123,12 +124,20 @@ class ccl_datatype_storage {
 public:
     const ccl_datatype& get(ccl::datatype idx) const;
     const std::string& name(const ccl_datatype& dtype) const;
-    static const ccl_datatype_storage& instance();
+    static ccl_datatype_storage& instance();
+    // user-defined datatypes, for ccl::reduction::custom (datatype.cpp:141-181): an element size and the next free
+    // index above the predefined ones; the name is "DTYPE_<index>"
+    ccl::datatype create_by_datatype_size(size_t datatype_size);
+    void free(ccl::datatype idx);
+    static bool is_predefined_datatype(ccl::datatype idx);
 
 private:
     ccl_datatype_storage();
     ccl_datatype table[12];
     std::string names[12];
+    mutable std::mutex guard;
+    std::map<int, std::pair<ccl_datatype, std::string>> custom_table;
+    int custom_idx = (int)ccl::datatype::last_predefined + 1;
 };
 
 // What this path needs of a schedule (src/sched/sched.hpp, src/sched/sched_base.hpp): the stream its kernels go to

@@ -119,6 +119,15 @@ static void custom_sum_i32(const void* in, size_t n, void* inout, size_t* out_co
     (void)dt; (void)ctx;
 }
 
+static int g_custom_dtype_seen = -1;
+static void custom_xyz_max(const void* in, size_t n, void* inout, size_t* out_count, ccl::datatype dt, const ccl::fn_context*) {
+    const int32_t* a = (const int32_t*)in; int32_t* b = (int32_t*)inout;
+    for (size_t e = 0; e < n; e++)
+        if (a[3 * e] > b[3 * e]) { b[3 * e] = a[3 * e]; b[3 * e + 1] = a[3 * e + 1]; b[3 * e + 2] = a[3 * e + 2]; }
+    if (out_count) *out_count = n;
+    g_custom_dtype_seen = (int)dt;
+}
+
 int main() {
     int ndev = 0; CK(hipGetDeviceCount(&ndev));
     if (ndev < 1) { printf("no GPU\n"); return 2; }
@@ -184,6 +193,41 @@ int main() {
         try { ccl_comp_reduce(&sched, da.p, 1000, db.p, &oc, DT(ccl::datatype::int32), ccl::reduction::custom, nullptr); }
         catch (const ccl::exception& e) { threw = strstr(e.what(), "custom reduction requires user callback") != nullptr; }
         EXPECT(threw, "missing callback must throw ccl::exception");
+    }
+    // a user-defined datatype (datatype.cpp:141-181): 12-byte elements reduced by a callback that sees the datatype's
+    // index; create / name / size / free and their errors
+    {
+        ccl_datatype_storage& st = ccl_datatype_storage::instance();
+        const ccl::datatype idx = st.create_by_datatype_size(12);
+        const ccl::datatype idx2 = st.create_by_datatype_size(3);
+        EXPECT((int)idx == (int)ccl::datatype::last_predefined + 1 && (int)idx2 == (int)idx + 1, "custom datatype indices %d %d", (int)idx, (int)idx2);
+        EXPECT(st.get(idx).size() == 12 && st.get(idx2).size() == 3 && st.name(st.get(idx)) == "DTYPE_" + std::to_string((int)idx),
+               "custom datatype size and name");
+        EXPECT(!ccl_datatype_storage::is_predefined_datatype(idx) && ccl_datatype_storage::is_predefined_datatype(ccl::datatype::bfloat16),
+               "is_predefined_datatype");
+        g_custom_dtype_seen = -1;
+        std::vector<int32_t> a(3 * 500), b(3 * 500);
+        for (size_t i = 0; i < a.size(); i++) { a[i] = (int32_t)i; b[i] = (int32_t)(1000 - i); }
+        DevBuf<int32_t> da(a), db(b);
+        size_t oc = 0;
+        ccl_comp_reduce(&sched, da.p, 500, db.p, &oc, st.get(idx), ccl::reduction::custom, custom_xyz_max);
+        std::vector<int32_t> got = db.host();
+        bool ok = oc == 500 && g_custom_dtype_seen == (int)idx;
+        for (size_t e = 0; e < 500; e++)        // the element with the larger first component wins as a whole
+            for (int c = 0; c < 3; c++) ok = ok && got[3 * e + c] == (a[3 * e] > b[3 * e] ? a[3 * e + c] : b[3 * e + c]);
+        EXPECT(ok, "custom reduction over a 12-byte user datatype");
+        st.free(idx2);
+        bool threw = false;
+        try { st.get(idx2); } catch (const ccl::exception&) { threw = true; }
+        EXPECT(threw, "a freed datatype is gone");
+        threw = false;
+        try { st.free(idx2); } catch (const ccl::exception& e) { threw = strstr(e.what(), "non-existing") != nullptr; }
+        EXPECT(threw, "freeing twice throws");
+        threw = false;
+        try { st.free(ccl::datatype::int32); } catch (const ccl::exception& e) { threw = strstr(e.what(), "predefined") != nullptr; }
+        EXPECT(threw, "freeing a predefined datatype throws");
+        EXPECT((int)st.create_by_datatype_size(5) == (int)idx + 1, "a freed index is handed out again");
+        st.free(idx);
     }
     // in_count == 0 succeeds without looking at anything; an unknown dtype throws
     {
