@@ -20,7 +20,10 @@
  *     succeeds without touching any pointer (comp.cpp:132-134, :61-63).
  *   - Results are bit-identical to the reference CPU reduction on the same inputs (integers wrap;
  *     one IEEE operation per pair in input order, no FMA; min/max return the same operand as the
- *     reference on ties and NaNs).  The payload and sign of a NaN produced by sum/prod are unspecified.
+ *     reference on ties and NaNs).  NaN results of sum and prod are the x86 ones too: a NaN operand comes back with
+ *     its quiet bit set, an invalid operation (Inf - Inf, 0 x Inf) gives the negative default NaN; only when both
+ *     operands of a step are NaNs is it unspecified which of the two comes back (in the reference that depends on
+ *     the operand order its compiler chose).
  */
 #ifndef MI_CCL_COMP_H
 #define MI_CCL_COMP_H
@@ -58,8 +61,9 @@ enum mi_ccl_bf16_impl { MI_CCL_BF16_SCALAR = 0, MI_CCL_BF16_AVX512F = 1, MI_CCL_
 /* ccl_fp16_impl_type, src/comp/fp16/fp16_utils.hpp:26-32 (CCL_FP16, env.cpp:715-720).  f16c and avx512f work
  * through fp32 and give the same bits; avx512fp16 works on the fp16 values (fp16_intrisics.cpp:24-35): same bits
  * for sum and prod, and min/max return the chosen operand untouched where the other two quiet a signalling NaN.
- * Process-wide like the reference's: mi_ccl_set_param("fp16_impl", value); default avx512f. */
-enum mi_ccl_fp16_impl { MI_CCL_FP16_F16C = 2, MI_CCL_FP16_AVX512F = 3, MI_CCL_FP16_AVX512FP16 = 4 };
+ * Every reduce entry point takes the choice as its fp16_impl argument (ignored for other dtypes); MI_CCL_FP16_DEFAULT
+ * there means the process-wide default, mi_ccl_set_param("fp16_impl", value), which starts as avx512f. */
+enum mi_ccl_fp16_impl { MI_CCL_FP16_DEFAULT = 0, MI_CCL_FP16_F16C = 2, MI_CCL_FP16_AVX512F = 3, MI_CCL_FP16_AVX512FP16 = 4 };
 
 /* How 16-bit floating types are carried through an N-input reduce (flags, OR them):
  *   MI_CCL_LP_PAIRWISE        round to the 16-bit type after every pair: a chain of ccl_comp_reduce calls
@@ -90,12 +94,12 @@ int mi_ccl_kernel_name(const char* kernel, int dtype, int op, char* buf, size_t 
  * (src/comp/comp.cpp:76-200) and reduce_local_inplace_kernel (src/kernels/kernels.cl:236-246,
  * launched from ze_reduce_local_entry.cpp:40-58).  in and inout must be identical or disjoint. */
 int mi_ccl_comp_reduce(int dtype, int op, const void* in, size_t count, void* inout, int bf16_impl,
-                       void* stream);
+                       int fp16_impl, void* stream);
 
 /* Replaces ccl_bf16_reduce (src/comp/bf16/bf16.cpp:87-110) and ccl_fp16_reduce
- * (src/comp/fp16/fp16.cpp:41-53; results of the f16c / avx512f implementations). */
+ * (src/comp/fp16/fp16.cpp:41-53). */
 int mi_ccl_bf16_reduce(const void* in, size_t count, void* inout, int op, int bf16_impl, void* stream);
-int mi_ccl_fp16_reduce(const void* in, size_t count, void* inout, int op, void* stream);
+int mi_ccl_fp16_reduce(const void* in, size_t count, void* inout, int op, int fp16_impl, void* stream);
 
 /* ---- N inputs ----------------------------------------------------------------------------------- */
 
@@ -106,7 +110,7 @@ int mi_ccl_fp16_reduce(const void* in, size_t count, void* inout, int op, void* 
  * launch sites ze_a2a_reduce_scatter_entry.cpp:48-136, ze_a2a_pipeline_reduce_scatter_entry.cpp:195-228)
  * and, with slice pointers, ccl_comp_batch_reduce (src/comp/comp.cpp:202-249). */
 int mi_ccl_comp_reduce_n(int dtype, int op, const void* const* srcs, int n, void* dst, size_t count,
-                         int lp_mode, int bf16_impl, void* stream);
+                         int lp_mode, int bf16_impl, int fp16_impl, void* stream);
 
 /* The same reduce with the result stored to each of m buffers (1 <= m <= 16) in one pass: (n + m) x bytes of
  * memory traffic instead of (n + 1 + 2(m - 1)) x bytes for a reduce followed by m - 1 copies.  dsts is a HOST
@@ -115,7 +119,7 @@ int mi_ccl_comp_reduce_n(int dtype, int op, const void* const* srcs, int n, void
  * n == 1 and MI_CCL_LP_PAIRWISE (a byte copy for every dtype), write_monolithic_kernel_{1..7}
  * (src/kernels/kernels.cl:423-560, launched from ze_a2a_allgatherv_entry.cpp:526-585: m = peer count). */
 int mi_ccl_comp_reduce_write_n(int dtype, int op, const void* const* srcs, int n, void* const* dsts, int m,
-                               size_t count, int lp_mode, int bf16_impl, void* stream);
+                               size_t count, int lp_mode, int bf16_impl, int fp16_impl, void* stream);
 
 /* Slice form of the same: slice i starts at in_buf + offsets[i] elements (offsets: HOST array); inout is
  * slice 0 and receives the result.  Replaces ccl_comp_batch_reduce (src/comp/comp.cpp:202-249); the tmp and
@@ -123,7 +127,7 @@ int mi_ccl_comp_reduce_write_n(int dtype, int op, const void* const* srcs, int n
  * reproduces the reference bit for bit, including the truncated tail (MI_CCL_LP_TAIL_QUIRK). */
 int mi_ccl_comp_batch_reduce(const void* in_buf, const size_t* offsets, size_t n_offsets, size_t count,
                              void* inout, int dtype, int op, int bf16_keep_precision_mode, int bf16_impl,
-                             void* stream);
+                             int fp16_impl, void* stream);
 
 /* ---- copies and converters ---------------------------------------------------------------------- */
 
@@ -177,7 +181,7 @@ int mi_ccl_fusion_unpack(mi_ccl_fusion_plan* plan, const void* fusion_buf, void*
  * where every peer is a fusion buffer with this plan's layout.  Same bits as the three-step sequence. */
 int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* own_tensors,
                          const void* const* peers, int n_peers, void* const* out_tensors, int lp_mode,
-                         int bf16_impl, void* stream);
+                         int bf16_impl, int fp16_impl, void* stream);
 
 /* ---- launch tuning ------------------------------------------------------------------------------- */
 
@@ -189,7 +193,7 @@ int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* ow
  * also keeps one-input calls on the general reduce kernels instead of the copy and broadcast kernels -- for tests and
  * measurements),
  * "phased_min_bytes" (scales the sizes from which the phased kernels are used; default 160 MB), "num_cus" (read
- * only), and "fp16_impl" (enum mi_ccl_fp16_impl above).
+ * only), and "fp16_impl" (what MI_CCL_FP16_DEFAULT stands for: 2, 3 or 4 of enum mi_ccl_fp16_impl above).
  * Returns invalid_arguments for an unknown name or out-of-range value. */
 int mi_ccl_set_param(const char* name, long value);
 long mi_ccl_get_param(const char* name);

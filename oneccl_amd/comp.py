@@ -17,6 +17,8 @@ SUM, PROD, MIN, MAX, CUSTOM = range(5)
 SUCCESS, OUT_OF_RESOURCE, INVALID_ARGUMENTS, RUNTIME_ERROR = range(4)
 # ccl_bf16_impl_type (src/comp/bf16/bf16_utils.hpp:26)
 BF16_SCALAR, BF16_AVX512F, BF16_AVX512BF = 0, 1, 2
+# ccl_fp16_impl_type (src/comp/fp16/fp16_utils.hpp:26-32); 0 = the process-wide default (set_param("fp16_impl"))
+FP16_DEFAULT, FP16_F16C, FP16_AVX512F, FP16_AVX512FP16 = 0, 2, 3, 4
 LP_PAIRWISE, LP_KEEP_PRECISION, LP_TAIL_QUIRK = 0, 1, 2
 
 DTYPE_SIZE = [1, 1, 2, 2, 4, 4, 8, 8, 2, 4, 8, 2]
@@ -58,12 +60,12 @@ def lib():
         getattr(L, f).restype = C.c_char_p
         getattr(L, f).argtypes = [i]
     L.mi_ccl_kernel_name.argtypes = [C.c_char_p, i, i, C.c_char_p, sz]
-    L.mi_ccl_comp_reduce.argtypes = [i, i, vp, sz, vp, i, vp]
+    L.mi_ccl_comp_reduce.argtypes = [i, i, vp, sz, vp, i, i, vp]
     L.mi_ccl_bf16_reduce.argtypes = [vp, sz, vp, i, i, vp]
-    L.mi_ccl_fp16_reduce.argtypes = [vp, sz, vp, i, vp]
-    L.mi_ccl_comp_reduce_n.argtypes = [i, i, vp, i, vp, sz, i, i, vp]
-    L.mi_ccl_comp_reduce_write_n.argtypes = [i, i, vp, i, vp, i, sz, i, i, vp]
-    L.mi_ccl_comp_batch_reduce.argtypes = [vp, vp, sz, sz, vp, i, i, i, i, vp]
+    L.mi_ccl_fp16_reduce.argtypes = [vp, sz, vp, i, i, vp]
+    L.mi_ccl_comp_reduce_n.argtypes = [i, i, vp, i, vp, sz, i, i, i, vp]
+    L.mi_ccl_comp_reduce_write_n.argtypes = [i, i, vp, i, vp, i, sz, i, i, i, vp]
+    L.mi_ccl_comp_batch_reduce.argtypes = [vp, vp, sz, sz, vp, i, i, i, i, i, vp]
     L.mi_ccl_comp_copy.argtypes = [vp, vp, sz, i, vp]
     L.mi_ccl_convert_fp32_to_bf16_arrays.argtypes = [vp, vp, sz, i, vp]
     L.mi_ccl_convert_bf16_to_fp32_arrays.argtypes = [vp, vp, sz, vp]
@@ -78,7 +80,7 @@ def lib():
     L.mi_ccl_fusion_plan_offset.argtypes = [vp, sz]
     L.mi_ccl_fusion_pack.argtypes = [vp, vp, vp, vp]
     L.mi_ccl_fusion_unpack.argtypes = [vp, vp, vp, vp]
-    L.mi_ccl_fusion_reduce.argtypes = [vp, i, vp, vp, i, vp, i, i, vp]
+    L.mi_ccl_fusion_reduce.argtypes = [vp, i, vp, vp, i, vp, i, i, i, vp]
     L.mi_ccl_set_param.argtypes = [C.c_char_p, C.c_long]
     L.mi_ccl_get_param.restype = C.c_long
     L.mi_ccl_get_param.argtypes = [C.c_char_p]
@@ -133,9 +135,9 @@ def kernel_name(kernel, dtype, op):
     return buf.value.decode()
 
 
-def comp_reduce(dtype, op, inp, count, inout, bf16_impl=BF16_AVX512BF, stream=None):
+def comp_reduce(dtype, op, inp, count, inout, bf16_impl=BF16_AVX512BF, fp16_impl=FP16_DEFAULT, stream=None):
     """inout[i] = inout[i] OP inp[i] (ccl_comp_reduce)."""
-    _check(lib().mi_ccl_comp_reduce(dtype, op, _ptr(inp), count, _ptr(inout), bf16_impl, _stream(stream)),
+    _check(lib().mi_ccl_comp_reduce(dtype, op, _ptr(inp), count, _ptr(inout), bf16_impl, fp16_impl, _stream(stream)),
            "mi_ccl_comp_reduce")
 
 
@@ -144,30 +146,33 @@ def bf16_reduce(inp, count, inout, op, bf16_impl=BF16_AVX512BF, stream=None):
            "mi_ccl_bf16_reduce")
 
 
-def fp16_reduce(inp, count, inout, op, stream=None):
-    _check(lib().mi_ccl_fp16_reduce(_ptr(inp), count, _ptr(inout), op, _stream(stream)), "mi_ccl_fp16_reduce")
+def fp16_reduce(inp, count, inout, op, fp16_impl=FP16_DEFAULT, stream=None):
+    _check(lib().mi_ccl_fp16_reduce(_ptr(inp), count, _ptr(inout), op, fp16_impl, _stream(stream)),
+           "mi_ccl_fp16_reduce")
 
 
-def comp_reduce_n(dtype, op, srcs, dst, count, lp_mode=LP_PAIRWISE, bf16_impl=BF16_AVX512BF, stream=None):
+def comp_reduce_n(dtype, op, srcs, dst, count, lp_mode=LP_PAIRWISE, bf16_impl=BF16_AVX512BF, fp16_impl=FP16_DEFAULT,
+                  stream=None):
     """dst = srcs[0] OP srcs[1] OP ... in argument order, one pass."""
     arr = _ptr_array(srcs)
-    _check(lib().mi_ccl_comp_reduce_n(dtype, op, arr, len(srcs), _ptr(dst), count, lp_mode, bf16_impl,
+    _check(lib().mi_ccl_comp_reduce_n(dtype, op, arr, len(srcs), _ptr(dst), count, lp_mode, bf16_impl, fp16_impl,
                                       _stream(stream)), "mi_ccl_comp_reduce_n")
 
 
-def comp_reduce_write_n(dtype, op, srcs, dsts, count, lp_mode=LP_PAIRWISE, bf16_impl=BF16_AVX512BF, stream=None):
+def comp_reduce_write_n(dtype, op, srcs, dsts, count, lp_mode=LP_PAIRWISE, bf16_impl=BF16_AVX512BF,
+                        fp16_impl=FP16_DEFAULT, stream=None):
     """Every dsts[k] = srcs[0] OP srcs[1] OP ... in argument order, one pass; one source and LP_PAIRWISE is a
     copy of one buffer to len(dsts) buffers."""
     s, d = _ptr_array(srcs), _ptr_array(dsts)
     _check(lib().mi_ccl_comp_reduce_write_n(dtype, op, s, len(srcs), d, len(dsts), count, lp_mode, bf16_impl,
-                                            _stream(stream)), "mi_ccl_comp_reduce_write_n")
+                                            fp16_impl, _stream(stream)), "mi_ccl_comp_reduce_write_n")
 
 
 def comp_batch_reduce(in_buf, offsets, count, inout, dtype, op, keep_precision, bf16_impl=BF16_AVX512BF,
-                      stream=None):
+                      fp16_impl=FP16_DEFAULT, stream=None):
     offs = (C.c_size_t * len(offsets))(*[int(o) for o in offsets])
     _check(lib().mi_ccl_comp_batch_reduce(_ptr(in_buf), offs, len(offsets), count, _ptr(inout), dtype, op,
-                                          int(keep_precision), bf16_impl, _stream(stream)),
+                                          int(keep_precision), bf16_impl, fp16_impl, _stream(stream)),
            "mi_ccl_comp_batch_reduce")
 
 
@@ -236,10 +241,10 @@ class FusionPlan:
                "mi_ccl_fusion_unpack")
 
     def reduce(self, op, own_tensors, peers, out_tensors, lp_mode=LP_PAIRWISE, bf16_impl=BF16_AVX512BF,
-               stream=None):
+               fp16_impl=FP16_DEFAULT, stream=None):
         assert len(own_tensors) == self.k and len(out_tensors) == self.k
         _check(lib().mi_ccl_fusion_reduce(self._h, op, _ptr_array(own_tensors), _ptr_array(peers), len(peers),
-                                          _ptr_array(out_tensors), lp_mode, bf16_impl, _stream(stream)),
+                                          _ptr_array(out_tensors), lp_mode, bf16_impl, fp16_impl, _stream(stream)),
                "mi_ccl_fusion_reduce")
 
     def close(self):

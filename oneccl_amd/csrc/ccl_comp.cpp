@@ -52,18 +52,21 @@ ccl::env_data parse_env() {
     return e;
 }
 
-// The library's float16 mode follows ccl::global_data::env().fp16_impl_type, which a caller may also set by hand.
-// Returns false when that value names no implementation: the reference's dispatch has no branch for it and leaves
-// inout as it was (src/comp/fp16/fp16_intrisics.hpp:204-248), and so do the functions below.
+// float16 follows ccl::global_data::env().fp16_impl_type, which a caller may also set by hand; the value travels
+// with every call (nothing process-wide is touched).  fp16_mode returns false when that value names no
+// implementation: the reference's dispatch has no branch for it and leaves inout as it was
+// (src/comp/fp16/fp16_intrisics.hpp:204-248), and so do the functions below.
+int fp16_impl() {
+    return (int)ccl::global_data::env().fp16_impl_type;
+}
 bool fp16_mode(const ccl_datatype& dtype) {
     if (dtype.idx() != ccl::datatype::float16)
         return true;
-    const int impl = (int)ccl::global_data::env().fp16_impl_type;
-    if (impl < MI_CCL_FP16_F16C || impl > MI_CCL_FP16_AVX512FP16)
-        return false;
-    if (mi_ccl_get_param("fp16_impl") != impl)
-        mi_ccl_set_param("fp16_impl", impl);
-    return true;
+    return fp16_impl() >= MI_CCL_FP16_F16C && fp16_impl() <= MI_CCL_FP16_AVX512FP16;
+}
+// the N-input device entry points have no "no implementation" state: such a value falls back to the library's default
+int fp16_impl_or_default() {
+    return (fp16_impl() >= MI_CCL_FP16_F16C && fp16_impl() <= MI_CCL_FP16_AVX512FP16) ? fp16_impl() : MI_CCL_FP16_DEFAULT;
 }
 
 int bf16_impl() {
@@ -202,7 +205,7 @@ ccl::status ccl_comp_reduce(ccl_sched* sched, const void* in_buf, size_t in_coun
     if (!fp16_mode(dtype))
         return ccl::status::success;        // float16 without an implementation selected: inout stays as it is
     return to_status(mi_ccl_comp_reduce((int)dtype.idx(), (int)reduction, in_buf, in_count, inout_buf,
-                                        bf16_impl(), stream_of(sched)),
+                                        bf16_impl(), fp16_impl_or_default(), stream_of(sched)),
                      "ccl_comp_reduce");
 }
 
@@ -228,7 +231,7 @@ ccl::status ccl_comp_batch_reduce(const void* in_buf, const std::vector<size_t>&
         return ccl::status::success;        // every pairwise call of the chain leaves inout as it is
     return to_status(mi_ccl_comp_batch_reduce(in_buf, offsets.data(), offsets.size(), in_count, inout_buf,
                                               (int)dtype.idx(), (int)reduction, bf16_keep_precision_mode,
-                                              bf16_impl(), stream_of(sched)),
+                                              bf16_impl(), fp16_impl_or_default(), stream_of(sched)),
                      "ccl_comp_batch_reduce");
 }
 
@@ -247,7 +250,8 @@ void ccl_fp16_reduce(const void* in_buf, size_t in_cnt, void* inout_buf, size_t*
         *out_cnt = in_cnt;                                             // fp16.cpp:48-50
     if (!fp16_mode(ccl_datatype_storage::instance().get(ccl::datatype::float16)))
         return;
-    to_status(mi_ccl_fp16_reduce(in_buf, in_cnt, inout_buf, (int)reduction_op, stream_of(sched)), "ccl_fp16_reduce");
+    to_status(mi_ccl_fp16_reduce(in_buf, in_cnt, inout_buf, (int)reduction_op, fp16_impl(), stream_of(sched)),
+              "ccl_fp16_reduce");
 }
 
 void ccl_convert_fp32_to_bf16_arrays(void* fp32_buf, void* bf16_buf, size_t count, ccl_sched* sched) {
@@ -301,9 +305,8 @@ ccl::status ccl_comp_reduce_n(ccl_sched* sched, const void* own_buf, const std::
     srcs.push_back(own_buf);
     srcs.insert(srcs.end(), peer_bufs.begin(), peer_bufs.end());
     int lp = bf16_keep_precision_mode ? MI_CCL_LP_KEEP_PRECISION : MI_CCL_LP_PAIRWISE;
-    (void)fp16_mode(dtype);     // the device kernels have no "no implementation" state: the library's current mode applies
     return to_status(mi_ccl_comp_reduce_n((int)dtype.idx(), (int)reduction, srcs.data(), (int)srcs.size(), out_buf,
-                                          count, lp, bf16_impl(), stream_of(sched)),
+                                          count, lp, bf16_impl(), fp16_impl_or_default(), stream_of(sched)),
                      "ccl_comp_reduce_n");
 }
 
@@ -319,9 +322,8 @@ ccl::status ccl_comp_reduce_write_n(ccl_sched* sched, const void* own_buf, const
     srcs.push_back(own_buf);
     srcs.insert(srcs.end(), peer_bufs.begin(), peer_bufs.end());
     int lp = bf16_keep_precision_mode ? MI_CCL_LP_KEEP_PRECISION : MI_CCL_LP_PAIRWISE;
-    (void)fp16_mode(dtype);
     return to_status(mi_ccl_comp_reduce_write_n((int)dtype.idx(), (int)reduction, srcs.data(), (int)srcs.size(),
                                                 out_bufs.data(), (int)out_bufs.size(), count, lp,
-                                                bf16_impl(), stream_of(sched)),
+                                                bf16_impl(), fp16_impl_or_default(), stream_of(sched)),
                      "ccl_comp_reduce_write_n");
 }

@@ -9,6 +9,7 @@
 #include <cctype>
 
 #include "../../include/mi_ccl_comp.h"
+#include "launch_geometry.hpp"
 #include "reduce_kernels.hpp"
 
 namespace mi {
@@ -44,6 +45,14 @@ static std::atomic<int> g_xcd_chunked{ 0 };
 static std::atomic<int> g_variant{ 0 };
 static std::atomic<long> g_phased_min_bytes{ 160L << 20 };
 static std::atomic<int> g_fp16_impl{ MI_CCL_FP16_AVX512F };
+static std::atomic<long> g_launch_block_limit{ 0 };     // 0: what HIP allows; smaller values are for tests of the splitting
+static_assert(kGeomBlock == kBlock, "the geometry header and the kernels agree on the block size");
+
+static uint64_t block_limit() {
+    const long v = g_launch_block_limit.load(std::memory_order_relaxed);
+    const uint64_t hw = hip_block_limit(kBlock);
+    return (v > 0 && (uint64_t)v < hw) ? (uint64_t)v : hw;
+}
 static std::atomic<int> g_num_cus[64];
 
 // Barrier words of the phased kernel: one copy per device (each GPU holds its own instance of a
@@ -139,8 +148,12 @@ static hipError_t dispatch(int dtype, bool keep, int bf16_impl, const LaunchArgs
 static int launch_copy(const void* in, void* out, size_t bytes, bool nontemporal, hipStream_t stream);
 static int launch_broadcast(const void* in, void* const* dsts, int m, size_t bytes, hipStream_t stream);
 
+static bool fp16_impl_ok(int v) {
+    return v == MI_CCL_FP16_DEFAULT || (v >= MI_CCL_FP16_F16C && v <= MI_CCL_FP16_AVX512FP16);
+}
+
 static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void* const* dsts, int m, size_t count,
-                         int lp_mode, int bf16_impl, void* stream) {
+                         int lp_mode, int bf16_impl, int fp16_impl, void* stream) {
     if (count == 0)
         return MI_CCL_SUCCESS;
     if (m < 1 || m > kMaxDsts || !dsts)
@@ -149,7 +162,7 @@ static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void
         return MI_CCL_INVALID_ARGUMENTS;
     if (n < 1 || n > kMaxSrcs || !srcs)
         return MI_CCL_INVALID_ARGUMENTS;
-    if (bf16_impl < MI_CCL_BF16_SCALAR || bf16_impl > MI_CCL_BF16_AVX512BF)
+    if (bf16_impl < MI_CCL_BF16_SCALAR || bf16_impl > MI_CCL_BF16_AVX512BF || !fp16_impl_ok(fp16_impl))
         return MI_CCL_INVALID_ARGUMENTS;
     if (lp_mode & ~(MI_CCL_LP_KEEP_PRECISION | MI_CCL_LP_TAIL_QUIRK))
         return MI_CCL_INVALID_ARGUMENTS;
@@ -168,7 +181,9 @@ static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void
 
     // one input, rounded after every pair: a chain of zero pairwise steps hands the input back as it is, whatever
     // the type -- a copy to one buffer or a broadcast to several
-    const Tuning tune = current_tuning();
+    Tuning tune = current_tuning();
+    if (fp16_impl != MI_CCL_FP16_DEFAULT)
+        tune.fp16_impl = fp16_impl;     // this call's choice; the process-wide value is only the default
     if (n == 1 && !keep && tune.variant == 0) {
         if (m == 1)
             return dsts[0] == srcs[0] ? MI_CCL_SUCCESS : launch_copy(srcs[0], dsts[0], count * esz, true, (hipStream_t)stream);
@@ -244,10 +259,9 @@ constexpr uint32_t kBcastSect = 4096;       // tiles of kBlock vectors per secti
 
 __global__ void __launch_bounds__(kBlock)
 broadcast_kernel(const unsigned char* in, DstTable d, int m, uint32_t head, uint64_t nvec, uint32_t tail, uint32_t sect_tiles) {
-    const uint32_t per = sect_tiles * (uint32_t)m;          // blocks per section
-    const uint32_t sect = blockIdx.x / per, r = blockIdx.x - sect * per;
-    const uint32_t k = r / sect_tiles, t = r - k * sect_tiles;
-    const uint64_t i = ((uint64_t)sect * sect_tiles + t) * kBlock + threadIdx.x;
+    const BcastLane l = bcast_lane(blockIdx.x, threadIdx.x, sect_tiles, (uint32_t)m);
+    const uint32_t k = l.dst;
+    const uint64_t i = l.vec;
     if (i < nvec) {
         const u32x4 v = *((const u32x4_u*)(in + head) + i);         // cached: the other destinations read it again
         st_loose((u32x4_u*)((unsigned char*)d.p[k] + head) + i, v);
@@ -394,27 +408,6 @@ f16_to_f32_kernel(const uint16_t* in, uint32_t* out, uint32_t head, uint64_t nqu
     }
 }
 
-// launch geometry of the two converters: `out_elem` bytes per element of the output array, `per` elements per group,
-// `unroll` groups per lane
-struct CvtShape {
-    uint32_t head, tail;
-    uint64_t ngroup;
-    unsigned grid;
-};
-static CvtShape cvt_shape(const void* out, size_t out_elem, size_t count, unsigned per, unsigned unroll) {
-    CvtShape c;
-    const uintptr_t mis = (uintptr_t)out & 15u;
-    uint64_t head = ((16u - mis) & 15u) / out_elem;
-    if (head > count) head = count;
-    c.head = (uint32_t)head;
-    c.ngroup = (count - head) / per;
-    c.tail = (uint32_t)(count - head - c.ngroup * per);
-    const uint64_t tile = (uint64_t)kBlock * unroll;
-    const uint64_t blocks = (c.ngroup + tile - 1) / tile;
-    c.grid = (unsigned)(blocks ? blocks : 1);
-    return c;
-}
-
 }  // namespace mi
 
 using namespace mi;
@@ -460,33 +453,35 @@ int mi_ccl_kernel_name(const char* kernel, int dtype, int op, char* buf, size_t 
     return MI_CCL_SUCCESS;
 }
 
-int mi_ccl_comp_reduce(int dtype, int op, const void* in, size_t count, void* inout, int bf16_impl, void* stream) {
+int mi_ccl_comp_reduce(int dtype, int op, const void* in, size_t count, void* inout, int bf16_impl, int fp16_impl,
+                       void* stream) {
     if (count == 0)
         return MI_CCL_SUCCESS;
     const void* srcs[2] = { inout, in };
-    return reduce_n_impl(dtype, op, srcs, 2, &inout, 1, count, MI_CCL_LP_PAIRWISE, bf16_impl, stream);
+    return reduce_n_impl(dtype, op, srcs, 2, &inout, 1, count, MI_CCL_LP_PAIRWISE, bf16_impl, fp16_impl, stream);
 }
 
 int mi_ccl_bf16_reduce(const void* in, size_t count, void* inout, int op, int bf16_impl, void* stream) {
-    return mi_ccl_comp_reduce(MI_CCL_BFLOAT16, op, in, count, inout, bf16_impl, stream);
+    return mi_ccl_comp_reduce(MI_CCL_BFLOAT16, op, in, count, inout, bf16_impl, MI_CCL_FP16_DEFAULT, stream);
 }
 
-int mi_ccl_fp16_reduce(const void* in, size_t count, void* inout, int op, void* stream) {
-    return mi_ccl_comp_reduce(MI_CCL_FLOAT16, op, in, count, inout, MI_CCL_BF16_AVX512BF, stream);
+int mi_ccl_fp16_reduce(const void* in, size_t count, void* inout, int op, int fp16_impl, void* stream) {
+    return mi_ccl_comp_reduce(MI_CCL_FLOAT16, op, in, count, inout, MI_CCL_BF16_AVX512BF, fp16_impl, stream);
 }
 
 int mi_ccl_comp_reduce_n(int dtype, int op, const void* const* srcs, int n, void* dst, size_t count, int lp_mode,
-                         int bf16_impl, void* stream) {
-    return reduce_n_impl(dtype, op, srcs, n, &dst, 1, count, lp_mode, bf16_impl, stream);
+                         int bf16_impl, int fp16_impl, void* stream) {
+    return reduce_n_impl(dtype, op, srcs, n, &dst, 1, count, lp_mode, bf16_impl, fp16_impl, stream);
 }
 
 int mi_ccl_comp_reduce_write_n(int dtype, int op, const void* const* srcs, int n, void* const* dsts, int m, size_t count,
-                               int lp_mode, int bf16_impl, void* stream) {
-    return reduce_n_impl(dtype, op, srcs, n, dsts, m, count, lp_mode, bf16_impl, stream);
+                               int lp_mode, int bf16_impl, int fp16_impl, void* stream) {
+    return reduce_n_impl(dtype, op, srcs, n, dsts, m, count, lp_mode, bf16_impl, fp16_impl, stream);
 }
 
 int mi_ccl_comp_batch_reduce(const void* in_buf, const size_t* offsets, size_t n_offsets, size_t count, void* inout,
-                             int dtype, int op, int bf16_keep_precision_mode, int bf16_impl, void* stream) {
+                             int dtype, int op, int bf16_keep_precision_mode, int bf16_impl, int fp16_impl,
+                             void* stream) {
     if (dtype < 0 || dtype >= MI_CCL_DATATYPE_LAST)
         return MI_CCL_INVALID_ARGUMENTS;
     if (n_offsets == 0 || n_offsets > (size_t)kMaxSrcs || !offsets)
@@ -499,53 +494,64 @@ int mi_ccl_comp_batch_reduce(const void* in_buf, const size_t* offsets, size_t n
     srcs[0] = inout; /* inout_buf => in_buf + offsets[0] (comp.cpp:217) */
     for (size_t i = 1; i < n_offsets; i++) srcs[i] = (const char*)in_buf + kDtypeSize[dtype] * offsets[i];
     int lp = bf16_keep_precision_mode ? (MI_CCL_LP_KEEP_PRECISION | MI_CCL_LP_TAIL_QUIRK) : MI_CCL_LP_PAIRWISE;
-    return reduce_n_impl(dtype, op, srcs, (int)n_offsets, &inout, 1, count, lp, bf16_impl, stream);
+    return reduce_n_impl(dtype, op, srcs, (int)n_offsets, &inout, 1, count, lp, bf16_impl, fp16_impl, stream);
 }
 
 } /* extern "C" */
 
 namespace mi {
 static int launch_copy(const void* in, void* out, size_t bytes, bool nontemporal, hipStream_t stream) {
-    const uintptr_t mis = (uintptr_t)out & 15u;
-    uint64_t head = mis ? 16u - mis : 0;
-    if (head > bytes)
-        head = bytes;
-    const uint64_t nvec = (bytes - head) / 16;
-    const uint32_t tail = (uint32_t)(bytes - head - nvec * 16);
-    uint64_t blocks = (nvec + kBlock - 1) / kBlock;
-    if (blocks > 0x7fffffffu)
-        blocks = 0x7fffffffu;      // beyond 8 TiB the kernel strides
-    const unsigned grid = (unsigned)(blocks ? blocks : 1);
-    if (nontemporal)
-        hipLaunchKernelGGL(copy_kernel<true>, dim3(grid), dim3(kBlock), 0, stream, (const unsigned char*)in,
-                           (unsigned char*)out, (uint32_t)head, nvec, tail);
-    else
-        hipLaunchKernelGGL(copy_kernel<false>, dim3(grid), dim3(kBlock), 0, stream, (const unsigned char*)in,
-                           (unsigned char*)out, (uint32_t)head, nvec, tail);
-    return status_of(hipGetLastError());
+    const LaneWork w = lane_work((uintptr_t)out, 1, bytes, 16);
+    const uint64_t limit = block_limit(), n = num_launches(w, kBlock, limit);
+    for (uint64_t i = 0; i < n; i++) {
+        const LaunchPiece p = launch_piece(w, kBlock, limit, i);
+        // a piece other than the first starts at the vector it begins with and has no head
+        const uint64_t skip = i ? w.head + p.group0 * 16 : 0;
+        const unsigned char* s = (const unsigned char*)in + skip;
+        unsigned char* d = (unsigned char*)out + skip;
+        if (nontemporal)
+            hipLaunchKernelGGL(copy_kernel<true>, dim3(p.grid), dim3(kBlock), 0, stream, s, d, p.head, p.ngroup, p.tail);
+        else
+            hipLaunchKernelGGL(copy_kernel<false>, dim3(p.grid), dim3(kBlock), 0, stream, s, d, p.head, p.ngroup, p.tail);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess)
+            return status_of(e);
+    }
+    return MI_CCL_SUCCESS;
 }
 
 // m >= 2 destinations; the vectors start where the first destination reaches a 16-byte boundary
 static int launch_broadcast(const void* in, void* const* dsts, int m, size_t bytes, hipStream_t stream) {
-    DstTable d;
-    for (int k = 0; k < kMaxDsts; k++) d.p[k] = dsts[k < m ? k : 0];
-    const uintptr_t mis = (uintptr_t)dsts[0] & 15u;
-    uint64_t head = mis ? 16u - mis : 0;
-    if (head > bytes)
-        head = bytes;
-    const uint64_t nvec = (bytes - head) / 16;
-    const uint32_t tail = (uint32_t)(bytes - head - nvec * 16);
-    uint64_t tiles = (nvec + kBlock - 1) / kBlock;
-    if (tiles == 0)
-        tiles = 1;
-    const uint32_t sect_tiles = tiles < kBcastSect ? (uint32_t)((tiles + 7) & ~7ull) : kBcastSect;
-    const uint64_t sects = (tiles + sect_tiles - 1) / sect_tiles;
-    const uint64_t blocks = sects * sect_tiles * (uint64_t)m;
-    if (blocks > 0x7fffffffu)
-        return MI_CCL_INVALID_ARGUMENTS;       // more than 8 TiB of destinations
-    hipLaunchKernelGGL(broadcast_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, (const unsigned char*)in, d, m,
-                       (uint32_t)head, nvec, tail, sect_tiles);
-    return status_of(hipGetLastError());
+    const BcastShape b = bcast_shape((uintptr_t)dsts[0], bytes, kBcastSect);
+    const uint64_t limit = block_limit(), n = bcast_num_launches(b, m, limit);
+    for (uint64_t i = 0; i < n; i++) {
+        const BcastPiece p = bcast_piece(b, m, limit, i);
+        const uint64_t skip = i ? b.head + p.vec0 * 16 : 0;
+        DstTable d;
+        for (int k = 0; k < kMaxDsts; k++) d.p[k] = (unsigned char*)dsts[k < m ? k : 0] + skip;
+        hipLaunchKernelGGL(broadcast_kernel, dim3(p.grid), dim3(kBlock), 0, stream, (const unsigned char*)in + skip, d, m,
+                           p.head, p.nvec, p.tail, b.sect_tiles);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess)
+            return status_of(e);
+    }
+    return MI_CCL_SUCCESS;
+}
+
+// The array converters: `per` elements per lane, vectors from the output's first 16-byte boundary on; launch(p, skip)
+// enqueues one piece whose arrays start `skip` elements in.
+template <class F>
+static int launch_converter(const void* out, uint32_t out_elem_bytes, size_t count, uint32_t per, F&& launch) {
+    const LaneWork w = lane_work((uintptr_t)out, out_elem_bytes, count, per);
+    const uint64_t limit = block_limit(), n = num_launches(w, kBlock, limit);
+    for (uint64_t i = 0; i < n; i++) {
+        const LaunchPiece p = launch_piece(w, kBlock, limit, i);
+        launch(p, i ? w.head + p.group0 * per : 0);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess)
+            return status_of(e);
+    }
+    return MI_CCL_SUCCESS;
 }
 
 }  // namespace mi
@@ -568,17 +574,19 @@ int mi_ccl_convert_fp32_to_bf16_arrays(const void* fp32_buf, void* bf16_buf, siz
         return MI_CCL_INVALID_ARGUMENTS;
     if (((uintptr_t)fp32_buf & 3u) || ((uintptr_t)bf16_buf & 1u))
         return MI_CCL_INVALID_ARGUMENTS;
-    if (count / 8 / (kBlock * kCvtUnroll) >= 0x7fffffffu)
-        return MI_CCL_INVALID_ARGUMENTS;
-    const CvtShape c = cvt_shape(bf16_buf, 2, count, 8, kCvtUnroll);
-    if (bf16_impl == MI_CCL_BF16_AVX512BF)
-        hipLaunchKernelGGL(f32_to_bf16_kernel<true>, dim3(c.grid), dim3(kBlock), 0, (hipStream_t)stream,
-                           (const uint32_t*)fp32_buf, (uint16_t*)bf16_buf, c.head, c.ngroup, c.tail,
-                           (uint64_t)(count - count % 16));
-    else
-        hipLaunchKernelGGL(f32_to_bf16_kernel<false>, dim3(c.grid), dim3(kBlock), 0, (hipStream_t)stream,
-                           (const uint32_t*)fp32_buf, (uint16_t*)bf16_buf, c.head, c.ngroup, c.tail, (uint64_t)0);
-    return status_of(hipGetLastError());
+    static_assert(kCvtUnroll == 1 && kWidenUnroll == 1, "one group per lane, as the launch geometry assumes");
+    const uint64_t rne_limit = bf16_impl == MI_CCL_BF16_AVX512BF ? count - count % 16 : 0;
+    return launch_converter(bf16_buf, 2, count, 8, [&](const LaunchPiece& p, uint64_t skip) {
+        const uint32_t* s = (const uint32_t*)fp32_buf + skip;
+        uint16_t* d = (uint16_t*)bf16_buf + skip;
+        const uint64_t lim = rne_limit > skip ? rne_limit - skip : 0;      // first truncated element, as this piece counts
+        if (bf16_impl == MI_CCL_BF16_AVX512BF)
+            hipLaunchKernelGGL(f32_to_bf16_kernel<true>, dim3(p.grid), dim3(kBlock), 0, (hipStream_t)stream, s, d, p.head,
+                               p.ngroup, p.tail, lim);
+        else
+            hipLaunchKernelGGL(f32_to_bf16_kernel<false>, dim3(p.grid), dim3(kBlock), 0, (hipStream_t)stream, s, d, p.head,
+                               p.ngroup, p.tail, (uint64_t)0);
+    });
 }
 
 int mi_ccl_convert_bf16_to_fp32_arrays(const void* bf16_buf, void* fp32_buf, size_t count, void* stream) {
@@ -586,12 +594,10 @@ int mi_ccl_convert_bf16_to_fp32_arrays(const void* bf16_buf, void* fp32_buf, siz
         return MI_CCL_SUCCESS;
     if (!fp32_buf || !bf16_buf || ((uintptr_t)fp32_buf & 3u) || ((uintptr_t)bf16_buf & 1u))
         return MI_CCL_INVALID_ARGUMENTS;
-    if (count / 4 / (kBlock * kWidenUnroll) >= 0x7fffffffu)
-        return MI_CCL_INVALID_ARGUMENTS;
-    const CvtShape c = cvt_shape(fp32_buf, 4, count, 4, kWidenUnroll);
-    hipLaunchKernelGGL(bf16_to_f32_kernel, dim3(c.grid), dim3(kBlock), 0, (hipStream_t)stream,
-                       (const uint16_t*)bf16_buf, (uint32_t*)fp32_buf, c.head, c.ngroup, c.tail);
-    return status_of(hipGetLastError());
+    return launch_converter(fp32_buf, 4, count, 4, [&](const LaunchPiece& p, uint64_t skip) {
+        hipLaunchKernelGGL(bf16_to_f32_kernel, dim3(p.grid), dim3(kBlock), 0, (hipStream_t)stream,
+                           (const uint16_t*)bf16_buf + skip, (uint32_t*)fp32_buf + skip, p.head, p.ngroup, p.tail);
+    });
 }
 
 int mi_ccl_convert_fp32_to_fp16_arrays(const void* fp32_buf, void* fp16_buf, size_t count, void* stream) {
@@ -599,12 +605,10 @@ int mi_ccl_convert_fp32_to_fp16_arrays(const void* fp32_buf, void* fp16_buf, siz
         return MI_CCL_SUCCESS;
     if (!fp32_buf || !fp16_buf || ((uintptr_t)fp32_buf & 3u) || ((uintptr_t)fp16_buf & 1u))
         return MI_CCL_INVALID_ARGUMENTS;
-    if (count / 8 / kBlock >= 0x7fffffffu)
-        return MI_CCL_INVALID_ARGUMENTS;
-    const CvtShape c = cvt_shape(fp16_buf, 2, count, 8, 1);
-    hipLaunchKernelGGL(f32_to_f16_kernel, dim3(c.grid), dim3(kBlock), 0, (hipStream_t)stream, (const uint32_t*)fp32_buf,
-                       (uint16_t*)fp16_buf, c.head, c.ngroup, c.tail);
-    return status_of(hipGetLastError());
+    return launch_converter(fp16_buf, 2, count, 8, [&](const LaunchPiece& p, uint64_t skip) {
+        hipLaunchKernelGGL(f32_to_f16_kernel, dim3(p.grid), dim3(kBlock), 0, (hipStream_t)stream,
+                           (const uint32_t*)fp32_buf + skip, (uint16_t*)fp16_buf + skip, p.head, p.ngroup, p.tail);
+    });
 }
 
 int mi_ccl_convert_fp16_to_fp32_arrays(const void* fp16_buf, void* fp32_buf, size_t count, void* stream) {
@@ -612,12 +616,10 @@ int mi_ccl_convert_fp16_to_fp32_arrays(const void* fp16_buf, void* fp32_buf, siz
         return MI_CCL_SUCCESS;
     if (!fp32_buf || !fp16_buf || ((uintptr_t)fp32_buf & 3u) || ((uintptr_t)fp16_buf & 1u))
         return MI_CCL_INVALID_ARGUMENTS;
-    if (count / 4 / kBlock >= 0x7fffffffu)
-        return MI_CCL_INVALID_ARGUMENTS;
-    const CvtShape c = cvt_shape(fp32_buf, 4, count, 4, 1);
-    hipLaunchKernelGGL(f16_to_f32_kernel, dim3(c.grid), dim3(kBlock), 0, (hipStream_t)stream, (const uint16_t*)fp16_buf,
-                       (uint32_t*)fp32_buf, c.head, c.ngroup, c.tail);
-    return status_of(hipGetLastError());
+    return launch_converter(fp32_buf, 4, count, 4, [&](const LaunchPiece& p, uint64_t skip) {
+        hipLaunchKernelGGL(f16_to_f32_kernel, dim3(p.grid), dim3(kBlock), 0, (hipStream_t)stream,
+                           (const uint16_t*)fp16_buf + skip, (uint32_t*)fp32_buf + skip, p.head, p.ngroup, p.tail);
+    });
 }
 
 int mi_ccl_set_param(const char* name, long value) {
@@ -647,6 +649,10 @@ int mi_ccl_set_param(const char* name, long value) {
         g_fp16_impl.store((int)value);
         return MI_CCL_SUCCESS;
     }
+    if (!strcmp(name, "launch_block_limit") && value >= 0) {
+        g_launch_block_limit.store(value);
+        return MI_CCL_SUCCESS;
+    }
     return MI_CCL_INVALID_ARGUMENTS;
 }
 
@@ -665,6 +671,8 @@ long mi_ccl_get_param(const char* name) {
         return g_phased_min_bytes.load();
     if (!strcmp(name, "fp16_impl"))
         return g_fp16_impl.load();
+    if (!strcmp(name, "launch_block_limit"))
+        return g_launch_block_limit.load();
     if (!strcmp(name, "num_cus"))
         return num_cus();
     return -1;

@@ -1,6 +1,7 @@
 // Fusion plans and the extern "C" fusion entry points of libmi_ccl_comp.so.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <new>
 #include <vector>
 
@@ -63,6 +64,35 @@ fusion_copy_kernel(FusionPtrs tensors, unsigned char* fusion_buf, const uint64_t
             copy_span(tp, fp, n);
         else
             copy_span(fp, tp, n);
+    }
+}
+
+// One fused reduce of the traits class that (dtype, 16-bit mode, bf16_impl, a.tune.fp16_impl) selects.
+static hipError_t dispatch_fusion(int dtype, bool keep, int bf16_impl, const FusionLaunchArgs& a) {
+    switch (dtype) {
+        case MI_CCL_INT8: return launch_fusion_reduce<I8Traits>(a);
+        case MI_CCL_UINT8: return launch_fusion_reduce<U8Traits>(a);
+        case MI_CCL_INT16: return launch_fusion_reduce<I16Traits>(a);
+        case MI_CCL_UINT16: return launch_fusion_reduce<U16Traits>(a);
+        case MI_CCL_INT32: return launch_fusion_reduce<I32Traits>(a);
+        case MI_CCL_UINT32: return launch_fusion_reduce<U32Traits>(a);
+        case MI_CCL_INT64: return launch_fusion_reduce<I64Traits>(a);
+        case MI_CCL_UINT64: return launch_fusion_reduce<U64Traits>(a);
+        case MI_CCL_FLOAT16:
+            return a.tune.fp16_impl == MI_CCL_FP16_AVX512FP16 ? launch_fusion_reduce<Fp16NativeTraits>(a)
+                                                              : launch_fusion_reduce<Fp16PairwiseTraits>(a);
+        case MI_CCL_FLOAT32: return launch_fusion_reduce<F32Traits>(a);
+        case MI_CCL_FLOAT64: return launch_fusion_reduce<F64Traits>(a);
+        case MI_CCL_BFLOAT16:
+            if (keep)
+                return (bf16_impl == MI_CCL_BF16_AVX512BF) ? launch_fusion_reduce<Bf16KeepTraits<true>>(a)
+                                                            : launch_fusion_reduce<Bf16KeepTraits<false>>(a);
+            if (bf16_impl == MI_CCL_BF16_SCALAR)
+                return launch_fusion_reduce<Bf16PairScalar>(a);
+            if (bf16_impl == MI_CCL_BF16_AVX512F)
+                return launch_fusion_reduce<Bf16PairAvx512f>(a);
+            return launch_fusion_reduce<Bf16PairAvx512bf>(a);
+        default: return hipErrorInvalidValue;
     }
 }
 
@@ -210,10 +240,12 @@ int mi_ccl_fusion_unpack(mi_ccl_fusion_plan* plan, const void* fusion_buf, void*
 }
 
 int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* own_tensors, const void* const* peers,
-                         int n_peers, void* const* out_tensors, int lp_mode, int bf16_impl, void* stream) {
+                         int n_peers, void* const* out_tensors, int lp_mode, int bf16_impl, int fp16_impl, void* stream) {
     if (!plan || !own_tensors || !out_tensors || n_peers < 0 || n_peers > kFusionMaxPeers || (n_peers && !peers))
         return MI_CCL_INVALID_ARGUMENTS;
     if (op < MI_CCL_SUM || op > MI_CCL_MAX || bf16_impl < MI_CCL_BF16_SCALAR || bf16_impl > MI_CCL_BF16_AVX512BF)
+        return MI_CCL_INVALID_ARGUMENTS;
+    if (fp16_impl != MI_CCL_FP16_DEFAULT && (fp16_impl < MI_CCL_FP16_F16C || fp16_impl > MI_CCL_FP16_AVX512FP16))
         return MI_CCL_INVALID_ARGUMENTS;
     const bool keep = (lp_mode & MI_CCL_LP_KEEP_PRECISION) != 0;
     // the truncated tail of the array converter belongs to the end of the *fused* buffer; this entry point
@@ -244,36 +276,9 @@ int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* ow
     a.item_begin = plan->item_begin.data();
     a.stream = (hipStream_t)stream;
     a.tune = current_tuning();
-    hipError_t e;
-    switch (plan->dtype) {
-        case MI_CCL_INT8: e = launch_fusion_reduce<I8Traits>(a); break;
-        case MI_CCL_UINT8: e = launch_fusion_reduce<U8Traits>(a); break;
-        case MI_CCL_INT16: e = launch_fusion_reduce<I16Traits>(a); break;
-        case MI_CCL_UINT16: e = launch_fusion_reduce<U16Traits>(a); break;
-        case MI_CCL_INT32: e = launch_fusion_reduce<I32Traits>(a); break;
-        case MI_CCL_UINT32: e = launch_fusion_reduce<U32Traits>(a); break;
-        case MI_CCL_INT64: e = launch_fusion_reduce<I64Traits>(a); break;
-        case MI_CCL_UINT64: e = launch_fusion_reduce<U64Traits>(a); break;
-        case MI_CCL_FLOAT16:
-            e = a.tune.fp16_impl == MI_CCL_FP16_AVX512FP16 ? launch_fusion_reduce<Fp16NativeTraits>(a)
-                                                           : launch_fusion_reduce<Fp16PairwiseTraits>(a);
-            break;
-        case MI_CCL_FLOAT32: e = launch_fusion_reduce<F32Traits>(a); break;
-        case MI_CCL_FLOAT64: e = launch_fusion_reduce<F64Traits>(a); break;
-        case MI_CCL_BFLOAT16:
-            if (keep)
-                e = (bf16_impl == MI_CCL_BF16_AVX512BF) ? launch_fusion_reduce<Bf16KeepTraits<true>>(a)
-                                                        : launch_fusion_reduce<Bf16KeepTraits<false>>(a);
-            else if (bf16_impl == MI_CCL_BF16_SCALAR)
-                e = launch_fusion_reduce<Bf16PairScalar>(a);
-            else if (bf16_impl == MI_CCL_BF16_AVX512F)
-                e = launch_fusion_reduce<Bf16PairAvx512f>(a);
-            else
-                e = launch_fusion_reduce<Bf16PairAvx512bf>(a);
-            break;
-        default: e = hipErrorInvalidValue; break;
-    }
-    return fusion_status_of(e);
+    if (fp16_impl != MI_CCL_FP16_DEFAULT)
+        a.tune.fp16_impl = fp16_impl;
+    return fusion_status_of(dispatch_fusion(plan->dtype, keep, bf16_impl, a));
 }
 
 } /* extern "C" */

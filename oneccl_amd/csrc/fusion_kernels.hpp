@@ -118,17 +118,28 @@ fusion_reduce_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 const uint32_t i = tid + u * kBlock;
-                if (i < nvec) st_loose(d + i, vec_finish<TR>(acc[u]));
+                if (i < nvec)
+                    st_loose(d + i, nan_checked<TR, OP>(vec_finish<TR>(acc[u]), n_peers + 1, [&](int j) {
+                                 return j == 0 ? s0 + i : (const u32x4_u*)((const unsigned char*)peers.p[j - 1] + poff + head * ES) + i;
+                             }));
             }
             if (tid < head + tail) {
                 const uint32_t i = (tid < head) ? tid : head + nvec * TR::VEC + (tid - head);
                 typename TR::acc_t r = TR::init(ld_elem<E>(a, i));
                 for (int j = 0; j < n_peers; j++)
-                    r = TR::template step<OP>(ld_elem<E>((const unsigned char*)peers.p[j] + poff, i), r);
+                    r = TR::template step_x86<OP>(ld_elem<E>((const unsigned char*)peers.p[j] + poff, i), r);
                 st_elem<E>(o, i, TR::finish(r));
             }
         }
     }
+}
+
+// Value that lane k of the wave holds, as a wave-uniform (scalar-register) value; k must be the same in every lane.
+__device__ __forceinline__ uint32_t lane_value(uint32_t v, int k) {
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, k);
+}
+__device__ __forceinline__ uint64_t lane_value(uint64_t v, int k) {
+    return (uint64_t)lane_value((uint32_t)v, k) | ((uint64_t)lane_value((uint32_t)(v >> 32), k) << 32);
 }
 
 // Items per phase of the phased fused kernel whose results wait in registers on top of the kPhaseU / 2 that wait in
@@ -186,14 +197,14 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
             }
         }
         for (int k = 0; k < SLOTS; k++) {
-            const uint32_t nb = __shfl(d_nb, k, 64);
+            const uint32_t nb = lane_value(d_nb, k);
             if (nb == 0) break;
-            const unsigned char* a = (const unsigned char*)(uintptr_t)__shfl(d_a, k, 64);
-            unsigned char* o = (unsigned char*)(uintptr_t)__shfl(d_o, k, 64);
-            const uint64_t poff = __shfl(d_poff, k, 64);
+            const unsigned char* a = (const unsigned char*)(uintptr_t)lane_value(d_a, k);
+            unsigned char* o = (unsigned char*)(uintptr_t)lane_value(d_o, k);
+            const uint64_t poff = lane_value(d_poff, k);
             const uint32_t nelem = nb / ES;
             {
-                uint32_t head = __shfl(d_head, k, 64);
+                uint32_t head = lane_value(d_head, k);
                 if (head > nelem) head = nelem;
                 const uint32_t nvec = (nelem - head) / TR::VEC, tail = nelem - head - nvec * TR::VEC;
                 const u32x4_u* s[NT];
@@ -222,19 +233,19 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                     typename TR::acc_t r = TR::init(ld_elem<E>(a, i));
 #pragma unroll
                     for (int j = 0; j < NP; j++)
-                        r = TR::template step<OP>(ld_elem<E>((const unsigned char*)peers.p[j] + poff, i), r);
+                        r = TR::template step_x86<OP>(ld_elem<E>((const unsigned char*)peers.p[j] + poff, i), r);
                     st_elem<E>(o, i, TR::finish(r));
                 }
             }
         }
         phase_barrier(ps, ++gen, give_up);
         for (int k = 0; k < SLOTS; k++) {
-            const uint32_t nb = __shfl(d_nb, k, 64);
+            const uint32_t nb = lane_value(d_nb, k);
             if (nb == 0) break;
-            unsigned char* o = (unsigned char*)(uintptr_t)__shfl(d_o, k, 64);
+            unsigned char* o = (unsigned char*)(uintptr_t)lane_value(d_o, k);
             {
                 const uint32_t nelem = nb / ES;
-                uint32_t head = __shfl(d_head, k, 64);
+                uint32_t head = lane_value(d_head, k);
                 if (head > nelem) head = nelem;
                 const uint32_t nvec = (nelem - head) / TR::VEC;
                 u32x4_u* d = (u32x4_u*)(o + head * ES);

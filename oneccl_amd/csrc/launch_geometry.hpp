@@ -1,0 +1,132 @@
+// Launch geometry of the copy-shaped kernels (copy, broadcast, array converters): plain host arithmetic, kept apart
+// from the kernels so that it can be compiled and tested without a GPU.
+//
+// These kernels give every lane one group of elements (one 16-byte vector, or the 4 or 8 elements that make one) and
+// every block one tile of kGeomBlock groups.  HIP refuses a launch whose gridDim.x * blockDim.x reaches 2^32, i.e. more
+// than 2^24 - 1 blocks of 256 lanes: 64 GiB of copy output.  Larger work is cut into several launches, each over its
+// own contiguous run of tiles.
+#pragma once
+
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define MI_GEOM_HD __host__ __device__
+#else
+#define MI_GEOM_HD
+#endif
+
+namespace mi {
+
+constexpr uint32_t kGeomBlock = 256;
+
+// blocks of `block` lanes one launch may have
+inline uint64_t hip_block_limit(uint32_t block) {
+    return ((1ull << 32) / block) - 1;
+}
+
+// `count` elements written to an array whose first byte is at address `out_addr`: `head` elements up to the array's
+// first 16-byte boundary, then `ngroup` groups of `per` elements (one group per lane), then `tail` elements.  The head
+// and tail elements (fewer than a group each) are handled one per lane by block 0 of a launch.
+struct LaneWork {
+    uint32_t head;
+    uint64_t ngroup;
+    uint32_t tail;
+};
+inline LaneWork lane_work(uint64_t out_addr, uint32_t out_elem_bytes, uint64_t count, uint32_t per) {
+    LaneWork w;
+    const uint64_t mis = out_addr & 15u;
+    uint64_t head = ((16u - mis) & 15u) / out_elem_bytes;
+    if (head > count) head = count;
+    w.head = (uint32_t)head;
+    w.ngroup = (count - head) / per;
+    w.tail = (uint32_t)(count - head - w.ngroup * per);
+    return w;
+}
+
+// One launch of the work: groups [group0, group0 + ngroup) by `grid` blocks; the first launch also takes the head
+// elements and the last one the tail elements.  Pointers are advanced by the caller so that the kernel sees a piece
+// as if it were the whole job (a piece other than the first has no head).
+struct LaunchPiece {
+    uint64_t group0, ngroup;
+    uint32_t head, tail, grid;
+};
+inline uint64_t num_launches(const LaneWork& w, uint32_t block, uint64_t limit) {
+    const uint64_t tiles = (w.ngroup + block - 1) / block;
+    return tiles ? (tiles + limit - 1) / limit : 1;
+}
+inline LaunchPiece launch_piece(const LaneWork& w, uint32_t block, uint64_t limit, uint64_t i) {
+    const uint64_t tiles = (w.ngroup + block - 1) / block;
+    const uint64_t n = num_launches(w, block, limit);
+    const uint64_t t0 = i * limit, t1 = (t0 + limit < tiles) ? t0 + limit : tiles;
+    LaunchPiece p;
+    p.group0 = t0 * block;
+    const uint64_t end = (t1 * block < w.ngroup) ? t1 * block : w.ngroup;
+    p.ngroup = end > p.group0 ? end - p.group0 : 0;
+    p.head = i == 0 ? w.head : 0;
+    p.tail = i == n - 1 ? w.tail : 0;
+    p.grid = (uint32_t)(t1 > t0 ? t1 - t0 : 1);
+    return p;
+}
+
+// One buffer to m buffers.  The source's tiles are taken in sections of `sect_tiles` tiles; within a section, all of
+// its tiles go to destination 0, then all of them to destination 1, and so on: `per` = sect_tiles * m blocks per
+// section.  A launch takes whole sections.
+struct BcastShape {
+    uint32_t head, tail;
+    uint64_t nvec;
+    uint32_t sect_tiles;    // a multiple of 8, so that a tile is always handled on the same XCD
+    uint64_t sects;
+};
+inline BcastShape bcast_shape(uint64_t dst0_addr, uint64_t bytes, uint32_t max_sect_tiles) {
+    const LaneWork w = lane_work(dst0_addr, 1, bytes, 16);
+    BcastShape b;
+    b.head = w.head;
+    b.nvec = w.ngroup;
+    b.tail = w.tail;
+    uint64_t tiles = (b.nvec + kGeomBlock - 1) / kGeomBlock;
+    if (tiles == 0) tiles = 1;
+    b.sect_tiles = tiles < max_sect_tiles ? (uint32_t)((tiles + 7) & ~7ull) : max_sect_tiles;
+    b.sects = (tiles + b.sect_tiles - 1) / b.sect_tiles;
+    return b;
+}
+struct BcastPiece {
+    uint64_t vec0, nvec;    // vectors [vec0, vec0 + nvec) of the source
+    uint32_t head, tail, grid;
+};
+inline uint64_t bcast_sects_per_launch(const BcastShape& b, int m, uint64_t limit) {
+    const uint64_t per = (uint64_t)b.sect_tiles * (uint64_t)m;
+    const uint64_t s = limit / per;
+    return s ? s : 1;
+}
+inline uint64_t bcast_num_launches(const BcastShape& b, int m, uint64_t limit) {
+    const uint64_t s = bcast_sects_per_launch(b, m, limit);
+    return (b.sects + s - 1) / s;
+}
+inline BcastPiece bcast_piece(const BcastShape& b, int m, uint64_t limit, uint64_t i) {
+    const uint64_t s = bcast_sects_per_launch(b, m, limit), n = bcast_num_launches(b, m, limit);
+    const uint64_t s0 = i * s, s1 = (s0 + s < b.sects) ? s0 + s : b.sects;
+    BcastPiece p;
+    p.vec0 = s0 * b.sect_tiles * kGeomBlock;
+    const uint64_t end = (s1 * b.sect_tiles * kGeomBlock < b.nvec) ? s1 * b.sect_tiles * kGeomBlock : b.nvec;
+    p.nvec = end > p.vec0 ? end - p.vec0 : 0;
+    p.head = i == 0 ? b.head : 0;
+    p.tail = i == n - 1 ? b.tail : 0;
+    p.grid = (uint32_t)((s1 - s0) * b.sect_tiles * (uint64_t)m);
+    return p;
+}
+// which destination and which vector of the piece a lane of block `blk` handles
+struct BcastLane {
+    uint32_t dst;
+    uint64_t vec;
+};
+MI_GEOM_HD inline BcastLane bcast_lane(uint32_t blk, uint32_t tid, uint32_t sect_tiles, uint32_t m) {
+    const uint32_t per = sect_tiles * m;
+    const uint32_t sect = blk / per, r = blk - sect * per;
+    const uint32_t k = r / sect_tiles, t = r - k * sect_tiles;
+    BcastLane l;
+    l.dst = k;
+    l.vec = ((uint64_t)sect * sect_tiles + t) * kGeomBlock + tid;
+    return l;
+}
+
+}  // namespace mi

@@ -18,13 +18,13 @@ int main() {
         void* b[5];
         for (int i = 0; i < 5; i++) { CK(hipMalloc(&b[i], bytes)); CK(hipMemset(b[i], 0, bytes)); }
         const void* srcs[4] = { b[0], b[1], b[2], b[3] };
-        for (int i = 0; i < 50; i++) mi_ccl_comp_reduce_n(MI_CCL_INT32, MI_CCL_SUM, srcs, 4, b[4], bytes / 4, 0, 2, s);
+        for (int i = 0; i < 50; i++) mi_ccl_comp_reduce_n(MI_CCL_INT32, MI_CCL_SUM, srcs, 4, b[4], bytes / 4, 0, 2, 0, s);
         CK(hipStreamSynchronize(s));
         hipEvent_t e0, e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
         const int iters = 2000;
         auto t0 = std::chrono::steady_clock::now();
         CK(hipEventRecord(e0, s));
-        for (int i = 0; i < iters; i++) mi_ccl_comp_reduce_n(MI_CCL_INT32, MI_CCL_SUM, srcs, 4, b[4], bytes / 4, 0, 2, s);
+        for (int i = 0; i < iters; i++) mi_ccl_comp_reduce_n(MI_CCL_INT32, MI_CCL_SUM, srcs, 4, b[4], bytes / 4, 0, 2, 0, s);
         CK(hipEventRecord(e1, s));
         auto t1 = std::chrono::steady_clock::now();
         CK(hipStreamSynchronize(s));
@@ -32,7 +32,7 @@ int main() {
         float ms; CK(hipEventElapsedTime(&ms, e0, e1));
         // single call + sync latency
         auto t3 = std::chrono::steady_clock::now();
-        for (int i = 0; i < 200; i++) { mi_ccl_comp_reduce_n(MI_CCL_INT32, MI_CCL_SUM, srcs, 4, b[4], bytes / 4, 0, 2, s); CK(hipStreamSynchronize(s)); }
+        for (int i = 0; i < 200; i++) { mi_ccl_comp_reduce_n(MI_CCL_INT32, MI_CCL_SUM, srcs, 4, b[4], bytes / 4, 0, 2, 0, s); CK(hipStreamSynchronize(s)); }
         auto t4 = std::chrono::steady_clock::now();
         printf("%8zu B x4: back-to-back %.2f us/call on GPU clock, host enqueue %.2f us/call, wall incl. drain %.2f us/call; call+sync %.2f us\n", bytes,
                ms * 1e3 / iters, std::chrono::duration<double, std::micro>(t1 - t0).count() / iters,

@@ -1,0 +1,129 @@
+// Host-only test of the launch geometry of the copy-shaped kernels (oneccl_amd/csrc/launch_geometry.hpp): for sizes
+// from one byte to 256 GiB and 1..16 destinations, every launch stays below HIP's limit of 2^32 lanes per grid, and
+// the launches together give every group of elements to exactly one lane (intervals checked at every size; every
+// lane enumerated at small sizes and with small artificial limits, through the same index function the kernel uses).
+#include <stdio.h>
+
+#include <map>
+#include <vector>
+
+#include "../../oneccl_amd/csrc/launch_geometry.hpp"
+
+using namespace mi;
+
+static int failed = 0, checks = 0;
+#define EXPECT(c)                                                       \
+    do {                                                                \
+        checks++;                                                       \
+        if (!(c)) {                                                     \
+            failed++;                                                   \
+            printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #c);       \
+        }                                                               \
+    } while (0)
+
+static void check_lane_work(uint64_t addr, uint32_t esz, uint64_t count, uint32_t per, uint64_t limit, bool enumerate) {
+    const LaneWork w = lane_work(addr, esz, count, per);
+    EXPECT((uint64_t)w.head + w.ngroup * per + w.tail == count);
+    EXPECT(w.tail < per && w.head < 16 / esz + 1);
+    EXPECT(w.head == count || ((addr + (uint64_t)w.head * esz) & 15u) == 0);
+    EXPECT(w.head + w.tail <= kGeomBlock);                 // one lane of block 0 each
+    const uint64_t n = num_launches(w, kGeomBlock, limit);
+    uint64_t next = 0, heads = 0, tails = 0;
+    for (uint64_t i = 0; i < n; i++) {
+        const LaunchPiece p = launch_piece(w, kGeomBlock, limit, i);
+        EXPECT(p.group0 == next);
+        EXPECT(p.grid >= 1 && (uint64_t)p.grid <= limit);
+        EXPECT((uint64_t)p.grid * kGeomBlock < (1ull << 32));
+        EXPECT((uint64_t)p.grid * kGeomBlock >= p.ngroup);              // a lane for every group
+        EXPECT(p.ngroup + kGeomBlock > (uint64_t)p.grid * kGeomBlock || p.ngroup == 0);     // no idle block
+        if (n > 1) EXPECT(p.ngroup > 0);
+        if (enumerate) {
+            std::vector<int> seen(p.ngroup, 0);
+            for (uint32_t b = 0; b < p.grid; b++)
+                for (uint32_t t = 0; t < kGeomBlock; t++) {
+                    const uint64_t g = (uint64_t)b * kGeomBlock + t;    // what the kernels compute
+                    if (g < p.ngroup) seen[g]++;
+                }
+            for (int s : seen) EXPECT(s == 1);
+        }
+        next += p.ngroup;
+        heads += p.head;
+        tails += p.tail;
+    }
+    EXPECT(next == w.ngroup && heads == w.head && tails == w.tail);
+}
+
+static void check_bcast(uint64_t addr, uint64_t bytes, int m, uint32_t max_sect, uint64_t limit, bool enumerate) {
+    const BcastShape b = bcast_shape(addr, bytes, max_sect);
+    EXPECT((uint64_t)b.head + b.nvec * 16 + b.tail == bytes);
+    EXPECT(b.sect_tiles % 8 == 0 && b.sect_tiles <= max_sect && b.sect_tiles >= 8);
+    EXPECT(b.sects * b.sect_tiles * kGeomBlock >= b.nvec);
+    const uint64_t n = bcast_num_launches(b, m, limit);
+    uint64_t next = 0, heads = 0, tails = 0;
+    for (uint64_t i = 0; i < n; i++) {
+        const BcastPiece p = bcast_piece(b, m, limit, i);
+        EXPECT(p.vec0 == next);
+        EXPECT((uint64_t)p.grid * kGeomBlock < (1ull << 32));
+        EXPECT((uint64_t)p.grid <= limit || bcast_sects_per_launch(b, m, limit) == 1);
+        EXPECT(p.grid % (b.sect_tiles * (uint32_t)m) == 0 && p.grid > 0);
+        EXPECT((uint64_t)p.grid / m * kGeomBlock >= p.nvec);
+        if (enumerate) {
+            std::map<std::pair<uint32_t, uint64_t>, int> seen;
+            for (uint32_t blk = 0; blk < p.grid; blk++)
+                for (uint32_t t = 0; t < kGeomBlock; t += (blk % 7 == 0 ? 1 : 85)) {    // every lane of some blocks, a few of the others
+                    const BcastLane l = bcast_lane(blk, t, b.sect_tiles, (uint32_t)m);
+                    EXPECT(l.dst < (uint32_t)m);
+                    if (l.vec < p.nvec) seen[{ l.dst, l.vec }]++;
+                }
+            for (auto& kv : seen) EXPECT(kv.second == 1);
+            // every (destination, vector) pair of the piece has its lane: count the pairs block by block
+            uint64_t pairs = 0;
+            for (uint32_t blk = 0; blk < p.grid; blk++) {
+                const BcastLane first = bcast_lane(blk, 0, b.sect_tiles, (uint32_t)m);
+                if (first.vec < p.nvec) pairs += (p.nvec - first.vec < kGeomBlock) ? p.nvec - first.vec : kGeomBlock;
+            }
+            EXPECT(pairs == p.nvec * (uint64_t)m);
+        }
+        next += p.nvec;
+        heads += p.head;
+        tails += p.tail;
+    }
+    EXPECT(next == b.nvec && heads == b.head && tails == b.tail);
+}
+
+int main() {
+    EXPECT(hip_block_limit(256) == (1u << 24) - 1);
+    const uint64_t hw = hip_block_limit(kGeomBlock);
+    // sizes 1 B ... 256 GiB (x2 steps, with odd neighbours), every misalignment class, the real limit
+    for (int sh = 0; sh <= 38; sh++)
+        for (int64_t d : { -17, -1, 0, 1, 4099 }) {
+            const int64_t bytes = (int64_t)(1ull << sh) + d;
+            if (bytes <= 0) continue;
+            for (uint64_t addr : { 0x7f0000000000ull, 0x7f0000000003ull, 0x7f000000000eull }) {
+                check_lane_work(addr, 1, (uint64_t)bytes, 16, hw, false);                        // copy
+                check_lane_work(addr & ~1ull, 2, (uint64_t)bytes / 2 + 1, 8, hw, false);         // fp32 -> 16-bit
+                check_lane_work(addr & ~3ull, 4, (uint64_t)bytes / 4 + 1, 4, hw, false);         // 16-bit -> fp32
+                for (int m = 1; m <= 16; m++) check_bcast(addr, (uint64_t)bytes, m, 4096, hw, false);
+            }
+        }
+    // a 64 GiB copy is the first that needs two launches; 1 -> 7 from 9.2 GiB likewise
+    {
+        const LaneWork w = lane_work(0, 1, 64ull << 30, 16);
+        EXPECT(num_launches(w, kGeomBlock, hw) == 2);
+        EXPECT(num_launches(lane_work(0, 1, (64ull << 30) - 4096, 16), kGeomBlock, hw) == 1);
+        const BcastShape b = bcast_shape(0, 10ull << 30, 4096);
+        EXPECT(bcast_num_launches(b, 7, hw) == 2 && bcast_num_launches(b, 6, hw) == 1);
+    }
+    // small sizes and small artificial limits, every lane enumerated
+    for (uint64_t limit : { 1ull, 2ull, 3ull, 7ull, 64ull, 1000ull })
+        for (uint64_t bytes : { 1ull, 15ull, 16ull, 17ull, 4095ull, 4096ull, 4097ull, 65536ull, 100003ull, 1048576ull + 5 })
+            for (uint64_t addr : { 0ull, 5ull, 15ull }) {
+                check_lane_work(addr, 1, bytes, 16, limit, true);
+                check_lane_work(addr & ~1ull, 2, bytes, 8, limit, true);
+                check_lane_work(addr & ~3ull, 4, bytes, 4, limit, true);
+                for (int m : { 1, 2, 3, 7, 16 })
+                    for (uint32_t max_sect : { 8u, 16u, 4096u }) check_bcast(addr, bytes, m, max_sect, limit, true);
+            }
+    printf("%d checks, %d failed\n", checks, failed);
+    return failed ? 1 : 0;
+}

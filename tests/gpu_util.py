@@ -46,8 +46,10 @@ def make_inputs(rng, dtype, count, op, n, kind="config"):
     return out
 
 
-def assert_same(got, want, dtype, what=""):
-    ok = O.same_bits_or_both_nan(got, want, dtype)
+def assert_same(got, want, dtype, what="", srcs=None, op=None, **kw):
+    """Bit equality; with srcs (chain order) and op given, NaN results of sum/prod steps that had two NaN operands
+    compare as a class (oracle_lib.same_bits)."""
+    ok = O.same_bits(got, want, dtype, srcs, op, **kw)
     if not ok.all():
         bad = np.flatnonzero(~ok)
         raise AssertionError(f"{what}: {bad.size} of {ok.size} elements differ, first at {bad[:5]}: "

@@ -210,20 +210,50 @@ def bf16_to_f32(h):
     return (np.asarray(h, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
 
 
-def same_bits_or_both_nan(a, b, dtype):
-    """Bit equality, except that two NaNs of a floating type compare equal whatever their payload."""
+def nan_mask(a, dtype):
+    """Which elements are NaNs (16-bit floats travel as raw uint16)."""
     a = np.asarray(a)
-    b = np.asarray(b)
-    eq = a == b if dtype not in (FLOAT32, FLOAT64) else a.view(np.uint32 if dtype == FLOAT32 else np.uint64) == \
-        b.view(np.uint32 if dtype == FLOAT32 else np.uint64)
-    if dtype == FLOAT32 or dtype == FLOAT64:
-        eq = eq | (np.isnan(a) & np.isnan(b))
-    elif dtype == BFLOAT16:
-        na = ((a & 0x7F80) == 0x7F80) & ((a & 0x7F) != 0)
-        nb = ((b & 0x7F80) == 0x7F80) & ((b & 0x7F) != 0)
-        eq = eq | (na & nb)
-    elif dtype == FLOAT16:
-        na = ((a & 0x7C00) == 0x7C00) & ((a & 0x3FF) != 0)
-        nb = ((b & 0x7C00) == 0x7C00) & ((b & 0x3FF) != 0)
-        eq = eq | (na & nb)
+    if dtype == FLOAT32:
+        return (a.view(np.uint32) & 0x7FFFFFFF) > 0x7F800000
+    if dtype == FLOAT64:
+        return (a.view(np.uint64) & 0x7FFFFFFFFFFFFFFF) > 0x7FF0000000000000
+    if dtype == BFLOAT16:
+        return (a & 0x7FFF) > 0x7F80
+    if dtype == FLOAT16:
+        return (a & 0x7FFF) > 0x7C00
+    return np.zeros(a.shape, bool)
+
+
+def two_nan_steps(srcs, dtype, op, idx, **kw):
+    """Of the elements idx: those at which some step of the chain srcs[0] OP srcs[1] OP ... has two NaN operands.
+    Only there is the result's payload not fixed by the reference (which of two NaN operands an x86 add or
+    multiply hands back depends on the operand order its compiler chose)."""
+    kw = dict(kw)
+    kw.pop("quirk_tail", None)      # how the tail is narrowed does not change which values are NaNs
+    sub = [np.ascontiguousarray(np.asarray(s)[idx]) for s in srcs]
+    amb = np.zeros(len(idx), bool)
+    acc_nan = nan_mask(sub[0], dtype)
+    for j in range(1, len(sub)):
+        amb |= acc_nan & nan_mask(sub[j], dtype)
+        acc_nan = nan_mask(reduce_n(sub[:j + 1], dtype, op, **kw), dtype)
+    return amb
+
+
+def same_bits(got, want, dtype, srcs=None, op=None, **kw):
+    """Bit equality per element.  The one exception: with srcs (the inputs in chain order, inout first) and op sum or
+    prod of a floating type, two NaNs also compare equal at elements where a step of the chain had two NaN
+    operands.  A NaN made from one NaN operand (that operand, quieted) or from none (the negative default NaN of
+    x86) is compared on bits like any other value.  kw: keep, bf16_impl, fp16_impl as for reduce_n."""
+    got = np.asarray(got)
+    want = np.asarray(want)
+    u = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[got.dtype.itemsize]
+    eq = got.view(u) == want.view(u)
+    if eq.all() or srcs is None or op not in (SUM, PROD) or dtype not in (FLOAT16, FLOAT32, FLOAT64, BFLOAT16):
+        return eq
+    bad = np.flatnonzero(~eq.ravel())
+    cand = bad[nan_mask(got.ravel()[bad], dtype) & nan_mask(want.ravel()[bad], dtype)]
+    if cand.size:
+        amb = two_nan_steps([np.asarray(s).ravel() for s in srcs], dtype, op, cand, **kw)
+        eq = eq.copy()
+        eq.ravel()[cand[amb]] = True
     return eq

@@ -49,7 +49,7 @@ def test_host_only_entry_points():
         c.set_param("no_such_knob", 1)
     # count == 0 is a successful no-op before any argument is looked at (comp.cpp:132-134)
     L = c.lib()
-    assert L.mi_ccl_comp_reduce(0, 0, None, 0, None, 2, None) == 0
+    assert L.mi_ccl_comp_reduce(0, 0, None, 0, None, 2, 0, None) == 0
     assert L.mi_ccl_comp_copy(None, None, 0, 0, None) == 0
 
 

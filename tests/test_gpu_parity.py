@@ -1,6 +1,8 @@
 """GPU parity: the HIP path, called through the C ABI (ctypes binding oneccl_amd.comp), against the CPU oracle
-and against the golden vectors made by the reference's own code.  Bit-exact for every type; two NaNs of a
-floating type compare equal whatever their payload (the reference itself does not pin it for sum/prod)."""
+and against the golden vectors made by the reference's own code.  Bit-exact for every type, NaN results of sum and
+prod included (one NaN operand comes back quieted, an invalid operation gives the negative default NaN of x86); only
+where a step of the chain meets two NaN operands do two NaNs compare equal whatever their payload (which of the two
+the reference returns was its compiler's choice)."""
 import numpy as np
 import pytest
 
@@ -49,7 +51,7 @@ def test_reduce_n_all_dtypes_ops(comp, dtype, op):
                     want = O.reduce_n(srcs, dtype, op, keep=keep, quirk_tail=quirk, bf16_impl=impl)
                     assert_same(to_host(out, O.NP_STORAGE[dtype]), want, dtype,
                                 f"dtype={O.DTYPE_NAMES[dtype]} op={O.OP_NAMES[op]} n={n} count={count} "
-                                f"kind={kind} lp={lp} impl={impl}")
+                                f"kind={kind} lp={lp} impl={impl}", srcs, op, keep=keep, bf16_impl=impl)
 
 
 @pytest.mark.parametrize("fam,dtype", [("bf16", O.BFLOAT16), ("fp16", O.FLOAT16)])
@@ -70,7 +72,8 @@ def test_pairwise_against_reference_made_golden_vectors(comp, golden, fam, dtype
             da, db = to_dev(a), to_dev(b)
             comp.comp_reduce(dtype, op, da, a.size, db, bf16_impl=impl if fam == "bf16" else 2)
             torch.cuda.synchronize()
-            assert_same(to_host(db, np.uint16), golden[stem + f"_impl{impl}"], dtype, f"{stem} impl{impl}")
+            assert_same(to_host(db, np.uint16), golden[stem + f"_impl{impl}"], dtype, f"{stem} impl{impl}", [b, a], op,
+                        bf16_impl=impl if fam == "bf16" else 2)
             checked += 1
     assert checked >= 4 * 11 * 2
 
@@ -92,7 +95,8 @@ def test_special_value_pairs_against_golden(comp, golden, fam, dtype):
             if op in (O.MIN, O.MAX):
                 assert (got == want).all(), (fam, op, impl, np.flatnonzero(got != want)[:8])
             else:
-                assert_same(got, want, dtype, f"{fam} specials op={op} impl={impl}")
+                assert_same(got, want, dtype, f"{fam} specials op={op} impl={impl}", [b, a], op,
+                            bf16_impl=impl if fam == "bf16" else 2)
     if fam == "bf16":   # scalar impl has no golden (not vector code): oracle, pinned by the recorded probes
         for op in range(4):
             da, db = to_dev(a), to_dev(b)
@@ -103,7 +107,7 @@ def test_special_value_pairs_against_golden(comp, golden, fam, dtype):
             if op in (O.MIN, O.MAX):
                 assert (got == want).all()
             else:
-                assert_same(got, want, dtype)
+                assert_same(got, want, dtype, f"bf16 specials op={op} scalar", [b, a], op, bf16_impl=0)
 
 
 def test_recorded_probe_values_on_gpu(comp, probes):
@@ -179,16 +183,16 @@ def test_misaligned_and_inplace(comp, dtype):
             comp.comp_reduce_n(dtype, op, ptrs, outbig.data_ptr() + lo * esz, count)
             torch.cuda.synchronize()
             o = to_host(outbig, np_t)
-            assert_same(o[lo:lo + count], want, dtype, f"shifts={shifts}")
+            assert_same(o[lo:lo + count], want, dtype, f"shifts={shifts}", srcs, op)
             assert (o[:lo] == 0).all() and (o[lo + count:] == 0).all(), "wrote outside the destination"
         d = [to_dev(s) for s in srcs]
         comp.comp_reduce_n(dtype, op, d, d[0], count)          # in place on the own buffer
         torch.cuda.synchronize()
-        assert_same(to_host(d[0], np_t), want, dtype, "in place")
+        assert_same(to_host(d[0], np_t), want, dtype, "in place", srcs, op)
         d = [to_dev(s) for s in srcs]
         comp.comp_reduce_n(dtype, op, d, d[2], count)          # output aliases a later input
         torch.cuda.synchronize()
-        assert_same(to_host(d[2], np_t), want, dtype, "alias")
+        assert_same(to_host(d[2], np_t), want, dtype, "alias", srcs, op)
 
 
 def test_batch_reduce_slices_keep_precision_tail(comp):
@@ -209,7 +213,10 @@ def test_batch_reduce_slices_keep_precision_tail(comp):
                         comp.comp_batch_reduce(d, offs, count, d, O.BFLOAT16, op, keep, bf16_impl=impl)
                         torch.cuda.synchronize()
                         want = O.batch_reduce(buf, offs, count, O.BFLOAT16, op, keep, bf16_impl=impl)
-                        assert_same(to_host(d, np.uint16), want, O.BFLOAT16, f"count={count} n={n} op={op} keep={keep} impl={impl}")
+                        got = to_host(d, np.uint16)
+                        what = f"count={count} n={n} op={op} keep={keep} impl={impl}"
+                        assert_same(got[:count], want[:count], O.BFLOAT16, what, slices, op, keep=keep, bf16_impl=impl)
+                        assert (got[count:] == want[count:]).all(), what + ": the other slices changed"
 
 
 def test_copy_and_converters(comp):
@@ -357,7 +364,7 @@ def test_all_pairs_of_16bit_values_sum_and_prod(comp, dtype, impl):
             comp.comp_reduce(dtype, op, da, a.size, db, bf16_impl=2)
             torch.cuda.synchronize()
             want = O.reduce_n([b, a], dtype, op, bf16_impl=impl, fp16_impl=3, threads=16)
-            assert_same(to_host(db, np.uint16), want, dtype, f"op={op} rows from {r0}")
+            assert_same(to_host(db, np.uint16), want, dtype, f"op={op} rows from {r0}", [b, a], op, bf16_impl=impl, fp16_impl=3)
 
 
 def test_arguments_and_errors(comp):
@@ -406,7 +413,8 @@ def test_phased_kernel_parity(comp, dtype, op, n):
             torch.cuda.synchronize()
             want = O.reduce_n([s[shift:] for s in srcs], dtype, op, keep=1 if dtype == O.BFLOAT16 else 0, threads=16)
             got = to_host(out, O.NP_STORAGE[dtype])
-            assert_same(got[shift:], want, dtype, f"phased count={count} shift={shift}")
+            assert_same(got[shift:], want, dtype, f"phased count={count} shift={shift}", [s[shift:] for s in srcs], op,
+                        keep=1 if dtype == O.BFLOAT16 else 0)
             assert (got[:shift] == 0).all()
     finally:
         comp.set_param("variant", 0)
@@ -455,7 +463,7 @@ def test_buffers_that_disagree_modulo_16_bytes(comp, variant, dtype, op, n, m):
                 torch.cuda.synchronize()
                 for o_, k in zip(outs, sh[n:]):
                     g = to_host(o_, np_t)
-                    assert_same(g[pad + k:pad + k + count], want, dtype, f"count={count} shifts={sh}")
+                    assert_same(g[pad + k:pad + k + count], want, dtype, f"count={count} shifts={sh}", srcs, op, keep=keep)
                     assert not g[:pad + k].view(np.uint8).any() and not g[pad + k + count:].view(np.uint8).any(), \
                         f"wrote outside a destination: count={count} shifts={sh}"
     finally:
@@ -515,10 +523,10 @@ def test_randomised_calls_against_oracle(comp):
         got = to_host(out_holder, np_t)
         what = (f"case {case}: dtype={O.DTYPE_NAMES[dtype]} op={O.OP_NAMES[op]} n={n} m={m} count={count} lp={lp} impl={impl} "
                 f"shifts={shifts} alias={alias} variant={variant} kind={kind}")
-        assert_same(got[out_lo:out_lo + count], want, dtype, what)
+        assert_same(got[out_lo:out_lo + count], want, dtype, what, srcs, op, keep=keep, bf16_impl=impl)
         for h, lo in extra:
             g2 = to_host(h, np_t)
-            assert_same(g2[lo:lo + count], want, dtype, what + " (further destination)")
+            assert_same(g2[lo:lo + count], want, dtype, what + " (further destination)", srcs, op, keep=keep, bf16_impl=impl)
             assert (g2[:lo] == 0).all() and (g2[lo + count:] == 0).all(), what + ": wrote outside a further destination"
         if alias < 0:
             assert (got[:out_lo] == 0).all() and (got[out_lo + count:] == 0).all(), what + ": wrote outside the destination"
@@ -528,7 +536,7 @@ def test_randomised_calls_against_oracle(comp):
 
 def test_fp16_native_mode_against_reference_made_vectors(comp, golden, golden_fp16_native):
     """fp16_impl = avx512fp16 (mi_ccl_set_param): the GPU against what the reference's native-fp16 code produced --
-    bits for min/max (a signalling NaN that is handed back stays signalling), NaNs as a class for sum/prod --
+    bits for min/max (a signalling NaN that is handed back stays signalling) and for sum/prod (two NaN operands aside) --
     then the N-input and multi-destination forms against the oracle in the same mode."""
     import torch
     from test_oracle_pins import _fp16_native_cases
@@ -544,7 +552,7 @@ def test_fp16_native_mode_against_reference_made_vectors(comp, golden, golden_fp
             if op in (O.MIN, O.MAX):
                 assert (got == want).all(), (name, np.flatnonzero(got != want)[:8])
             else:
-                assert_same(got, want, O.FLOAT16, name)
+                assert_same(got, want, O.FLOAT16, name, [b, a], op, fp16_impl=O.FP16_AVX512FP16)
             n += 1
         assert n == 96
         rng = np.random.default_rng(123)
@@ -558,7 +566,7 @@ def test_fp16_native_mode_against_reference_made_vectors(comp, golden, golden_fp
             for o in outs:
                 got = to_host(o, np.uint16)
                 if op == O.SUM:
-                    assert_same(got, want, O.FLOAT16, "native fp16 sum")
+                    assert_same(got, want, O.FLOAT16, "native fp16 sum", srcs, op, fp16_impl=O.FP16_AVX512FP16)
                 else:
                     assert (got == want).all()
     finally:

@@ -45,7 +45,7 @@ def test_reduce_write_n_all_dtypes_ops(comp, dtype, op):
                     got = to_host(outs[k], O.NP_STORAGE[dtype])
                     assert_same(got[:count], want[k], dtype,
                                 f"dtype={O.DTYPE_NAMES[dtype]} op={O.OP_NAMES[op]} n={n} m={m} k={k} count={count} "
-                                f"lp={lp} impl={impl}")
+                                f"lp={lp} impl={impl}", srcs, op, keep=keep, bf16_impl=impl)
                     assert not got[count:].view(np.uint8).any(), "wrote past the end"
 
 

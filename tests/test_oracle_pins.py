@@ -32,7 +32,7 @@ def test_golden_pairwise(golden, fam, dtype):
         for impl in impls:
             want = golden[stem + f"_impl{impl}"]
             got = O.comp_reduce(a, b, dtype, op, bf16_impl=impl, fp16_impl=impl)
-            ok = O.same_bits_or_both_nan(got, want, dtype)
+            ok = O.same_bits(got, want, dtype, [b, a], op, bf16_impl=impl, fp16_impl=impl)
             assert ok.all(), (stem, impl, np.flatnonzero(~ok)[:5], a[~ok][:5], b[~ok][:5], got[~ok][:5], want[~ok][:5])
             checked += 1
     assert checked >= 2 * 4 * 11 * 2
@@ -41,7 +41,7 @@ def test_golden_pairwise(golden, fam, dtype):
 @pytest.mark.parametrize("fam,dtype", [("bf16", O.BFLOAT16), ("fp16", O.FLOAT16)])
 def test_golden_special_pairs_exact(golden, fam, dtype):
     """All pairs of special values.  For min/max the result is one of the operands, so NaN payloads are
-    pinned too and the comparison is on bits; sum/prod compare NaNs as a class."""
+    pinned too and the comparison is on bits; so is it for sum/prod, except where both operands are NaNs."""
     impls = (1, 2) if fam == "bf16" else (2, 3)
     a, b = golden[f"{fam}_specials_in"], golden[f"{fam}_specials_inout"]
     for op in range(4):
@@ -51,7 +51,7 @@ def test_golden_special_pairs_exact(golden, fam, dtype):
             if op in (O.MIN, O.MAX):
                 assert (got == want).all(), (fam, op, impl, np.flatnonzero(got != want)[:8])
             else:
-                assert O.same_bits_or_both_nan(got, want, dtype).all(), (fam, op, impl)
+                assert O.same_bits(got, want, dtype, [b, a], op, bf16_impl=impl, fp16_impl=impl).all(), (fam, op, impl)
 
 
 def test_golden_converters(golden):
@@ -261,7 +261,7 @@ def test_fp_sum_prod_are_single_ieee_ops_in_chain_order(dtype, np_t):
             for s in srcs[1:]:
                 want = f(want, s)          # numpy elementwise ops are single IEEE operations
         got = O.reduce_n(srcs, dtype, op)
-        assert O.same_bits_or_both_nan(got, want, dtype).all()
+        assert O.same_bits(got, want, dtype).all()
     # exact fractions: ((0.1f + 0.2f) + 0.3f) differs from (0.1f + (0.2f + 0.3f)) -- order matters
     x = [np.full(4, v, np_t) for v in (0.1, 0.2, 0.3)]
     assert (O.reduce_n(x, dtype, O.SUM) == (x[0] + x[1]) + x[2]).all()
@@ -360,13 +360,13 @@ def test_reduce_n_equals_chain_of_pairwise(dtype, op):
     for s in srcs[1:]:
         want = O.comp_reduce(s, want, dtype, op)
     got = O.reduce_n(srcs, dtype, op)
-    assert O.same_bits_or_both_nan(got, want, dtype).all()
+    assert O.same_bits(got, want, dtype, srcs, op).all()
     # slice form (ccl_comp_batch_reduce, keep_precision 0) and the partitioned form agree too
     buf = np.concatenate(srcs)
     got2 = O.batch_reduce(buf, [i * count for i in range(n)], count, dtype, op, 0)[:count]
-    assert O.same_bits_or_both_nan(got2, want, dtype).all()
+    assert O.same_bits(got2, want, dtype, srcs, op).all()
     got3 = O.reduce_n(srcs, dtype, op, threads=3)
-    assert O.same_bits_or_both_nan(got3, want, dtype).all()
+    assert O.same_bits(got3, want, dtype, srcs, op).all()
 
 
 @pytest.mark.parametrize("impl", [0, 1, 2])
@@ -445,7 +445,7 @@ def test_against_reference_code_random(fam, dtype, impls):
                 if op in (O.MIN, O.MAX):
                     assert (got == want).all()
                 else:
-                    assert O.same_bits_or_both_nan(got, want, dtype).all()
+                    assert O.same_bits(got, want, dtype, [b, a], op, bf16_impl=impl, fp16_impl=impl).all()
 
 
 @needs_ref
@@ -475,7 +475,8 @@ def test_keep_precision_batch_reduce_against_the_reference_helpers_in_its_pass_s
                 got = buf.copy()
                 assert L.orc_comp_batch_reduce(got.ctypes.data, offs.ctypes.data, n, count, got.ctypes.data, O.BFLOAT16,
                                                O.SUM, 1, tmp.ctypes.data, acc.ctypes.data, impl, O.FP16_AVX512F) == 0
-                assert O.same_bits_or_both_nan(got[:count], want[:count], O.BFLOAT16).all(), (n, count, kind)
+                slices = [buf[i * count:(i + 1) * count] for i in range(n)]
+                assert O.same_bits(got[:count], want[:count], O.BFLOAT16, slices, O.SUM, keep=1, bf16_impl=impl).all(), (n, count, kind)
                 assert (got[count:] == buf[count:]).all()
 
 
@@ -489,7 +490,7 @@ def test_against_reference_code_every_bf16_pair_sampled():
     want = b.copy()
     assert R.ref_bf16_reduce(a.ctypes.data, a.size, want.ctypes.data, O.SUM, 2) == 0
     got = O.comp_reduce(a, b, O.BFLOAT16, O.SUM, bf16_impl=2)
-    assert O.same_bits_or_both_nan(got, want, O.BFLOAT16).all()
+    assert O.same_bits(got, want, O.BFLOAT16, [b, a], O.SUM, bf16_impl=2).all()
 
 
 def test_reduce_write_n_is_reduce_n_stored_m_times():
@@ -507,7 +508,7 @@ def test_reduce_write_n_is_reduce_n_stored_m_times():
         for alias in (None, (m - 1, n - 1)):
             outs = O.reduce_write_n(srcs, m, dtype, op, alias=alias)
             for o in outs:
-                assert O.same_bits_or_both_nan(o, want, dtype).all()
+                assert O.same_bits(o, want, dtype).all()
     src = rng.integers(0, 65536, 517, dtype=np.uint16)      # any bf16 bit pattern, NaNs and denormals included
     for o in O.reduce_write_n([src], 7, O.BFLOAT16, O.SUM):
         assert (o == src).all()
@@ -536,14 +537,14 @@ def _fp16_native_cases(golden, native):
 
 def test_fp16_avx512fp16_against_reference_made_vectors(golden, golden_fp16_native):
     """The native-fp16 implementation (fp16_intrisics.cpp:23-41): min/max return one operand untouched, so bits
-    are compared, signalling NaNs included; sum/prod compare NaNs as a class."""
+    are compared, signalling NaNs included; sum/prod compare on bits too, except where both operands are NaNs."""
     n = 0
     for name, op, a, b, want in _fp16_native_cases(golden, golden_fp16_native):
         got = O.comp_reduce(a, b, O.FLOAT16, op, fp16_impl=O.FP16_AVX512FP16)
         if op in (O.MIN, O.MAX):
             assert (got == want).all(), (name, np.flatnonzero(got != want)[:8])
         else:
-            assert O.same_bits_or_both_nan(got, want, O.FLOAT16).all(), name
+            assert O.same_bits(got, want, O.FLOAT16, [b, a], op, fp16_impl=O.FP16_AVX512FP16).all(), name
         n += 1
     assert n == 4 * 11 * 2 + 4 + 4
     # and the point of the mode: a signalling NaN handed back by min/max stays signalling, the other modes quiet it
@@ -574,4 +575,44 @@ def test_fp16_avx512fp16_against_reference_library_when_built():
         if op in (O.MIN, O.MAX):
             assert (got == want).all()
         else:
-            assert O.same_bits_or_both_nan(got, want, O.FLOAT16).all()
+            assert O.same_bits(got, want, O.FLOAT16, [b, a], op, fp16_impl=O.FP16_AVX512FP16).all()
+
+
+@pytest.mark.parametrize("dtype", [O.FLOAT32, O.FLOAT64, O.BFLOAT16, O.FLOAT16])
+def test_nan_results_of_sum_and_prod_follow_the_x86_rules(dtype):
+    """Literal expected patterns (tests/nan_cases.py): a NaN operand comes back quieted, an invalid operation gives
+    the negative default NaN -- for every implementation of the 16-bit types, pairwise and keep-precision, and as
+    the first NaN of a longer chain."""
+    import nan_cases
+    impls = {O.BFLOAT16: [dict(bf16_impl=i) for i in (0, 1, 2)], O.FLOAT16: [dict(fp16_impl=i) for i in (2, 3, 4)]}
+    for op in (O.SUM, O.PROD):
+        a, b, want = nan_cases.table(dtype, op)
+        for kw in impls.get(dtype, [{}]):
+            got = O.comp_reduce(a, b, dtype, op, **kw)
+            assert O.same_bits(got, want, dtype).all(), (op, kw, got, want)
+            # the same pair as the first two inputs of a chain: the NaN travels to the end unchanged
+            one = np.ones_like(a) if dtype in (O.FLOAT32, O.FLOAT64) else np.full_like(a, 0x3F80 if dtype == O.BFLOAT16 else 0x3C00)
+            got3 = O.reduce_n([b, a, one, one], dtype, op, **kw)
+            nan = O.nan_mask(want, dtype)
+            assert O.same_bits(got3[nan], want[nan], dtype).all(), (op, kw)
+            if dtype == O.BFLOAT16:
+                gk = O.reduce_n([b, a, one], dtype, op, keep=1, **kw)
+                assert O.same_bits(gk[nan], want[nan], dtype).all(), (op, kw, "keep")
+
+
+@pytest.mark.parametrize("dtype", [O.FLOAT32, O.FLOAT64, O.BFLOAT16, O.FLOAT16])
+def test_ambiguity_mask_marks_exactly_the_steps_with_two_nan_operands(dtype):
+    """same_bits lets two different NaNs pass only where a chain step had two NaN operands."""
+    import nan_cases
+    sp = nan_cases.specials(dtype)
+    a, b = np.repeat(sp, sp.size), np.tile(sp, sp.size)
+    want = O.comp_reduce(a, b, dtype, O.SUM)
+    other = want.copy()
+    u = other.view({2: np.uint16, 4: np.uint32, 8: np.uint64}[other.dtype.itemsize])
+    nan = O.nan_mask(want, dtype)
+    u[nan] ^= 1                              # another payload for every NaN result
+    ok = O.same_bits(other, want, dtype, [b, a], O.SUM)
+    both = O.nan_mask(a, dtype) & O.nan_mask(b, dtype)
+    assert (ok == (~nan | both)).all()
+    assert both.sum() == 49 and (nan & ~both).sum() > 0
+
