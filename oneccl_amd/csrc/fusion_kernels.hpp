@@ -118,16 +118,13 @@ fusion_reduce_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 const uint32_t i = tid + u * kBlock;
-                if (i < nvec)
-                    st_loose(d + i, nan_checked<TR, OP>(vec_finish<TR>(acc[u]), n_peers + 1, [&](int j) {
-                                 return j == 0 ? s0 + i : (const u32x4_u*)((const unsigned char*)peers.p[j - 1] + poff + head * ES) + i;
-                             }));
+                if (i < nvec) st_loose(d + i, vec_finish<TR>(acc[u]));
             }
             if (tid < head + tail) {
                 const uint32_t i = (tid < head) ? tid : head + nvec * TR::VEC + (tid - head);
                 typename TR::acc_t r = TR::init(ld_elem<E>(a, i));
                 for (int j = 0; j < n_peers; j++)
-                    r = TR::template step_x86<OP>(ld_elem<E>((const unsigned char*)peers.p[j] + poff, i), r);
+                    r = TR::template step<OP>(ld_elem<E>((const unsigned char*)peers.p[j] + poff, i), r);
                 st_elem<E>(o, i, TR::finish(r));
             }
         }
@@ -233,7 +230,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                     typename TR::acc_t r = TR::init(ld_elem<E>(a, i));
 #pragma unroll
                     for (int j = 0; j < NP; j++)
-                        r = TR::template step_x86<OP>(ld_elem<E>((const unsigned char*)peers.p[j] + poff, i), r);
+                        r = TR::template step<OP>(ld_elem<E>((const unsigned char*)peers.p[j] + poff, i), r);
                     st_elem<E>(o, i, TR::finish(r));
                 }
             }

@@ -104,6 +104,10 @@ __device__ __forceinline__ uint32_t f32_minmax_bits(uint32_t in, uint32_t io) {
     return (OP == OP_MIN) ? ((b < a) ? io : in) : ((a < b) ? io : in);
 }
 
+// Sum and prod are the hardware's own add and multiply, NaN results included: gfx950 returns a single NaN operand with
+// its quiet bit set (sign and payload kept) and makes the negative default NaN (0xffc00000, 0xfff8000000000000) from an
+// invalid operation (Inf - Inf, 0 x Inf) -- the same bits as the ADDPS / MULPS family of the reference's CPU path.
+// Only with two NaN operands does the result depend on the operand order, which the reference leaves to its compiler.
 template <int OP, bool VEC_SEM>
 __device__ __forceinline__ uint32_t f32_step_bits(uint32_t in, uint32_t io) {
     if (OP == OP_SUM) return as_u32(as_f32(io) + as_f32(in));
@@ -111,36 +115,8 @@ __device__ __forceinline__ uint32_t f32_step_bits(uint32_t in, uint32_t io) {
     return f32_minmax_bits<OP, VEC_SEM>(in, io);
 }
 
-// NaN results of sum and prod as the x86 instructions of the reference give them (ADDPS / MULPS and their scalar and
-// double forms): one NaN operand comes back with its quiet bit set; no NaN operand (Inf - Inf, 0 x Inf) gives the
-// negative default NaN; with two NaN operands the first source wins, and which operand that is was the reference
-// compiler's choice (`inout` here).  gfx950's own add and multiply make a positive default NaN, so the kernels look
-// at every finished vector and recompute the ones that hold a NaN element by element with step_x86 below.  A NaN,
-// once made, stays one to the end of a sum or product chain, so the finished vector shows every case.
-__device__ __forceinline__ bool f32_is_nan(uint32_t u) { return (u & 0x7fffffffu) > 0x7f800000u; }
-__device__ __forceinline__ uint32_t f32_nan_x86(uint32_t in, uint32_t io) {
-    return f32_is_nan(io) ? (io | 0x00400000u) : f32_is_nan(in) ? (in | 0x00400000u) : 0xffc00000u;
-}
-template <int OP, bool VEC_SEM>
-__device__ __forceinline__ uint32_t f32_step_x86(uint32_t in, uint32_t io) {
-    uint32_t r = f32_step_bits<OP, VEC_SEM>(in, io);
-    if ((OP == OP_SUM || OP == OP_PROD) && f32_is_nan(r)) r = f32_nan_x86(in, io);
-    return r;
-}
-// does a vector of eight 16-bit floats hold a NaN?  A half h is one iff (h & 0x7fff) + BIAS reaches bit 15, with
-// BIAS = 0x7fff - (the pattern of infinity): 0x007f for bf16, 0x03ff for fp16.
-template <uint32_t BIAS>
-__device__ __forceinline__ bool halves_have_nan(u32x4 r) {
-    constexpr uint32_t kBias2 = BIAS | (BIAS << 16);
-    uint32_t t = 0;
-#pragma unroll
-    for (int k = 0; k < 4; k++) t |= (r[k] & 0x7fff7fffu) + kBias2;
-    return (t & 0x80008000u) != 0;
-}
-
 // ---------------------------------------------------------------------------------------------------
-// element traits: elem_t (storage), acc_t (what is carried between steps), init / step / finish; step_x86 is step
-// with the x86 NaN results above (slower, exact for every input); vec_has_nan looks at a finished vector
+// element traits: elem_t (storage), acc_t (what is carried between steps), init / step / finish
 
 // Integers and fp32/fp64 (CCL_REDUCE, comp.cpp:31-58).  Integer sum/prod are done on the unsigned type of
 // the same width (two's-complement wrap).  min/max: ties and unordered operands return `in`.
@@ -158,10 +134,6 @@ struct PlainTraits {
         return (in < io) ? io : in;
     }
     static __device__ __forceinline__ elem_t finish(acc_t a) { return a; }
-    static constexpr bool kFloatArith = false;
-    template <int OP>
-    static __device__ __forceinline__ acc_t step_x86(elem_t in, acc_t io) { return step<OP>(in, io); }
-    static __device__ __forceinline__ bool vec_has_nan(u32x4) { return false; }
 };
 
 // float and double go through their bit patterns for min/max so that no floating-point instruction can
@@ -174,12 +146,6 @@ struct F32Traits {
     template <int OP>
     static __device__ __forceinline__ acc_t step(elem_t in, acc_t io) { return f32_step_bits<OP, false>(in, io); }
     static __device__ __forceinline__ elem_t finish(acc_t a) { return a; }
-    static constexpr bool kFloatArith = true;
-    template <int OP>
-    static __device__ __forceinline__ acc_t step_x86(elem_t in, acc_t io) { return f32_step_x86<OP, false>(in, io); }
-    static __device__ __forceinline__ bool vec_has_nan(u32x4 r) {
-        return f32_is_nan(r[0]) | f32_is_nan(r[1]) | f32_is_nan(r[2]) | f32_is_nan(r[3]);
-    }
 };
 
 struct F64Traits {
@@ -196,19 +162,6 @@ struct F64Traits {
         return (a < b) ? io : in;
     }
     static __device__ __forceinline__ elem_t finish(acc_t a) { return a; }
-    static constexpr bool kFloatArith = true;
-    static __device__ __forceinline__ bool is_nan(uint64_t u) { return (u & 0x7fffffffffffffffull) > 0x7ff0000000000000ull; }
-    template <int OP>
-    static __device__ __forceinline__ acc_t step_x86(elem_t in, acc_t io) {
-        uint64_t r = step<OP>(in, io);
-        if ((OP == OP_SUM || OP == OP_PROD) && is_nan(r))
-            r = is_nan(io) ? (io | 0x0008000000000000ull) : is_nan(in) ? (in | 0x0008000000000000ull) : 0xfff8000000000000ull;
-        return r;
-    }
-    static __device__ __forceinline__ bool vec_has_nan(u32x4 r) {       // on the high dwords; an infinity has a zero low dword
-        return ((r[1] & 0x7fffffffu) > 0x7ff00000u) | ((r[3] & 0x7fffffffu) > 0x7ff00000u) |
-               (((r[1] & 0x7fffffffu) == 0x7ff00000u) & (r[0] != 0)) | (((r[3] & 0x7fffffffu) == 0x7ff00000u) & (r[2] != 0));
-    }
 };
 
 // bfloat16, rounded to bf16 after every pair (ccl_bf16_reduce, src/comp/bf16/bf16.cpp:63-110,
@@ -227,13 +180,6 @@ struct Bf16PairwiseTraits {
         return RNE ? bf16_narrow_rne(r) : bf16_narrow_trunc(r);
     }
     static __device__ __forceinline__ elem_t finish(acc_t a) { return (elem_t)a; }
-    static constexpr bool kFloatArith = true;
-    template <int OP>
-    static __device__ __forceinline__ acc_t step_x86(elem_t in, acc_t io) {
-        uint32_t r = f32_step_x86<OP, VEC_SEM>((uint32_t)in << 16, io << 16);
-        return RNE ? bf16_narrow_rne(r) : bf16_narrow_trunc(r);
-    }
-    static __device__ __forceinline__ bool vec_has_nan(u32x4 r) { return halves_have_nan<0x007fu>(r); }
 };
 
 // bfloat16, widened once, accumulated in fp32 with the plain fp32 step (std:: min/max), narrowed once
@@ -251,12 +197,6 @@ struct Bf16KeepTraits {
     static __device__ __forceinline__ elem_t finish(acc_t a) {
         return (elem_t)(RNE ? bf16_narrow_rne(a) : bf16_narrow_trunc(a));
     }
-    static constexpr bool kFloatArith = true;
-    template <int OP>
-    static __device__ __forceinline__ acc_t step_x86(elem_t in, acc_t io) {
-        return f32_step_x86<OP, false>((uint32_t)in << 16, io);
-    }
-    static __device__ __forceinline__ bool vec_has_nan(u32x4 r) { return halves_have_nan<0x007fu>(r); }
 };
 
 // float16, rounded after every pair through fp32 (ccl_fp16_reduce f16c / avx512f implementations,
@@ -291,18 +231,6 @@ struct Fp16Traits {
         return (rf != rf) ? (r | 0x0200u) : r;
     }
     static __device__ __forceinline__ elem_t finish(acc_t a) { return (elem_t)a; }
-    static constexpr bool kFloatArith = true;
-    // VCVTPH2PS quiets a signalling NaN, the fp32 (or native fp16) operation hands a NaN operand back, VCVTPS2PH
-    // keeps the top of its payload: the operand with its quiet bit set; an invalid operation gives 0xfe00
-    template <int OP>
-    static __device__ __forceinline__ acc_t step_x86(elem_t in, acc_t io) {
-        acc_t r = step<OP>(in, io);
-        if ((OP == OP_SUM || OP == OP_PROD) && is_nan(r))
-            r = is_nan(io) ? (io | 0x0200u) : is_nan(in) ? ((uint32_t)in | 0x0200u) : 0xfe00u;
-        return r;
-    }
-    static __device__ __forceinline__ bool is_nan(uint32_t h) { return (h & 0x7fffu) > 0x7c00u; }
-    static __device__ __forceinline__ bool vec_has_nan(u32x4 r) { return halves_have_nan<0x03ffu>(r); }
 };
 typedef Fp16Traits<false> Fp16PairwiseTraits;
 typedef Fp16Traits<true> Fp16NativeTraits;
@@ -580,37 +508,6 @@ __device__ __forceinline__ void st_elem(void* p, uint64_t i, E x) {
     ((LooseElem<E>*)p)[i].v = x;
 }
 
-// Sum and prod of floating types: a finished vector that holds a NaN is computed again, element by element, with the
-// x86 NaN results (step_x86).  at(j) is the address of this lane's vector in input j; the inputs are read again, which
-// happens before the lane stores the vector anywhere, so an output that is one of the inputs still holds its input.
-template <class TR, int OP>
-struct NanRedo {
-    static constexpr bool value = TR::kFloatArith && (OP == OP_SUM || OP == OP_PROD);
-};
-template <class TR, int OP, class AT>
-__device__ __forceinline__ u32x4 redo_vector_x86(int n, AT&& at) {
-    Lanes<TR> l = __builtin_bit_cast(Lanes<TR>, ld_loose(at(0)));
-    typename TR::acc_t a[TR::VEC];
-#pragma unroll
-    for (int k = 0; k < TR::VEC; k++) a[k] = TR::init(l.v[k]);
-#pragma unroll
-    for (int j = 1; j < n; j++) {
-        l = __builtin_bit_cast(Lanes<TR>, ld_loose(at(j)));
-#pragma unroll
-        for (int k = 0; k < TR::VEC; k++) a[k] = TR::template step_x86<OP>(l.v[k], a[k]);
-    }
-#pragma unroll
-    for (int k = 0; k < TR::VEC; k++) l.v[k] = TR::finish(a[k]);
-    return __builtin_bit_cast(u32x4, l);
-}
-template <class TR, int OP, class AT>
-__device__ __forceinline__ u32x4 nan_checked(u32x4 r, int n, AT&& at) {
-    if constexpr (NanRedo<TR, OP>::value) {
-        if (__builtin_expect(TR::vec_has_nan(r), 0)) r = redo_vector_x86<TR, OP>(n, at);
-    }
-    return r;
-}
-
 // The count % VEC elements after the last full vector and the elements before the first aligned one:
 // at most 2*(VEC-1) <= 30 elements, one per lane of the first wave of block 0.
 template <class TR, int OP, class SRC>
@@ -621,7 +518,7 @@ __device__ __forceinline__ void reduce_edges(const SRC& src, int n, void* dst, u
     if (t < head + tail) {
         uint64_t i = (t < head) ? t : (uint64_t)head + nvec * TR::VEC + (t - head);
         typename TR::acc_t a = TR::init(ld_elem<E>(src.p[0], i));
-        for (int j = 1; j < n; j++) a = TR::template step_x86<OP>(ld_elem<E>(src.p[j], i), a);
+        for (int j = 1; j < n; j++) a = TR::template step<OP>(ld_elem<E>(src.p[j], i), a);
         st_elem<E>(dst, i, TR::finish(a));
     }
 }
@@ -672,8 +569,7 @@ reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint
                 Accs<TR> a = vec_init<TR>(x[0][u]);
 #pragma unroll
                 for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j][u], a);
-                const uint64_t i = base + (uint64_t)u * kBlock;
-                st_loose(d + i, nan_checked<TR, OP>(vec_finish<TR>(a), N, [&](int j) { return s[j] + i; }));
+                st_loose(d + base + (uint64_t)u * kBlock, vec_finish<TR>(a));
             }
         }
         else {
@@ -687,7 +583,7 @@ reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint
                     Accs<TR> a = vec_init<TR>(x[0]);
 #pragma unroll
                     for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j], a);
-                    st_loose(d + i, nan_checked<TR, OP>(vec_finish<TR>(a), N, [&](int j) { return s[j] + i; }));
+                    st_loose(d + i, vec_finish<TR>(a));
                 }
             }
         }
@@ -770,9 +666,6 @@ __device__ __forceinline__ void reduce_group(const u32x4_u* const (&s)[N], const
         for (int j = 1; j < N; j++) vec_step<TR, OP>(x[g][j], a);
         out[g] = vec_finish<TR>(a);
     }
-    // after the last use of the loaded vectors, so that the rare path costs no registers while they are held
-#pragma unroll
-    for (int g = 0; g < G; g++) out[g] = nan_checked<TR, OP>(out[g], N, [&](int j) { return s[j] + idx[g]; });
 }
 
 // the same for a group that may reach past the end of the buffer: slots at or beyond nvec are left alone
@@ -819,19 +712,6 @@ __device__ __forceinline__ void reduce_rt_tile(const SrcTable& src, int n, uint3
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) out[u] = vec_finish<TR>(a[u]);
-    if constexpr (NanRedo<TR, OP>::value) {
-        bool any = false;
-#pragma unroll
-        for (int u = 0; u < UNROLL; u++) any |= TR::vec_has_nan(out[u]);
-        if (__builtin_expect(any, 0)) {
-#pragma unroll
-            for (int u = 0; u < UNROLL; u++)
-                if (idx[u] < nvec && TR::vec_has_nan(out[u]))
-                    out[u] = redo_vector_x86<TR, OP>(n, [&](int j) {
-                        return (const u32x4_u*)((const unsigned char*)src.p[j] + head * sizeof(E)) + idx[u];
-                    });
-        }
-    }
 }
 
 template <class TR, int OP>
@@ -842,7 +722,7 @@ __device__ __forceinline__ void reduce_multi_edges(const SrcTable& src, int n, c
     if (t < head + tail) {
         uint64_t i = (t < head) ? t : (uint64_t)head + nvec * TR::VEC + (t - head);
         typename TR::acc_t a = TR::init(ld_elem<E>(src.p[0], i));
-        for (int j = 1; j < n; j++) a = TR::template step_x86<OP>(ld_elem<E>(src.p[j], i), a);
+        for (int j = 1; j < n; j++) a = TR::template step<OP>(ld_elem<E>(src.p[j], i), a);
         const E r = TR::finish(a);
         for (int k = 0; k < m; k++) st_elem<E>(dst.p[k], i, r);
     }

@@ -375,16 +375,18 @@ def test_arguments_and_errors(comp):
     assert [comp.reduction_to_str(i) for i in range(6)] == ["sum", "prod", "min", "max", "custom", "unknown"]
     assert comp.kernel_name("reduce_monolithic_kernel_7", O.BFLOAT16, O.SUM) == "reduce_monolithic_kernel_7_bfloat16_sum"
     # count 0 succeeds without touching pointers (comp.cpp:132-134), even with a bad dtype
-    assert L.mi_ccl_comp_reduce(99, 0, None, 0, None, 2, None) == 0
+    assert L.mi_ccl_comp_reduce(99, 0, None, 0, None, 2, 0, None) == 0
     x = torch.zeros(64, dtype=torch.int32, device="cuda")
-    assert L.mi_ccl_comp_reduce(99, 0, x.data_ptr(), 4, x.data_ptr(), 2, None) == comp.INVALID_ARGUMENTS
-    assert L.mi_ccl_comp_reduce(O.INT32, 4, x.data_ptr(), 4, x.data_ptr(), 2, None) == comp.INVALID_ARGUMENTS  # custom
-    assert L.mi_ccl_comp_reduce(O.INT32, 0, None, 4, x.data_ptr(), 2, None) == comp.INVALID_ARGUMENTS
-    assert L.mi_ccl_comp_reduce(O.INT32, 0, x.data_ptr() + 2, 4, x.data_ptr(), 2, None) == comp.INVALID_ARGUMENTS
+    assert L.mi_ccl_comp_reduce(99, 0, x.data_ptr(), 4, x.data_ptr(), 2, 0, None) == comp.INVALID_ARGUMENTS
+    assert L.mi_ccl_comp_reduce(O.INT32, 4, x.data_ptr(), 4, x.data_ptr(), 2, 0, None) == comp.INVALID_ARGUMENTS  # custom
+    assert L.mi_ccl_comp_reduce(O.INT32, 0, None, 4, x.data_ptr(), 2, 0, None) == comp.INVALID_ARGUMENTS
+    assert L.mi_ccl_comp_reduce(O.INT32, 0, x.data_ptr() + 2, 4, x.data_ptr(), 2, 0, None) == comp.INVALID_ARGUMENTS
     with pytest.raises(comp.CclError):
         comp.comp_reduce_n(O.FLOAT32, O.SUM, [x], x, 4, lp_mode=comp.LP_KEEP_PRECISION)   # keep needs bfloat16
     with pytest.raises(comp.CclError):
         comp.comp_reduce_n(O.INT32, O.SUM, [x] * 65, x, 4)
+    for bad in (1, 5, -1):          # fp16_impl: 0 (the default), 2, 3 or 4
+        assert L.mi_ccl_comp_reduce(O.FLOAT16, 0, x.data_ptr(), 4, x.data_ptr(), 2, bad, None) == comp.INVALID_ARGUMENTS
     torch.cuda.synchronize()
     assert (x == 0).all()
 
