@@ -183,6 +183,23 @@ int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* ow
                          const void* const* peers, int n_peers, void* const* out_tensors, int lp_mode,
                          int bf16_impl, int fp16_impl, void* stream);
 
+/* The same fused reduce for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): no plan, and no hipMalloc, hipFree or other allocating call -- the work
+ * table that a plan keeps in memory of its own lives in an array inside the library (about 1 MiB per GPU, held until
+ * the process ends) and is rewritten by a small kernel on `stream` in front of the reduce of every call.  The layout
+ * is given directly: counts[k] elements of `dtype`, starts rounded up to `align` bytes (as mi_ccl_fusion_offsets).
+ * Same results as mi_ccl_fusion_reduce on a plan of the same layout.  Limits: k <= MI_CCL_FUSION_STATIC_MAX_TENSORS and
+ * at most MI_CCL_FUSION_STATIC_MAX_ITEMS pieces of 16 KiB (a tensor takes ceil(bytes / 16384) of them: 2 GiB of payload
+ * when the tensors are multiples of 16 KiB); beyond either the call returns out_of_resource and does nothing.  All
+ * calls on one GPU share the one table: calls on the same stream are ordered, calls that overlap on different
+ * streams of one GPU race (results undefined).  The first call on a GPU looks the array's address up; make that call
+ * outside a capture.  This entry point has no counterpart in the reference. */
+#define MI_CCL_FUSION_STATIC_MAX_TENSORS 1024
+#define MI_CCL_FUSION_STATIC_MAX_ITEMS 131072
+int mi_ccl_fusion_reduce_static(const size_t* counts, size_t k, int dtype, size_t align, int op,
+                                const void* const* own_tensors, const void* const* peers, int n_peers,
+                                void* const* out_tensors, int lp_mode, int bf16_impl, int fp16_impl, void* stream);
+
 /* ---- launch tuning ------------------------------------------------------------------------------- */
 
 /* Launch-shape knobs, the counterpart of CCL_KERNEL_GROUP_SIZE / CCL_KERNEL_MEM_ALIGN

@@ -31,6 +31,7 @@ EXPORTS = [
     "mi_ccl_convert_fp32_to_fp16_arrays", "mi_ccl_convert_fp16_to_fp32_arrays", "mi_ccl_fusion_offsets",
     "mi_ccl_fusion_plan_create", "mi_ccl_fusion_plan_destroy", "mi_ccl_fusion_plan_bytes",
     "mi_ccl_fusion_plan_offset", "mi_ccl_fusion_pack", "mi_ccl_fusion_unpack", "mi_ccl_fusion_reduce",
+    "mi_ccl_fusion_reduce_static",
     "mi_ccl_set_param", "mi_ccl_get_param",
 ]
 
@@ -81,6 +82,7 @@ def lib():
     L.mi_ccl_fusion_pack.argtypes = [vp, vp, vp, vp]
     L.mi_ccl_fusion_unpack.argtypes = [vp, vp, vp, vp]
     L.mi_ccl_fusion_reduce.argtypes = [vp, i, vp, vp, i, vp, i, i, i, vp]
+    L.mi_ccl_fusion_reduce_static.argtypes = [vp, sz, i, sz, i, vp, vp, i, vp, i, i, i, vp]
     L.mi_ccl_set_param.argtypes = [C.c_char_p, C.c_long]
     L.mi_ccl_get_param.restype = C.c_long
     L.mi_ccl_get_param.argtypes = [C.c_char_p]
@@ -257,6 +259,19 @@ class FusionPlan:
             self.close()
         except Exception:
             pass
+
+
+FUSION_STATIC_MAX_TENSORS, FUSION_STATIC_MAX_ITEMS = 1024, 131072
+
+
+def fusion_reduce_static(counts, dtype, align, op, own_tensors, peers, out_tensors, lp_mode=LP_PAIRWISE,
+                         bf16_impl=BF16_AVX512BF, fp16_impl=FP16_DEFAULT, stream=None):
+    """FusionPlan.reduce without a plan and without any allocation (mi_ccl_fusion_reduce_static)."""
+    k = len(counts)
+    cnt = (C.c_size_t * k)(*[int(c) for c in counts])
+    _check(lib().mi_ccl_fusion_reduce_static(cnt, k, dtype, align, op, _ptr_array(own_tensors), _ptr_array(peers),
+                                             len(peers), _ptr_array(out_tensors), lp_mode, bf16_impl, fp16_impl,
+                                             _stream(stream)), "mi_ccl_fusion_reduce_static")
 
 
 def set_param(name, value):

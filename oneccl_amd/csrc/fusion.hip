@@ -96,6 +96,66 @@ static hipError_t dispatch_fusion(int dtype, bool keep, int bf16_impl, const Fus
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// The fused reduce for callers that cannot allocate: its work table (the per-tensor offset and size tables and the
+// item list that a plan keeps in memory of its own) lives in a file-scope device array and is written by a small
+// kernel on the caller's stream in front of the reduce kernels.  Every GPU holds its own copy of the array at its own
+// address, looked up once per device with that device current; host code only ever uses that looked-up address.
+
+struct StaticFusionTable {
+    uint64_t off[MI_CCL_FUSION_STATIC_MAX_TENSORS];
+    uint64_t bytes[MI_CCL_FUSION_STATIC_MAX_TENSORS];
+    FusionItem items[MI_CCL_FUSION_STATIC_MAX_ITEMS];
+};
+static __device__ __align__(256) unsigned char scratch[sizeof(StaticFusionTable)];
+static std::atomic<StaticFusionTable*> g_scratch_ptr[64];
+
+static hipError_t scratch_table(StaticFusionTable** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return e;
+    if (dev < 0 || dev >= 64)
+        return hipErrorInvalidDevice;
+    StaticFusionTable* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess)
+            return e;
+        p = (StaticFusionTable*)ptr;
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return hipSuccess;
+}
+
+struct FusionSizes {                // by-value kernel argument: the sizes of one launch group of tensors, in bytes
+    uint64_t bytes[kFusionGroup];
+};
+
+// Block b writes the table rows of tensor t0 + b: its byte offset in the fusion buffer (running end rounded up to
+// `align`, from `end0`, the end of the tensor before the group), its size, and its work items from item index
+// `item0` + (items of the group's tensors before it).  Every lane walks the (at most kFusionGroup) sizes before its
+// tensor; they are kernel arguments, so the walk is scalar work.
+__global__ void __launch_bounds__(kBlock)
+fusion_table_kernel(FusionSizes sz, uint32_t t0, uint64_t end0, uint64_t align, uint64_t item0, StaticFusionTable* tab) {
+    const uint32_t b = blockIdx.x;
+    uint64_t end = end0, item = item0;
+    for (uint32_t u = 0; u < b; u++) {
+        end = ((end + align - 1) & ~(align - 1)) + sz.bytes[u];
+        item += (sz.bytes[u] + kFusionChunk - 1) / kFusionChunk;
+    }
+    const uint64_t off = (end + align - 1) & ~(align - 1);
+    const uint64_t nb = sz.bytes[b];
+    if (threadIdx.x == 0) {
+        tab->off[t0 + b] = off;
+        tab->bytes[t0 + b] = nb;
+    }
+    const uint64_t chunks = (nb + kFusionChunk - 1) / kFusionChunk;
+    for (uint64_t c = threadIdx.x; c < chunks; c += kBlock) tab->items[item + c] = FusionItem{ t0 + b, (uint32_t)c };
+}
+
 }  // namespace mi
 
 using namespace mi;
@@ -279,6 +339,79 @@ int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* ow
     if (fp16_impl != MI_CCL_FP16_DEFAULT)
         a.tune.fp16_impl = fp16_impl;
     return fusion_status_of(dispatch_fusion(plan->dtype, keep, bf16_impl, a));
+}
+
+int mi_ccl_fusion_reduce_static(const size_t* counts, size_t k, int dtype, size_t align, int op,
+                                const void* const* own_tensors, const void* const* peers, int n_peers,
+                                void* const* out_tensors, int lp_mode, int bf16_impl, int fp16_impl, void* stream) {
+    const size_t esz = fusion_dtype_size(dtype);
+    if (esz == 0 || k == 0 || !counts || align == 0 || (align & (align - 1)) != 0)
+        return MI_CCL_INVALID_ARGUMENTS;
+    if (!own_tensors || !out_tensors || n_peers < 0 || n_peers > kFusionMaxPeers || (n_peers && !peers))
+        return MI_CCL_INVALID_ARGUMENTS;
+    if (op < MI_CCL_SUM || op > MI_CCL_MAX || bf16_impl < MI_CCL_BF16_SCALAR || bf16_impl > MI_CCL_BF16_AVX512BF)
+        return MI_CCL_INVALID_ARGUMENTS;
+    if (fp16_impl != MI_CCL_FP16_DEFAULT && (fp16_impl < MI_CCL_FP16_F16C || fp16_impl > MI_CCL_FP16_AVX512FP16))
+        return MI_CCL_INVALID_ARGUMENTS;
+    const bool keep = (lp_mode & MI_CCL_LP_KEEP_PRECISION) != 0;
+    if ((lp_mode & ~MI_CCL_LP_KEEP_PRECISION) != 0 || (keep && dtype != MI_CCL_BFLOAT16))
+        return MI_CCL_INVALID_ARGUMENTS;
+    if (k > MI_CCL_FUSION_STATIC_MAX_TENSORS)
+        return MI_CCL_OUT_OF_RESOURCE;          // more tensors than the table holds
+    uint64_t item_begin[MI_CCL_FUSION_STATIC_MAX_TENSORS + 1];      // on the stack: nothing is allocated here
+    uint64_t items = 0;
+    for (size_t t = 0; t < k; t++) {
+        item_begin[t] = items;
+        if (counts[t] > ((uint64_t)1 << 40) / esz)
+            return MI_CCL_OUT_OF_RESOURCE;
+        items += ((uint64_t)counts[t] * esz + kFusionChunk - 1) / kFusionChunk;
+        if (items > MI_CCL_FUSION_STATIC_MAX_ITEMS)
+            return MI_CCL_OUT_OF_RESOURCE;      // more payload than the item list holds
+        if (counts[t] == 0)
+            continue;
+        if (!own_tensors[t] || !out_tensors[t] || ((uintptr_t)own_tensors[t] % esz) || ((uintptr_t)out_tensors[t] % esz))
+            return MI_CCL_INVALID_ARGUMENTS;
+    }
+    item_begin[k] = items;
+    for (int j = 0; j < n_peers; j++)
+        if (!peers[j] || ((uintptr_t)peers[j] % esz))
+            return MI_CCL_INVALID_ARGUMENTS;
+    if (items == 0)
+        return MI_CCL_SUCCESS;
+
+    StaticFusionTable* tab = nullptr;
+    hipError_t e = scratch_table(&tab);
+    if (e != hipSuccess)
+        return fusion_status_of(e);
+    // the table first: one small launch per group of kFusionGroup tensors, in stream order before the reduce
+    uint64_t end = 0;
+    for (size_t t0 = 0; t0 < k; t0 += kFusionGroup) {
+        const size_t t1 = (t0 + kFusionGroup < k) ? t0 + kFusionGroup : k;
+        FusionSizes sz;
+        for (size_t t = t0; t < t1; t++) sz.bytes[t - t0] = (uint64_t)counts[t] * esz;
+        hipLaunchKernelGGL(fusion_table_kernel, dim3((unsigned)(t1 - t0)), dim3(kBlock), 0, (hipStream_t)stream, sz,
+                           (uint32_t)t0, end, (uint64_t)align, item_begin[t0], tab);
+        e = hipGetLastError();
+        if (e != hipSuccess)
+            return fusion_status_of(e);
+        for (size_t t = t0; t < t1; t++) end = ((end + align - 1) & ~((uint64_t)align - 1)) + sz.bytes[t - t0];
+    }
+    FusionLaunchArgs a;
+    a.own = own_tensors;
+    a.out = out_tensors;
+    a.peers = peers;
+    a.n_peers = n_peers;
+    a.op = op;
+    a.k = k;
+    a.d_off = tab->off;             // address arithmetic on the looked-up device address, no host access
+    a.d_bytes = tab->bytes;
+    a.d_items = tab->items;
+    a.item_begin = item_begin;
+    a.stream = (hipStream_t)stream;
+    a.tune = current_tuning();
+    if (fp16_impl != MI_CCL_FP16_DEFAULT)
+        a.tune.fp16_impl = fp16_impl;
+    return fusion_status_of(dispatch_fusion(dtype, keep, bf16_impl, a));
 }
 
 } /* extern "C" */

@@ -51,6 +51,14 @@ def test_host_only_entry_points():
     L = c.lib()
     assert L.mi_ccl_comp_reduce(0, 0, None, 0, None, 2, 0, None) == 0
     assert L.mi_ccl_comp_copy(None, None, 0, 0, None) == 0
+    # the entry point that allocates nothing refuses what its table cannot hold before it touches the GPU
+    k = c.FUSION_STATIC_MAX_TENSORS + 1
+    cnt = (ctypes.c_size_t * k)(*([1] * k))
+    ptrs = (ctypes.c_void_p * k)(*([16] * k))
+    assert L.mi_ccl_fusion_reduce_static(cnt, k, c.FLOAT32, 4, c.SUM, ptrs, None, 0, ptrs, 0, 2, 0, None) == c.OUT_OF_RESOURCE
+    one = (ctypes.c_size_t * 1)((c.FUSION_STATIC_MAX_ITEMS + 1) * 4096)
+    assert L.mi_ccl_fusion_reduce_static(one, 1, c.FLOAT32, 4, c.SUM, ptrs, None, 0, ptrs, 0, 2, 0, None) == c.OUT_OF_RESOURCE
+    assert L.mi_ccl_fusion_reduce_static(one, 1, c.FLOAT32, 4, c.SUM, ptrs, None, 0, ptrs, 0, 2, 7, None) == c.INVALID_ARGUMENTS
 
 
 def test_missing_library_fails_loudly(monkeypatch):
