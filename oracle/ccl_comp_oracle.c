@@ -30,8 +30,11 @@
  *   orc_fusion_*                    pack/unpack round trip, offsets closed form
  *   orc_reduce_write_n              composition of orc_reduce_n (pinned above) and memcpy: every destination equals
  *                                   orc_reduce_n's output; closed forms of the reference's functional tests
- * NaN payload and sign of NaN *results* are not pinned by the reference itself (operand order of a
- * commutative SSE/AVX add is the compiler's choice); tests compare NaN-ness only.
+ *   NaN results of sum/prod         the host's own SSE/AVX add and multiply, as in the reference: a NaN operand comes
+ *                                   back quieted, an invalid operation gives the negative default NaN -- literal patterns
+ *                                   in tests/nan_cases.py, golden special-value pairs made by oracle/_ref.  Only a step
+ *                                   with TWO NaN operands is not pinned (which one comes back follows the operand order
+ *                                   the compiler chose, here as in the reference); tests compare those as NaN == NaN.
  */
 #define _GNU_SOURCE
 #include "ccl_comp_oracle.h"
