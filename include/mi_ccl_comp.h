@@ -121,6 +121,20 @@ int mi_ccl_comp_reduce_n(int dtype, int op, const void* const* srcs, int n, void
 int mi_ccl_comp_reduce_write_n(int dtype, int op, const void* const* srcs, int n, void* const* dsts, int m,
                                size_t count, int lp_mode, int bf16_impl, int fp16_impl, void* stream);
 
+/* n_jobs independent reduces of one dtype and operation in ONE launch: for job j and i < counts[j],
+ * dsts[j][i] = srcs[j * n + 0][i] OP srcs[j * n + 1][i] OP ... OP srcs[j * n + n - 1][i] (1 <= n <= 8, the same for every
+ * job).  srcs (n_jobs x n pointers, job after job), dsts and counts are HOST arrays; a job's output may be one of its
+ * own inputs, the jobs must not overlap one another; a job with count 0 is skipped without looking at its pointers.
+ * The job table travels in the kernel arguments (96 jobs or 288 pointers per launch, more jobs take more launches):
+ * nothing is allocated.  Replaces read_reduce_write (n = 2: even[i] = pair[i] + local[i] for every peer i in one kernel,
+ * src/coll/algorithms/reduce_scatter/sycl/reduce_scatter_large_sycl_impl.hpp:22-66), reduce_read_write_kernel_{1..7}
+ * (src/kernels/kernels.cl:156-177) and, with n = 1, copy_data (N copies in one kernel, used at :216-224 of the same
+ * file); it is also the small-message path: 64 reduces of a few KiB cost one launch, not 64.  lp_mode:
+ * MI_CCL_LP_PAIRWISE or MI_CCL_LP_KEEP_PRECISION (bfloat16). */
+int mi_ccl_comp_reduce_batch(int dtype, int op, const void* const* srcs, int n, void* const* dsts,
+                             const size_t* counts, int n_jobs, int lp_mode, int bf16_impl, int fp16_impl,
+                             void* stream);
+
 /* Slice form of the same: slice i starts at in_buf + offsets[i] elements (offsets: HOST array); inout is
  * slice 0 and receives the result.  Replaces ccl_comp_batch_reduce (src/comp/comp.cpp:202-249); the tmp and
  * acc scratch arrays of the reference are not needed.  keep_precision != 0 requires dtype bfloat16 and

@@ -26,7 +26,8 @@ DTYPE_SIZE = [1, 1, 2, 2, 4, 4, 8, 8, 2, 4, 8, 2]
 EXPORTS = [
     "mi_ccl_datatype_size", "mi_ccl_datatype_name", "mi_ccl_reduction_to_str", "mi_ccl_status_str",
     "mi_ccl_kernel_name", "mi_ccl_comp_reduce", "mi_ccl_bf16_reduce", "mi_ccl_fp16_reduce",
-    "mi_ccl_comp_reduce_n", "mi_ccl_comp_reduce_write_n", "mi_ccl_comp_batch_reduce", "mi_ccl_comp_copy",
+    "mi_ccl_comp_reduce_n", "mi_ccl_comp_reduce_write_n", "mi_ccl_comp_reduce_batch", "mi_ccl_comp_batch_reduce",
+    "mi_ccl_comp_copy",
     "mi_ccl_convert_fp32_to_bf16_arrays", "mi_ccl_convert_bf16_to_fp32_arrays",
     "mi_ccl_convert_fp32_to_fp16_arrays", "mi_ccl_convert_fp16_to_fp32_arrays", "mi_ccl_fusion_offsets",
     "mi_ccl_fusion_plan_create", "mi_ccl_fusion_plan_destroy", "mi_ccl_fusion_plan_bytes",
@@ -66,6 +67,7 @@ def lib():
     L.mi_ccl_fp16_reduce.argtypes = [vp, sz, vp, i, i, vp]
     L.mi_ccl_comp_reduce_n.argtypes = [i, i, vp, i, vp, sz, i, i, i, vp]
     L.mi_ccl_comp_reduce_write_n.argtypes = [i, i, vp, i, vp, i, sz, i, i, i, vp]
+    L.mi_ccl_comp_reduce_batch.argtypes = [i, i, vp, i, vp, vp, i, i, i, i, vp]
     L.mi_ccl_comp_batch_reduce.argtypes = [vp, vp, sz, sz, vp, i, i, i, i, i, vp]
     L.mi_ccl_comp_copy.argtypes = [vp, vp, sz, i, vp]
     L.mi_ccl_convert_fp32_to_bf16_arrays.argtypes = [vp, vp, sz, i, vp]
@@ -168,6 +170,20 @@ def comp_reduce_write_n(dtype, op, srcs, dsts, count, lp_mode=LP_PAIRWISE, bf16_
     s, d = _ptr_array(srcs), _ptr_array(dsts)
     _check(lib().mi_ccl_comp_reduce_write_n(dtype, op, s, len(srcs), d, len(dsts), count, lp_mode, bf16_impl,
                                             fp16_impl, _stream(stream)), "mi_ccl_comp_reduce_write_n")
+
+
+def comp_reduce_batch(dtype, op, jobs, lp_mode=LP_PAIRWISE, bf16_impl=BF16_AVX512BF, fp16_impl=FP16_DEFAULT, stream=None):
+    """Many independent reduces in one launch.  jobs: list of (srcs, dst, count), every job with the same number of
+    inputs; dst = srcs[0] OP srcs[1] OP ... over count elements."""
+    if not jobs:
+        return
+    n = len(jobs[0][0])
+    assert all(len(j[0]) == n for j in jobs), "every job takes the same number of inputs"
+    srcs = _ptr_array([s for j in jobs for s in j[0]])
+    dsts = _ptr_array([j[1] for j in jobs])
+    counts = (C.c_size_t * len(jobs))(*[int(j[2]) for j in jobs])
+    _check(lib().mi_ccl_comp_reduce_batch(dtype, op, srcs, n, dsts, counts, len(jobs), lp_mode, bf16_impl, fp16_impl,
+                                          _stream(stream)), "mi_ccl_comp_reduce_batch")
 
 
 def comp_batch_reduce(in_buf, offsets, count, inout, dtype, op, keep_precision, bf16_impl=BF16_AVX512BF,

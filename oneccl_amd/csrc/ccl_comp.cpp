@@ -327,3 +327,19 @@ ccl::status ccl_comp_reduce_write_n(ccl_sched* sched, const void* own_buf, const
                                                 bf16_impl(), fp16_impl_or_default(), stream_of(sched)),
                      "ccl_comp_reduce_write_n");
 }
+
+ccl::status ccl_comp_reduce_batch(ccl_sched* sched, const std::vector<const void*>& srcs, int n_inputs,
+                                  const std::vector<void*>& dsts, const std::vector<size_t>& counts,
+                                  const ccl_datatype& dtype, ccl::reduction reduction, int bf16_keep_precision_mode) {
+    if (dsts.empty())
+        return ccl::status::success;
+    if (reduction == ccl::reduction::custom)
+        fail("custom reduction is not available for the batched device reduce");
+    if (n_inputs < 1 || counts.size() != dsts.size() || srcs.size() != dsts.size() * (size_t)n_inputs)
+        fail("ccl_comp_reduce_batch: srcs must hold n_inputs pointers per job, dsts and counts one entry per job");
+    int lp = bf16_keep_precision_mode ? MI_CCL_LP_KEEP_PRECISION : MI_CCL_LP_PAIRWISE;
+    return to_status(mi_ccl_comp_reduce_batch((int)dtype.idx(), (int)reduction, srcs.data(), n_inputs, dsts.data(),
+                                              counts.data(), (int)dsts.size(), lp, bf16_impl(), fp16_impl_or_default(),
+                                              stream_of(sched)),
+                     "ccl_comp_reduce_batch");
+}

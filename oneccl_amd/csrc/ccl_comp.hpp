@@ -210,3 +210,11 @@ ccl::status ccl_comp_reduce_n(ccl_sched* sched, const void* own_buf, const std::
 ccl::status ccl_comp_reduce_write_n(ccl_sched* sched, const void* own_buf, const std::vector<const void*>& peer_bufs,
                                     size_t count, const std::vector<void*>& out_bufs, const ccl_datatype& dtype,
                                     ccl::reduction reduction, int bf16_keep_precision_mode = 0);
+
+// Many independent reduces in ONE launch -- the reference's read_reduce_write (even[i] = pair[i] + local[i] for every
+// peer i, src/coll/algorithms/reduce_scatter/sycl/reduce_scatter_large_sycl_impl.hpp:22-66), reduce_read_write_kernel_N
+// (src/kernels/kernels.cl:156-177) and, with one input per job, copy_data.  Job j: dsts[j] = srcs[j * n_inputs] OP ... OP
+// srcs[j * n_inputs + n_inputs - 1] over counts[j] elements.
+ccl::status ccl_comp_reduce_batch(ccl_sched* sched, const std::vector<const void*>& srcs, int n_inputs,
+                                  const std::vector<void*>& dsts, const std::vector<size_t>& counts,
+                                  const ccl_datatype& dtype, ccl::reduction reduction, int bf16_keep_precision_mode = 0);

@@ -9,12 +9,15 @@
 #include <cctype>
 
 #include "../../include/mi_ccl_comp.h"
+#include "batch_kernels.hpp"
 #include "launch_geometry.hpp"
 #include "reduce_kernels.hpp"
 
 namespace mi {
 
-#define MI_DECLARE(TR) extern template hipError_t launch_reduce<TR>(const LaunchArgs&)
+#define MI_DECLARE(TR)                                                   \
+    extern template hipError_t launch_reduce<TR>(const LaunchArgs&);     \
+    extern template hipError_t launch_reduce_batch<TR>(const BatchLaunchArgs&)
 MI_DECLARE(I8Traits);
 MI_DECLARE(U8Traits);
 MI_DECLARE(I16Traits);
@@ -141,6 +144,35 @@ static hipError_t dispatch(int dtype, bool keep, int bf16_impl, const LaunchArgs
             if (bf16_impl == MI_CCL_BF16_AVX512F)
                 return launch_reduce<Bf16PairAvx512f>(a);
             return launch_reduce<Bf16PairAvx512bf>(a);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+// The same choice for a launch of many independent jobs.
+static hipError_t dispatch_batch(int dtype, bool keep, int bf16_impl, const BatchLaunchArgs& a) {
+    switch (dtype) {
+        case MI_CCL_INT8: return launch_reduce_batch<I8Traits>(a);
+        case MI_CCL_UINT8: return launch_reduce_batch<U8Traits>(a);
+        case MI_CCL_INT16: return launch_reduce_batch<I16Traits>(a);
+        case MI_CCL_UINT16: return launch_reduce_batch<U16Traits>(a);
+        case MI_CCL_INT32: return launch_reduce_batch<I32Traits>(a);
+        case MI_CCL_UINT32: return launch_reduce_batch<U32Traits>(a);
+        case MI_CCL_INT64: return launch_reduce_batch<I64Traits>(a);
+        case MI_CCL_UINT64: return launch_reduce_batch<U64Traits>(a);
+        case MI_CCL_FLOAT16:
+            return a.tune.fp16_impl == MI_CCL_FP16_AVX512FP16 ? launch_reduce_batch<Fp16NativeTraits>(a)
+                                                              : launch_reduce_batch<Fp16PairwiseTraits>(a);
+        case MI_CCL_FLOAT32: return launch_reduce_batch<F32Traits>(a);
+        case MI_CCL_FLOAT64: return launch_reduce_batch<F64Traits>(a);
+        case MI_CCL_BFLOAT16:
+            if (keep)
+                return (bf16_impl == MI_CCL_BF16_AVX512BF) ? launch_reduce_batch<Bf16KeepTraits<true>>(a)
+                                                            : launch_reduce_batch<Bf16KeepTraits<false>>(a);
+            if (bf16_impl == MI_CCL_BF16_SCALAR)
+                return launch_reduce_batch<Bf16PairScalar>(a);
+            if (bf16_impl == MI_CCL_BF16_AVX512F)
+                return launch_reduce_batch<Bf16PairAvx512f>(a);
+            return launch_reduce_batch<Bf16PairAvx512bf>(a);
         default: return hipErrorInvalidValue;
     }
 }
@@ -477,6 +509,43 @@ int mi_ccl_comp_reduce_n(int dtype, int op, const void* const* srcs, int n, void
 int mi_ccl_comp_reduce_write_n(int dtype, int op, const void* const* srcs, int n, void* const* dsts, int m, size_t count,
                                int lp_mode, int bf16_impl, int fp16_impl, void* stream) {
     return reduce_n_impl(dtype, op, srcs, n, dsts, m, count, lp_mode, bf16_impl, fp16_impl, stream);
+}
+
+int mi_ccl_comp_reduce_batch(int dtype, int op, const void* const* srcs, int n, void* const* dsts, const size_t* counts,
+                             int n_jobs, int lp_mode, int bf16_impl, int fp16_impl, void* stream) {
+    if (n_jobs == 0)
+        return MI_CCL_SUCCESS;
+    if (n_jobs < 0 || !srcs || !dsts || !counts || n < 1 || n > kMaxFixedN)
+        return MI_CCL_INVALID_ARGUMENTS;
+    if (dtype < 0 || dtype >= MI_CCL_DATATYPE_LAST || op < MI_CCL_SUM || op > MI_CCL_MAX)
+        return MI_CCL_INVALID_ARGUMENTS;
+    if (bf16_impl < MI_CCL_BF16_SCALAR || bf16_impl > MI_CCL_BF16_AVX512BF || !fp16_impl_ok(fp16_impl))
+        return MI_CCL_INVALID_ARGUMENTS;
+    const bool keep = (lp_mode & MI_CCL_LP_KEEP_PRECISION) != 0;
+    if ((lp_mode & ~MI_CCL_LP_KEEP_PRECISION) != 0 || (keep && dtype != MI_CCL_BFLOAT16))
+        return MI_CCL_INVALID_ARGUMENTS;        // the truncated tail (MI_CCL_LP_TAIL_QUIRK) belongs to ccl_comp_batch_reduce
+    const size_t esz = kDtypeSize[dtype];
+    for (int j = 0; j < n_jobs; j++) {
+        if (counts[j] == 0)
+            continue;                           // an empty job's pointers are not looked at
+        if (!dsts[j] || ((uintptr_t)dsts[j] % esz) != 0)
+            return MI_CCL_INVALID_ARGUMENTS;
+        for (int k = 0; k < n; k++)
+            if (!srcs[(size_t)j * n + k] || ((uintptr_t)srcs[(size_t)j * n + k] % esz) != 0)
+                return MI_CCL_INVALID_ARGUMENTS;
+    }
+    BatchLaunchArgs a;
+    a.srcs = srcs;
+    a.dsts = dsts;
+    a.counts = counts;
+    a.n = n;
+    a.n_jobs = n_jobs;
+    a.op = op;
+    a.stream = (hipStream_t)stream;
+    a.tune = current_tuning();
+    if (fp16_impl != MI_CCL_FP16_DEFAULT)
+        a.tune.fp16_impl = fp16_impl;
+    return status_of(dispatch_batch(dtype, keep, bf16_impl, a));
 }
 
 int mi_ccl_comp_batch_reduce(const void* in_buf, const size_t* offsets, size_t n_offsets, size_t count, void* inout,

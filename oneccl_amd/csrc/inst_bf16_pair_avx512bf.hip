@@ -1,4 +1,5 @@
 // Kernels of one element-traits class: Bf16PairwiseTraits<true, true>
+#include "batch_kernels.hpp"
 #include "fusion_kernels.hpp"
 
 namespace mi {
@@ -9,4 +10,5 @@ struct StreamUnroll<Bf16PairwiseTraits<true, true>> {
 };
 template hipError_t launch_reduce<Bf16PairwiseTraits<true, true>>(const LaunchArgs&);
 template hipError_t launch_fusion_reduce<Bf16PairwiseTraits<true, true>>(const FusionLaunchArgs&);
+template hipError_t launch_reduce_batch<Bf16PairwiseTraits<true, true>>(const BatchLaunchArgs&);
 }  // namespace mi

@@ -1,4 +1,5 @@
 // Kernels of one element-traits class: F32Traits
+#include "batch_kernels.hpp"
 #include "fusion_kernels.hpp"
 
 namespace mi {
@@ -8,4 +9,5 @@ struct HasUnrollVariants<F32Traits> {
 };
 template hipError_t launch_reduce<F32Traits>(const LaunchArgs&);
 template hipError_t launch_fusion_reduce<F32Traits>(const FusionLaunchArgs&);
+template hipError_t launch_reduce_batch<F32Traits>(const BatchLaunchArgs&);
 }  // namespace mi

@@ -15,6 +15,7 @@
 
 #include "../../oneccl_amd/csrc/ccl_comp.hpp"
 #include "../../oneccl_amd/csrc/ccl_fusion.hpp"
+#include "../../oneccl_amd/csrc/ccl_pipeline.hpp"
 #include "../../oracle/ccl_comp_oracle.h"
 
 #define CK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { printf("HIP error %s at line %d\n", hipGetErrorString(e_), __LINE__); exit(2); } } while (0)
@@ -398,6 +399,104 @@ int main() {
         mgr.reset();
         for (auto* p : peer_bufs) delete p;
         for (int t = 0; t < K; t++) { delete send[t]; delete recv[t]; }
+    }
+    // read_reduce_write shape (reduce_scatter_large_sycl_impl.hpp:22-66): even[i] = pair[i] + local[i] for seven peers in
+    // one launch, against seven oracle calls; then copy_data shape (one input per job)
+    {
+        const int J = 7;
+        const size_t cnt[J] = { 1, 17, 4099, 0, 70001, 16, 262144 };
+        std::vector<std::vector<uint16_t>> pairv(J), localv(J);
+        std::vector<std::unique_ptr<DevBuf<uint16_t>>> dp, dl, de;
+        std::vector<const void*> srcs, copy_srcs;
+        std::vector<void*> dsts;
+        std::vector<size_t> counts;
+        uint32_t x = 12345;
+        for (int j = 0; j < J; j++) {
+            pairv[j].resize(cnt[j]); localv[j].resize(cnt[j]);
+            for (size_t i = 0; i < cnt[j]; i++) {
+                x = x * 1664525u + 1013904223u; pairv[j][i] = to_lp((float)((int)(x >> 8) % 2001 - 1000) / 256.f, ccl::datatype::bfloat16);
+                x = x * 1664525u + 1013904223u; localv[j][i] = to_lp((float)((int)(x >> 8) % 2001 - 1000) / 512.f, ccl::datatype::bfloat16);
+            }
+            dp.emplace_back(new DevBuf<uint16_t>(pairv[j])); dl.emplace_back(new DevBuf<uint16_t>(localv[j]));
+            de.emplace_back(new DevBuf<uint16_t>(cnt[j]));
+            srcs.push_back(dp[j]->p); srcs.push_back(dl[j]->p); copy_srcs.push_back(dl[j]->p);
+            dsts.push_back(de[j]->p); counts.push_back(cnt[j]);
+        }
+        ccl_sched sched; sched.stream = stream;
+        ccl_comp_reduce_batch(&sched, srcs, 2, dsts, counts, DT(ccl::datatype::bfloat16), ccl::reduction::sum);
+        for (int j = 0; j < J; j++) {
+            std::vector<uint16_t> want = pairv[j];
+            orc_comp_reduce(localv[j].data(), cnt[j], want.data(), ORC_BFLOAT16, ORC_SUM, (int)ccl::global_data::env().bf16_impl_type, ORC_FP16_AVX512F);
+            EXPECT(de[j]->host() == want, "read_reduce_write shape: job %d of %zu elements", j, cnt[j]);
+        }
+        ccl_comp_reduce_batch(&sched, copy_srcs, 1, dsts, counts, DT(ccl::datatype::bfloat16), ccl::reduction::sum);
+        for (int j = 0; j < J; j++) EXPECT(de[j]->host() == localv[j], "copy_data shape: job %d", j);
+        bool threw = false;
+        try { ccl_comp_reduce_batch(&sched, copy_srcs, 2, dsts, counts, DT(ccl::datatype::bfloat16), ccl::reduction::sum); } catch (const ccl::exception&) { threw = true; }
+        EXPECT(threw, "a pointer table of the wrong length must throw");
+    }
+    // The chunked, double-buffered pipeline (reduce_scatter_large_impl, reduce_scatter_large_sycl_impl.hpp:98-301): chunk
+    // sizes that do and do not divide the count, with and without the pair-reduce stage, in place -- bit-identical to
+    // the unchunked reduce and to the oracle.
+    {
+        const int N = 5;
+        ccl_sched sched; sched.stream = stream;
+        for (ccl::datatype d : { ccl::datatype::bfloat16, ccl::datatype::float32 }) {
+            const size_t esz = DT(d).size();
+            for (size_t count : { (size_t)1000003, (size_t)8 * 65536, (size_t)100 }) {
+                for (size_t chunk_bytes : { (size_t)65536 * esz, (size_t)48000 }) {
+                    for (int with_pair = 0; with_pair < 2; with_pair++) {
+                        for (int keep = 0; keep < (d == ccl::datatype::bfloat16 ? 2 : 1); keep++) {
+                            std::vector<std::vector<unsigned char>> hl(N), hp(N);
+                            std::vector<std::unique_ptr<DevBuf<unsigned char>>> dl, dp;
+                            std::vector<const void*> local, pair;
+                            uint32_t x = 777 + (uint32_t)count + with_pair;
+                            auto fill = [&](std::vector<unsigned char>& h) {
+                                h.resize(count * esz);
+                                for (size_t i = 0; i < count; i++) {
+                                    x = x * 1664525u + 1013904223u;
+                                    const float v = (float)((int)(x >> 8) % 20001 - 10000) / 4096.f;
+                                    if (d == ccl::datatype::bfloat16) { uint16_t b = to_lp(v, d); memcpy(&h[i * 2], &b, 2); }
+                                    else memcpy(&h[i * 4], &v, 4);
+                                }
+                            };
+                            for (int i = 0; i < N; i++) {
+                                fill(hl[i]); dl.emplace_back(new DevBuf<unsigned char>(hl[i])); local.push_back(dl[i]->p);
+                                if (with_pair) { fill(hp[i]); dp.emplace_back(new DevBuf<unsigned char>(hp[i])); pair.push_back(dp[i]->p); }
+                            }
+                            const int impl = (int)ccl::global_data::env().bf16_impl_type;
+                            // oracle: staged_i = pair_i OP local_i (rounded to dtype), then the chain over i
+                            std::vector<std::vector<unsigned char>> staged = hl;
+                            if (with_pair)
+                                for (int i = 0; i < N; i++) {
+                                    staged[i] = hp[i];
+                                    orc_comp_reduce(hl[i].data(), count, staged[i].data(), (int)d, ORC_SUM, impl, ORC_FP16_AVX512F);
+                                }
+                            std::vector<const void*> sp;
+                            for (int i = 0; i < N; i++) sp.push_back(staged[i].data());
+                            std::vector<unsigned char> want(count * esz);
+                            orc_reduce_n(sp.data(), N, want.data(), count, (int)d, ORC_SUM, keep, 0, impl, ORC_FP16_AVX512F);
+                            ccl_chunked_reducer red(chunk_bytes, N);
+                            DevBuf<unsigned char> out(count * esz);
+                            red.run(&sched, local, pair, count, out.p, DT(d), ccl::reduction::sum, keep);
+                            EXPECT(out.host() == want, "chunked reduce: dtype %d count %zu chunk %zu pair %d keep %d", (int)d, count, chunk_bytes, with_pair, keep);
+                            EXPECT(red.chunks_of_last_run() == (count * esz + chunk_bytes - 1) / chunk_bytes, "chunk count");
+                            if (!with_pair) {       // the same bits as the unchunked call, and in place on input 2
+                                DevBuf<unsigned char> whole(count * esz);
+                                std::vector<const void*> peers(local.begin() + 1, local.end());
+                                ccl_comp_reduce_n(&sched, local[0], peers, count, whole.p, DT(d), ccl::reduction::sum, keep);
+                                EXPECT(whole.host() == out.host(), "chunked and unchunked reduce differ");
+                                red.run(&sched, local, pair, count, dl[2]->p, DT(d), ccl::reduction::sum, keep);
+                                EXPECT(dl[2]->host() == want, "chunked reduce in place");
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        bool threw = false;
+        try { ccl_chunked_reducer bad(1000, 4); } catch (const ccl::exception&) { threw = true; }
+        EXPECT(threw, "a chunk size that is not a multiple of 16 bytes must throw");
     }
     CK(hipStreamDestroy(stream));
     printf("%d checks, %d failed\n", g_checks, g_fail);
