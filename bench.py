@@ -43,12 +43,63 @@ WORKLOADS = {
     # calibration for the rocprofv3 FETCH_SIZE / WRITE_SIZE counters: a plain copy of known size
     "copy_ref": dict(dtype="bfloat16", n=1, count=1_003_782_144, keep=False, sets=1, copy=True,
                      desc="mi_ccl_comp_copy of 2,007,564,288 bytes (counter calibration: reads and writes that many bytes)"),
+    # the ceiling of the memory system beside the kernel's figure: reads alone, writes alone, the runtime's own copy
+    "read_only": dict(dtype="bfloat16", n=8, m=0, count=1_003_782_144, keep=False, sets=1, probe="read",
+                      desc="eight 2,007,564,288-byte buffers read, nothing written (mi_ccl_probe_bandwidth, the streaming "
+                           "reduce's access shape)"),
+    "write_only_one": dict(dtype="bfloat16", n=0, m=1, count=1_003_782_144, keep=False, sets=1, probe="write_one",
+                           desc="one 2,007,564,288-byte buffer written, one 16-byte store per lane (the copy kernels' shape)"),
+    "write_only_four": dict(dtype="bfloat16", n=0, m=1, count=1_003_782_144, keep=False, sets=1, probe="write_four",
+                            desc="one 2,007,564,288-byte buffer written, four 16-byte stores per lane (the reduce kernels' shape)"),
+    "memcpy_dtod": dict(dtype="bfloat16", n=1, count=1_003_782_144, keep=False, sets=1, probe="memcpy",
+                        desc="hipMemcpyDtoDAsync of 2,007,564,288 bytes (the runtime's own device-to-device copy)"),
 }
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two runs), each scaled by what the
-# same counter reads for a plain copy of known size (x2.0000 and x1.0000); the summary is kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"c5_bf16": (15_684_420 + 1_963_194) * 1024,
-                          "rw_8to8_bf16": (8_388_986 + 8_396_252) * 1024, "write_1to7_bf16": (1_048_613 + 7_341_101) * 1024}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "measured_traffic.json")
+
+
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch from profiles/measured_traffic.json (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each
+    scaled by what the same counter reads for a plain copy of known size), or None when the file holds no entry for
+    this workload with the kernel that was actually launched."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None
+    e = table.get("workloads", {}).get(workload)
+    if not e or e.get("kernel") != kernel:
+        return None
+    return int(e["hbm_bytes_per_launch"])
+
+
+def host_cpu():
+    """Model name, physical cores per socket, sockets and NUMA nodes of the host, from /proc/cpuinfo and sysfs."""
+    model, cores, phys = "unknown", {}, set()
+    try:
+        pid = cid = None
+        for line in open("/proc/cpuinfo"):
+            k, _, v = line.partition(":")
+            k, v = k.strip(), v.strip()
+            if k == "model name":
+                model = v
+            elif k == "physical id":
+                pid = v
+                phys.add(v)
+            elif k == "core id":
+                cid = v
+            elif not k and pid is not None:
+                cores.setdefault(pid, set()).add(cid)
+                pid = cid = None
+    except OSError:
+        pass
+    per_socket = max((len(c) for c in cores.values()), default=os.cpu_count() or 1)
+    try:
+        numa = len([d for d in os.listdir("/sys/devices/system/node") if d.startswith("node") and d[4:].isdigit()])
+    except OSError:
+        numa = 1
+    return dict(cpu_model=model, physical_cores_per_socket=per_socket, sockets=max(1, len(phys)), numa_nodes=max(1, numa),
+                logical_cpus=os.cpu_count() or 1)
 
 
 def make_buffers(torch, w, seed):
@@ -114,13 +165,42 @@ def cpu_baseline(torch, comp, w, bufs, sample_elems):
     one = algo_bytes / (t1 - t0) / 1e9
     ref_out = buf[:s].copy()
     del buf, tmp, acc
-    # (ii) W threads on disjoint count/W partitions (what CCL_WORKER_COUNT=W does), fused single pass
-    W = min(16, os.cpu_count() or 1)
+    # (ii) W threads on disjoint count/W partitions -- the reference's only parallelism inside a rank
+    # (CCL_WORKER_COUNT=W: src/parallelizer/parallelizer.cpp:230-241,374-379) -- W = physical cores of one socket, as
+    # far as this process may use them; threads are left to the scheduler (no pinning, first-touch placement)
+    cpu = host_cpu()
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    W = max(1, min(cpu["physical_cores_per_socket"], usable, int(os.environ.get("OMP_NUM_THREADS", "1024"))))
     t0 = time.perf_counter()
     out = O.reduce_n(host, dt, O.SUM, keep=1 if w["keep"] else 0, quirk_tail=1, threads=W)
     t1 = time.perf_counter()
     multi = algo_bytes / (t1 - t0) / 1e9
     assert (out.view(np.uint8) == ref_out.view(np.uint8)).all(), "oracle forms disagree"
+    # ... and the same partitions through the reference's own pass structure and helpers (widen / fp32 add / narrow)
+    ref_multi = None
+    if ref_keep is not None:
+        from concurrent.futures import ThreadPoolExecutor
+        buf3 = np.concatenate(host)
+        tmp3, acc3 = np.zeros(s, np.float32), np.zeros(s, np.float32)
+        part = (s // W) // 16 * 16
+        bounds = [(p_ * part, part if p_ < W - 1 else s - p_ * part) for p_ in range(W)]
+
+        def one_partition(b_):
+            lo, ln = b_
+            return R.ref_batch_reduce_keep_sum(buf3.ctypes.data + 2 * lo, offs.ctypes.data, w["n"], ln,
+                                               buf3.ctypes.data + 2 * lo, tmp3.ctypes.data + 4 * lo,
+                                               acc3.ctypes.data + 4 * lo, O.BF16_AVX512BF)
+        with ThreadPoolExecutor(W) as pool:
+            t0 = time.perf_counter()
+            rcs = list(pool.map(one_partition, bounds))
+            t1 = time.perf_counter()
+        assert all(rc == 0 for rc in rcs)
+        assert (buf3[:s] == ref_out).all(), "the partitioned reference passes and the oracle disagree"
+        ref_multi = algo_bytes / (t1 - t0) / 1e9
+        del buf3, tmp3, acc3
     # (iii) the reference's own AVX-512 code (oracle/_ref, compiled from the reference's sources where the library
     # was built): its bf16 reduce rounds after every input, so this times the pairwise mode of the same reduction --
     # 2^31 elements per call at most, one thread
@@ -145,13 +225,19 @@ def cpu_baseline(torch, comp, w, bufs, sample_elems):
         return dict(value=round(ref_keep[0], 3), unit="GB/s", cores=1, kind="reference",
                     sample=sample + "; conversions by the reference's own ccl_bf16_load_as_fp32 / "
                            "ccl_fp32_store_as_bf16_avx512bf compiled from its sources, results equal to the oracle's; "
-                           f"scalar C port of the same passes: {one:.2f} GB/s; {W}-thread partitioned single-pass "
-                           f"port: {multi:.2f} GB/s",
-                    port=dict(value=round(one, 3), cores=1), multi_thread=dict(value=round(multi, 3), cores=W),
+                           f"scalar C port of the same passes: {one:.2f} GB/s; the reference passes on {W} partitions "
+                           f"(CCL_WORKER_COUNT={W}): {ref_multi:.2f} GB/s; {W}-thread partitioned single-pass port: "
+                           f"{multi:.2f} GB/s",
+                    **cpu, worker_count=W, placement="threads unpinned, first-touch pages",
+                    port=dict(value=round(one, 3), cores=1),
+                    multi_thread=dict(value=round(ref_multi, 3), cores=W, kind="reference",
+                                      what="ccl_comp_batch_reduce pass structure on count/W partitions"),
+                    multi_thread_fused_port=dict(value=round(multi, 3), cores=W, kind="port"),
                     **({"reference_pairwise": ref_leg} if ref_leg else {})), out, s
     return dict(value=round(one, 3), unit="GB/s", cores=1, kind="port",
                 sample=sample + f"; {W}-thread partitioned single-pass port: {multi:.2f} GB/s",
-                multi_thread=dict(value=round(multi, 3), cores=W),
+                **cpu, worker_count=W, placement="threads unpinned, first-touch pages",
+                multi_thread_fused_port=dict(value=round(multi, 3), cores=W, kind="port"),
                 **({"reference_pairwise": ref_leg} if ref_leg else {})), out, s
 
 
@@ -183,16 +269,30 @@ def main():
     esz = 2 if dt == comp.BFLOAT16 else 4
     lp = comp.LP_KEEP_PRECISION if w["keep"] else comp.LP_PAIRWISE
     n, count = w["n"], w["count"]
-    sets = [make_buffers(torch, w, 1234 + i) for i in range(w["sets"])]
+    probe = w.get("probe")
+    sets = [make_buffers(torch, dict(w, n=max(n, 1)), 1234 + i) for i in range(w["sets"])]
     m = w.get("m", 1)
-    outs = [s[0] if w.get("in_place") else torch.empty_like(s[0]) for s in sets]
-    extra_outs = [[torch.empty_like(s[0]) for _ in range(m - 1)] for s in sets]
+    outs = [s[0] if (w.get("in_place") or probe in ("read", "write_one", "write_four")) else torch.empty_like(s[0]) for s in sets]
+    extra_outs = [[torch.empty_like(s[0]) for _ in range(max(m, 1) - 1)] for s in sets]
     algo_bytes = (n + m) * count * esz
     stream = torch.cuda.current_stream()
+    hip = None
+    if probe == "memcpy":
+        import ctypes
+        hip = ctypes.CDLL("libamdhip64.so")
+        hip.hipMemcpyDtoDAsync.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
 
     def step(i):
         s = sets[i % len(sets)]
-        if w.get("copy"):
+        if probe == "read":
+            comp.probe_bandwidth(comp.PROBE_READ, s, count * esz, stream=stream)
+        elif probe in ("write_one", "write_four"):
+            comp.probe_bandwidth(comp.PROBE_WRITE_ONE if probe == "write_one" else comp.PROBE_WRITE_FOUR, s[:1], count * esz,
+                                 stream=stream)
+        elif probe == "memcpy":
+            rc = hip.hipMemcpyDtoDAsync(outs[i % len(sets)].data_ptr(), s[0].data_ptr(), count * esz, stream.cuda_stream)
+            assert rc == 0, f"hipMemcpyDtoDAsync: {rc}"
+        elif w.get("copy"):
             comp.comp_copy(s[0], outs[i % len(sets)], count * esz, use_nontemporal=True, stream=stream)
         elif m > 1:
             comp.comp_reduce_write_n(dt, comp.SUM, s, [outs[i % len(sets)]] + extra_outs[i % len(sets)], count,
@@ -202,7 +302,7 @@ def main():
 
     # parity outside the timed region: GPU result of set 0 against the oracle on a sample
     base = None
-    if not args.no_cpu_baseline and not w.get("copy"):
+    if not args.no_cpu_baseline and not w.get("copy") and not probe:
         snapshot = [b.clone() for b in sets[0]] if w.get("in_place") else sets[0]
         base, want, s_elems = cpu_baseline(torch, comp, w, snapshot, args.cpu_sample)
         step(0)
@@ -236,6 +336,7 @@ def main():
 
     ms_per_step = (t1 - t0) / args.steps * 1e3
     kernel_ms = ev0.elapsed_time(ev1) / args.steps
+    kernel = "hipMemcpyDtoDAsync" if probe == "memcpy" else comp.last_kernel()
     value = algo_bytes / (ms_per_step * 1e-3) / 1e9
     achieved = algo_bytes / (kernel_ms * 1e-3) / 1e9
     out = {
@@ -258,8 +359,8 @@ def main():
                    "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
                    "parity": "bit-exact vs oracle on the CPU-baseline sample" if base else "not checked in this run"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                     "kernel_ms": round(kernel_ms, 4)},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(args.workload, kernel),
+                     "kernel_ms": round(kernel_ms, 4), "kernel": kernel},
         "cpu_baseline": base,
     }
     print(json.dumps(out))

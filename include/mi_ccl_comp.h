@@ -125,7 +125,7 @@ int mi_ccl_comp_reduce_write_n(int dtype, int op, const void* const* srcs, int n
  * dsts[j][i] = srcs[j * n + 0][i] OP srcs[j * n + 1][i] OP ... OP srcs[j * n + n - 1][i] (1 <= n <= 8, the same for every
  * job).  srcs (n_jobs x n pointers, job after job), dsts and counts are HOST arrays; a job's output may be one of its
  * own inputs, the jobs must not overlap one another; a job with count 0 is skipped without looking at its pointers.
- * The job table travels in the kernel arguments (96 jobs or 288 pointers per launch, more jobs take more launches):
+ * The job table travels in the kernel arguments (96 jobs or 320 pointers (inputs and outputs) per launch, more jobs take more launches):
  * nothing is allocated.  Replaces read_reduce_write (n = 2: even[i] = pair[i] + local[i] for every peer i in one kernel,
  * src/coll/algorithms/reduce_scatter/sycl/reduce_scatter_large_sycl_impl.hpp:22-66), reduce_read_write_kernel_{1..7}
  * (src/kernels/kernels.cl:156-177) and, with n = 1, copy_data (N copies in one kernel, used at :216-224 of the same
@@ -214,6 +214,20 @@ int mi_ccl_fusion_reduce_static(const size_t* counts, size_t k, int dtype, size_
                                 const void* const* own_tensors, const void* const* peers, int n_peers,
                                 void* const* out_tensors, int lp_mode, int bf16_impl, int fp16_impl, void* stream);
 
+/* ---- measurement aid ------------------------------------------------------------------------------ */
+
+/* Read-only and write-only streams in the access shapes of the kernels above, for putting a measured ceiling of the
+ * memory system beside a kernel's figure (no counterpart in the reference).  bytes: per buffer, a multiple of 16;
+ * buffers 16-byte aligned.  MI_CCL_PROBE_READ reads n buffers and writes nothing; MI_CCL_PROBE_WRITE_ONE /
+ * MI_CCL_PROBE_WRITE_FOUR overwrite bufs[0] (n = 1) with one / four 16-byte stores per lane. */
+enum mi_ccl_probe_kind { MI_CCL_PROBE_READ = 0, MI_CCL_PROBE_WRITE_ONE = 1, MI_CCL_PROBE_WRITE_FOUR = 2 };
+int mi_ccl_probe_bandwidth(int kind, void* const* bufs, int n, size_t bytes, void* stream);
+
+/* Name of the kernel template that the calling thread's most recent reduce / copy / fusion / probe call launched
+ * ("reduce_multi_phased_kernel", "reduce_vec_kernel", "copy_kernel", ...; "" before the first call), so that a
+ * measurement can say which kernel it belongs to.  No counterpart in the reference. */
+const char* mi_ccl_last_kernel(void);
+
 /* ---- launch tuning ------------------------------------------------------------------------------- */
 
 /* Launch-shape knobs, the counterpart of CCL_KERNEL_GROUP_SIZE / CCL_KERNEL_MEM_ALIGN
@@ -224,7 +238,9 @@ int mi_ccl_fusion_reduce_static(const size_t* counts, size_t k, int dtype, size_
  * also keeps one-input calls on the general reduce kernels instead of the copy and broadcast kernels -- for tests and
  * measurements),
  * "phased_min_bytes" (scales the sizes from which the phased kernels are used; default 160 MB), "num_cus" (read
- * only), and "fp16_impl" (what MI_CCL_FP16_DEFAULT stands for: 2, 3 or 4 of enum mi_ccl_fp16_impl above).
+ * only), "fp16_impl" (what MI_CCL_FP16_DEFAULT stands for: 2, 3 or 4 of enum mi_ccl_fp16_impl above), and
+ * "launch_block_limit" (blocks per launch of the copy, broadcast and converter kernels, which cut larger work into
+ * several launches; 0 = what HIP allows, 2^24 - 1; smaller values let tests exercise the cutting).
  * Returns invalid_arguments for an unknown name or out-of-range value. */
 int mi_ccl_set_param(const char* name, long value);
 long mi_ccl_get_param(const char* name);

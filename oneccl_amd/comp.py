@@ -33,7 +33,7 @@ EXPORTS = [
     "mi_ccl_fusion_plan_create", "mi_ccl_fusion_plan_destroy", "mi_ccl_fusion_plan_bytes",
     "mi_ccl_fusion_plan_offset", "mi_ccl_fusion_pack", "mi_ccl_fusion_unpack", "mi_ccl_fusion_reduce",
     "mi_ccl_fusion_reduce_static",
-    "mi_ccl_set_param", "mi_ccl_get_param",
+    "mi_ccl_probe_bandwidth", "mi_ccl_last_kernel", "mi_ccl_set_param", "mi_ccl_get_param",
 ]
 
 
@@ -85,6 +85,9 @@ def lib():
     L.mi_ccl_fusion_unpack.argtypes = [vp, vp, vp, vp]
     L.mi_ccl_fusion_reduce.argtypes = [vp, i, vp, vp, i, vp, i, i, i, vp]
     L.mi_ccl_fusion_reduce_static.argtypes = [vp, sz, i, sz, i, vp, vp, i, vp, i, i, i, vp]
+    L.mi_ccl_probe_bandwidth.argtypes = [i, vp, i, sz, vp]
+    L.mi_ccl_last_kernel.restype = C.c_char_p
+    L.mi_ccl_last_kernel.argtypes = []
     L.mi_ccl_set_param.argtypes = [C.c_char_p, C.c_long]
     L.mi_ccl_get_param.restype = C.c_long
     L.mi_ccl_get_param.argtypes = [C.c_char_p]
@@ -288,6 +291,20 @@ def fusion_reduce_static(counts, dtype, align, op, own_tensors, peers, out_tenso
     _check(lib().mi_ccl_fusion_reduce_static(cnt, k, dtype, align, op, _ptr_array(own_tensors), _ptr_array(peers),
                                              len(peers), _ptr_array(out_tensors), lp_mode, bf16_impl, fp16_impl,
                                              _stream(stream)), "mi_ccl_fusion_reduce_static")
+
+
+PROBE_READ, PROBE_WRITE_ONE, PROBE_WRITE_FOUR = 0, 1, 2
+
+
+def probe_bandwidth(kind, bufs, nbytes, stream=None):
+    """Read-only (kind PROBE_READ, all of bufs) or write-only (PROBE_WRITE_ONE / PROBE_WRITE_FOUR, bufs[0]) stream."""
+    _check(lib().mi_ccl_probe_bandwidth(kind, _ptr_array(bufs), len(bufs), nbytes, _stream(stream)),
+           "mi_ccl_probe_bandwidth")
+
+
+def last_kernel():
+    """Kernel template the calling thread's most recent call launched."""
+    return lib().mi_ccl_last_kernel().decode()
 
 
 def set_param(name, value):

@@ -16,15 +16,16 @@
 namespace mi {
 
 constexpr int kBatchMaxJobs = 96;       // jobs per launch
-constexpr int kBatchMaxPtrs = 288;      // pointers per launch: jobs x (n + 1)
+constexpr int kBatchMaxPtrs = 320;      // pointers per launch: jobs x (n + 1); 64 jobs of four inputs fit
 constexpr int kBatchUnroll = 4;         // vectors per lane and tile: 16 KiB of every buffer per tile
 
-struct BatchTable {                     // by-value kernel argument (3.5 KB of the 4 KB there are)
+struct BatchTable {                     // by-value kernel argument (3.8 KB of the 4 KB there are)
     const void* p[kBatchMaxPtrs];       // job j: inputs p[j * (n + 1) + 0 .. n - 1], output p[j * (n + 1) + n]
     uint64_t count[kBatchMaxJobs];      // elements
     uint32_t tile_end[kBatchMaxJobs];   // tiles of jobs 0..j together
     uint8_t head[kBatchMaxJobs];        // elements before job j's first vector
 };
+static_assert(sizeof(BatchTable) + 64 <= 4096, "the job table and the other arguments must fit the kernel-argument segment");
 
 struct BatchLaunchArgs {
     const void* const* srcs;            // host array, n_jobs x n device pointers, job after job
@@ -128,6 +129,7 @@ inline hipError_t launch_batch_op(const BatchLaunchArgs& a) {
         j0 += nj;
         if (tiles == 0) continue;
         const int grid = grid_for(tiles, a.tune);
+        g_last_kernel = "reduce_batch_kernel";
         hipLaunchKernelGGL((reduce_batch_kernel<TR, OP>), dim3(grid), dim3(kBlock), 0, a.stream, tb, a.n, nj, (uint32_t)tiles);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;

@@ -42,6 +42,8 @@ MI_DECLARE(Bf16KeepTraits<true>);
 // ---------------------------------------------------------------------------------------------------
 // tuning state and device facts
 
+thread_local const char* g_last_kernel = "";
+
 static std::atomic<int> g_waves_per_cu{ 256 };
 static std::atomic<int> g_max_blocks{ 0 };
 static std::atomic<int> g_xcd_chunked{ 0 };
@@ -440,11 +442,99 @@ f16_to_f32_kernel(const uint16_t* in, uint32_t* out, uint32_t head, uint64_t nqu
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Calibration kernels: what the memory system sustains for reads alone and for writes alone, in the access shapes
+// the kernels above use.  Measurement aids, not part of any reduce.
+
+// n buffers read as the streaming reduce reads them (a tile of 256 x 4 vectors per block, the inputs one after the
+// other, nontemporal loads), nothing written: the xor of what was read decides a store that practically never happens.
+__global__ void __launch_bounds__(kBlock)
+probe_read_kernel(SrcTable src, int n, uint64_t nvec, u32x4* sink) {
+    constexpr int U = 4;
+    constexpr uint64_t kTile = (uint64_t)kBlock * U;
+    u32x4 acc = { 0, 0, 0, 0 };
+    for (uint64_t t = blockIdx.x; t * kTile < nvec; t += gridDim.x) {
+        const uint64_t base = t * kTile + threadIdx.x;
+        for (int j = 0; j < n; j++) {
+            const u32x4* s = (const u32x4*)src.p[j];
+            u32x4 x[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) x[u] = (base + (uint64_t)u * kBlock < nvec) ? __builtin_nontemporal_load(s + base + (uint64_t)u * kBlock) : u32x4{ 0, 0, 0, 0 };
+#pragma unroll
+            for (int u = 0; u < U; u++) acc ^= x[u];
+        }
+    }
+    if (acc[0] == 0x12345678u && acc[1] == 0x9abcdef0u && acc[2] == 0x0fedcba9u && acc[3] == 0x87654321u) sink[threadIdx.x] = acc;
+}
+
+// U vectors per lane stored with nontemporal stores, one tile per block.  U = 1 is the shape of the copy, broadcast
+// and converter kernels (a wave issues one store and ends), U = 4 that of the streaming reduce.
+template <int U>
+__global__ void __launch_bounds__(kBlock)
+probe_write_kernel(u32x4* dst, uint64_t nvec) {
+    constexpr uint64_t kTile = (uint64_t)kBlock * U;
+    const u32x4 v = { 1u, 2u, 3u, blockIdx.x };
+    for (uint64_t t = blockIdx.x; t * kTile < nvec; t += gridDim.x) {
+        const uint64_t base = t * kTile + threadIdx.x;
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            if (base + (uint64_t)u * kBlock < nvec) __builtin_nontemporal_store(v, dst + base + (uint64_t)u * kBlock);
+    }
+}
+
+static __device__ u32x4 g_probe_sink[kBlock];
+static std::atomic<u32x4*> g_probe_sink_ptr[64];
+
 }  // namespace mi
 
 using namespace mi;
 
 extern "C" {
+
+int mi_ccl_probe_bandwidth(int kind, void* const* bufs, int n, size_t bytes, void* stream) {
+    if (!bufs || n < 1 || n > kMaxSrcs || (bytes % 16) != 0 || bytes == 0)
+        return MI_CCL_INVALID_ARGUMENTS;
+    for (int j = 0; j < n; j++)
+        if (!bufs[j] || ((uintptr_t)bufs[j] & 15u))
+            return MI_CCL_INVALID_ARGUMENTS;
+    const uint64_t nvec = bytes / 16;
+    if (kind == MI_CCL_PROBE_READ) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+            return MI_CCL_RUNTIME_ERROR;
+        u32x4* sink = g_probe_sink_ptr[dev].load(std::memory_order_acquire);
+        if (!sink) {
+            void* sym = nullptr;
+            const hipError_t e = hipGetSymbolAddress(&sym, HIP_SYMBOL(g_probe_sink));
+            if (e != hipSuccess)
+                return status_of(e);
+            sink = (u32x4*)sym;
+            g_probe_sink_ptr[dev].store(sink, std::memory_order_release);
+        }
+        SrcTable s;
+        for (int j = 0; j < n; j++) s.p[j] = bufs[j];
+        const uint64_t tiles = (nvec + kBlock * 4 - 1) / (kBlock * 4);
+        g_last_kernel = "probe_read_kernel";
+        hipLaunchKernelGGL(probe_read_kernel, dim3((unsigned)(tiles < 65536 ? tiles : 65536)), dim3(kBlock), 0,
+                           (hipStream_t)stream, s, n, nvec, sink);
+        return status_of(hipGetLastError());
+    }
+    if (kind == MI_CCL_PROBE_WRITE_ONE || kind == MI_CCL_PROBE_WRITE_FOUR) {
+        if (n != 1)
+            return MI_CCL_INVALID_ARGUMENTS;
+        const unsigned u = kind == MI_CCL_PROBE_WRITE_ONE ? 1 : 4;
+        const uint64_t tiles = (nvec + kBlock * u - 1) / (kBlock * u);
+        const uint64_t cap = kind == MI_CCL_PROBE_WRITE_ONE ? hip_block_limit(kBlock) : 65536;
+        const unsigned grid = (unsigned)(tiles < cap ? tiles : cap);
+        g_last_kernel = "probe_write_kernel";
+        if (u == 1)
+            hipLaunchKernelGGL(probe_write_kernel<1>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, (u32x4*)bufs[0], nvec);
+        else
+            hipLaunchKernelGGL(probe_write_kernel<4>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, (u32x4*)bufs[0], nvec);
+        return status_of(hipGetLastError());
+    }
+    return MI_CCL_INVALID_ARGUMENTS;
+}
 
 size_t mi_ccl_datatype_size(int dtype) {
     return (dtype >= 0 && dtype < MI_CCL_DATATYPE_LAST) ? kDtypeSize[dtype] : 0;
@@ -578,6 +668,7 @@ static int launch_copy(const void* in, void* out, size_t bytes, bool nontemporal
         const uint64_t skip = i ? w.head + p.group0 * 16 : 0;
         const unsigned char* s = (const unsigned char*)in + skip;
         unsigned char* d = (unsigned char*)out + skip;
+        g_last_kernel = "copy_kernel";
         if (nontemporal)
             hipLaunchKernelGGL(copy_kernel<true>, dim3(p.grid), dim3(kBlock), 0, stream, s, d, p.head, p.ngroup, p.tail);
         else
@@ -598,6 +689,7 @@ static int launch_broadcast(const void* in, void* const* dsts, int m, size_t byt
         const uint64_t skip = i ? b.head + p.vec0 * 16 : 0;
         DstTable d;
         for (int k = 0; k < kMaxDsts; k++) d.p[k] = (unsigned char*)dsts[k < m ? k : 0] + skip;
+        g_last_kernel = "broadcast_kernel";
         hipLaunchKernelGGL(broadcast_kernel, dim3(p.grid), dim3(kBlock), 0, stream, (const unsigned char*)in + skip, d, m,
                            p.head, p.nvec, p.tail, b.sect_tiles);
         const hipError_t e = hipGetLastError();
@@ -689,6 +781,10 @@ int mi_ccl_convert_fp16_to_fp32_arrays(const void* fp16_buf, void* fp32_buf, siz
         hipLaunchKernelGGL(f16_to_f32_kernel, dim3(p.grid), dim3(kBlock), 0, (hipStream_t)stream,
                            (const uint16_t*)fp16_buf + skip, (uint32_t*)fp32_buf + skip, p.head, p.ngroup, p.tail);
     });
+}
+
+const char* mi_ccl_last_kernel(void) {
+    return g_last_kernel;
 }
 
 int mi_ccl_set_param(const char* name, long value) {

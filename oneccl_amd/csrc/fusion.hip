@@ -281,6 +281,7 @@ static int fusion_copy(mi_ccl_fusion_plan* plan, const void* const* tensors, voi
         FusionPtrs ptrs;
         for (size_t t = t0; t < t1; t++) ptrs.p[t - t0] = tensors[t];
         int grid = grid_for(i1 - i0, tune);
+        g_last_kernel = "fusion_copy_kernel";
         hipLaunchKernelGGL(fusion_copy_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ptrs,
                            (unsigned char*)fusion_buf, plan->d_off, plan->d_bytes, plan->d_items + i0,
                            (uint32_t)(i1 - i0), (uint32_t)t0, to_fusion);

@@ -272,6 +272,7 @@ template <class TR, int OP, int NT>
 inline hipError_t launch_fusion_phased(const FusionLaunchArgs& a, const FusionPtrs& own, const FusionPtrs& out,
                                        const PeerPtrs& pp, uint64_t i0, uint64_t i1, size_t t0) {
     int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
+    g_last_kernel = "fusion_reduce_phased_kernel";
     hipLaunchKernelGGL((fusion_reduce_phased_kernel<TR, OP, NT>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, own, out, pp,
                        a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0, a.tune.sync);
     return hipGetLastError();
@@ -310,6 +311,7 @@ inline hipError_t launch_fusion_op(const FusionLaunchArgs& a) {
         }
         else {
             int grid = grid_for(i1 - i0, a.tune);
+            g_last_kernel = "fusion_reduce_kernel";
             hipLaunchKernelGGL((fusion_reduce_kernel<TR, OP>), dim3(grid), dim3(kBlock), 0, a.stream, own, out, pp,
                                a.n_peers, a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0);
             e = hipGetLastError();

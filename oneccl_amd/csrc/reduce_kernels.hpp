@@ -48,6 +48,10 @@ struct Tuning {
     int fp16_impl;           // which CPU implementation's float16 results to reproduce: 2, 3 (through fp32) or 4 (native)
 };
 
+// Name of the kernel template the calling thread's most recent entry-point call launched (diagnostics and
+// measurement: lets a benchmark say which kernel its figures belong to).
+extern thread_local const char* g_last_kernel;
+
 struct LaunchArgs {
     const void* const* srcs;    // host array of n device pointers
     int n;
@@ -841,6 +845,7 @@ inline hipError_t launch_fixed(const LaunchArgs& a, uint32_t head, uint64_t nvec
     for (int j = 0; j < N; j++) s.p[j] = a.srcs[j];
     const uint64_t tile = (uint64_t)kBlock * UNROLL;
     int grid = grid_for((nvec + tile - 1) / tile, a.tune);
+    g_last_kernel = "reduce_vec_kernel";
     hipLaunchKernelGGL((reduce_vec_kernel<TR, OP, N, UNROLL>), dim3(grid), dim3(kBlock), 0, a.stream, s, a.dst,
                        head, nvec, tail, a.tune.xcd_chunked);
     return hipGetLastError();
@@ -916,6 +921,7 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
     const uint32_t tail = (uint32_t)(a.count - head - nvec * VEC);
     if (wants_phased(a, nvec)) {
         int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
+        g_last_kernel = "reduce_multi_phased_kernel";
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
                            a.m, (uint32_t)head, nvec, tail, a.tune.sync);
         return hipGetLastError();
@@ -923,6 +929,7 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
     constexpr int UNROLL = 4;
     const uint64_t tile = (uint64_t)kBlock * UNROLL;
     int grid = grid_for((nvec + tile - 1) / tile, a.tune);
+    g_last_kernel = "reduce_multi_kernel";
     hipLaunchKernelGGL((reduce_multi_kernel<TR, OP, UNROLL>), dim3(grid), dim3(kBlock), 0, a.stream, s, a.n, d, a.m,
                        (uint32_t)head, nvec, tail, a.tune.xcd_chunked);
     return hipGetLastError();

@@ -1,5 +1,6 @@
 // Per-call time of small 4-input int32 reduces issued from C++ through the C ABI: what a latency-bound caller sees
 // (the Python binding used by the other benchmarks adds about 5 us of its own per call).
+// The result of every timed form is checked (all inputs are constant bytes, so the sums are known in closed form).
 // Prints one line per size: GPU-clock time per call of 2000 back-to-back calls, host time to enqueue one call, and
 // the round trip of one call followed by a stream synchronisation.  Then the case fusion exists for: 1,024 small bf16
 // gradient tensors reduced against 7 peers, one call per tensor against the fusion manager (requests queued one by
@@ -39,6 +40,43 @@ int main() {
                std::chrono::duration<double, std::micro>(t2 - t0).count() / iters,
                std::chrono::duration<double, std::micro>(t4 - t3).count() / 200);
         for (int i = 0; i < 5; i++) CK(hipFree(b[i]));
+    }
+    // Many small reduces: 64 independent 4-input int32 sums as 64 calls and as ONE call of mi_ccl_comp_reduce_batch
+    // (one launch).  Input k of every job holds the byte k + 1, so every output word must be 0x0a0a0a0a.
+    for (size_t bytes : {1024ul, 4096ul, 16384ul, 65536ul, 262144ul, 1048576ul, 4194304ul}) {
+        const int J = 64, N = 4;
+        std::vector<void*> in(J * N), out(J);
+        std::vector<const void*> srcs(J * N);
+        std::vector<size_t> counts(J, bytes / 4);
+        for (int j = 0; j < J; j++) {
+            for (int k = 0; k < N; k++) { CK(hipMalloc(&in[j * N + k], bytes)); CK(hipMemset(in[j * N + k], k + 1, bytes)); srcs[j * N + k] = in[j * N + k]; }
+            CK(hipMalloc(&out[j], bytes));
+        }
+        auto check = [&](const char* what) -> bool {
+            std::vector<uint32_t> h(bytes / 4);
+            for (int j = 0; j < J; j += 21) {
+                if (hipMemcpy(h.data(), out[j], bytes, hipMemcpyDeviceToHost) != hipSuccess) return false;
+                for (uint32_t v : h) if (v != 0x0a0a0a0au) { printf("WRONG RESULT (%s, job %d)\n", what, j); return false; }
+                (void)hipMemset(out[j], 0, bytes);
+            }
+            return true;
+        };
+        hipEvent_t e0, e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
+        const int rounds = 50;
+        auto calls = [&]() { for (int j = 0; j < J; j++) mi_ccl_comp_reduce_n(MI_CCL_INT32, MI_CCL_SUM, &srcs[j * N], N, out[j], bytes / 4, 0, 2, 0, s); };
+        auto batch = [&]() { mi_ccl_comp_reduce_batch(MI_CCL_INT32, MI_CCL_SUM, srcs.data(), N, out.data(), counts.data(), J, 0, 2, 0, s); };
+        float ms_calls, ms_batch;
+        calls(); CK(hipStreamSynchronize(s)); if (!check("64 calls")) return 1;
+        CK(hipEventRecord(e0, s)); for (int r = 0; r < rounds; r++) calls(); CK(hipEventRecord(e1, s)); CK(hipStreamSynchronize(s));
+        CK(hipEventElapsedTime(&ms_calls, e0, e1));
+        batch(); CK(hipStreamSynchronize(s)); if (!check("one batch call")) return 1;
+        CK(hipEventRecord(e0, s)); for (int r = 0; r < rounds; r++) batch(); CK(hipEventRecord(e1, s)); CK(hipStreamSynchronize(s));
+        CK(hipEventElapsedTime(&ms_batch, e0, e1));
+        const double gb = 5.0 * bytes * J / 1e9;
+        printf("64 jobs x %8zu B x4: 64 calls %.2f us per job (%.0f GB/s); one batch launch %.2f us per job (%.0f GB/s)\n", bytes,
+               ms_calls * 1e3 / rounds / J, gb / (ms_calls * 1e-3 / rounds), ms_batch * 1e3 / rounds / J, gb / (ms_batch * 1e-3 / rounds));
+        for (auto p : in) CK(hipFree(p));
+        for (auto p : out) CK(hipFree(p));
     }
     {
         const int K = 1024, NPEER = 7;

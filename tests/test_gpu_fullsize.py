@@ -1,6 +1,9 @@
 """The benchmark's full-size configurations, bit for bit: 8 x 1,003,782,144 bf16 (fp32 accumulate, RNE once) and
 4 x 1,003,782,144 fp32, compared over every element with the 16-thread oracle, plus size-independent properties
-(reduce with zeros is the identity on finite values, x + (-x) = +0, in-place equals out-of-place)."""
+(reduce with zeros is the identity on finite values, x + (-x) = +0, in-place equals out-of-place); the 2-input in-place
+fp32 sum at 16,777,216 elements, the 8-input bf16 sum at 33,554,432, and the fusion configuration at its full counts
+(256 bf16 tensors, log-uniform over [2,048, 2,097,152], 256-byte aligned offsets, seven peer fusion buffers) through
+pack + reduce + unpack and through the fused single pass."""
 import numpy as np
 import pytest
 
@@ -116,3 +119,92 @@ def test_more_than_2_pow_32_elements(comp, variant):
         assert torch.equal(big[0][:3], head_before)             # the bytes in front of the buffer are untouched
     finally:
         comp.set_param("variant", 0)
+
+
+def test_c1_fp32_two_inputs_in_place_16M(comp):
+    """2-input in-place sum, fp32, 16,777,216 elements per buffer, i.i.d. uniform[-1, 1): ccl_comp_reduce's shape."""
+    import torch
+    n = 16_777_216
+    rng = np.random.default_rng(101)
+    a = rng.uniform(-1, 1, n).astype(np.float32)
+    b = rng.uniform(-1, 1, n).astype(np.float32)
+    want = O.comp_reduce(a, b, O.FLOAT32, O.SUM)
+    assert (want.view(np.uint32) == (b + a).view(np.uint32)).all()        # one IEEE add per pair (numpy's is one too)
+    da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    comp.comp_reduce(comp.FLOAT32, comp.SUM, da, n, db)
+    torch.cuda.synchronize()
+    assert comp.last_kernel() == "reduce_vec_kernel"
+    assert (db.cpu().numpy().view(np.uint32) == want.view(np.uint32)).all()
+    assert torch.equal(da.cpu(), torch.from_numpy(a)), "the in buffer changed"
+
+
+def test_c2_bf16_eight_inputs_32M(comp):
+    """8-input bf16 sum, 33,554,432 elements per buffer, N(0, 1) cast with RNE, fp32 accumulation in input order, one
+    RNE narrowing: every element against the oracle, by the default kernel choice and by the streaming kernel."""
+    import torch
+    n = 33_554_432
+    rng = np.random.default_rng(102)
+    host = [O.bf16_from_f32(rng.standard_normal(n).astype(np.float32)) for _ in range(8)]
+    want = O.reduce_n(host, O.BFLOAT16, O.SUM, keep=1, threads=16)
+    dev = [torch.from_numpy(h.view(np.int16)).cuda() for h in host]
+    for variant in (0, 4):
+        comp.set_param("variant", variant)
+        try:
+            out = torch.zeros_like(dev[0])
+            comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, dev, out, n, lp_mode=comp.LP_KEEP_PRECISION)
+            torch.cuda.synchronize()
+        finally:
+            comp.set_param("variant", 0)
+        got = out.cpu().numpy().view(np.uint16)
+        assert (got == want).all(), f"variant {variant}: {np.count_nonzero(got != want)} elements differ"
+
+
+def test_c4_fusion_256_tensors_full_counts(comp):
+    """The fusion configuration at its real sizes: pack -> 8-input sum over the fusion buffer -> unpack, and the
+    fused single pass in both kernel forms, every tensor against the oracle's pack / reduce / unpack."""
+    import math
+    import torch
+    rng = np.random.default_rng(4)
+    counts = [int(round(math.exp(rng.uniform(math.log(2048), math.log(2_097_152))))) for _ in range(256)]
+    assert min(counts) >= 2048 and max(counts) <= 2_097_152 and sum(counts) > 50_000_000
+    tensors = [O.bf16_from_f32((rng.standard_normal(c) * 0.02).astype(np.float32)) for c in counts]
+    offs, total = O.fusion_offsets(counts, 2, 256)
+    assert all(int(o) % 256 == 0 for o in offs)
+    nelem = total // 2
+    peers = [O.bf16_from_f32((rng.standard_normal(nelem) * 0.02).astype(np.float32)) for _ in range(7)]
+    fb = O.fusion_pack(tensors, offs, total, 2)
+    fused = O.reduce_n([fb.view(np.uint16)] + peers, O.BFLOAT16, O.SUM, keep=1, threads=16)
+    want = O.fusion_unpack(fused.view(np.uint8), counts, offs, np.uint16)
+    plan = comp.FusionPlan(counts, comp.BFLOAT16, 256)
+    assert plan.nbytes == total and [plan.offset(i) for i in (0, 1, 255)] == [int(offs[i]) for i in (0, 1, 255)]
+    d_t = [torch.from_numpy(t.view(np.int16)).cuda() for t in tensors]
+    d_p = [torch.from_numpy(p.view(np.int16)).cuda() for p in peers]
+    # three steps
+    d_fb = torch.zeros(nelem, dtype=torch.int16, device="cuda")
+    plan.pack(d_t, d_fb)
+    comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, [d_fb] + d_p, d_fb, nelem, lp_mode=comp.LP_KEEP_PRECISION)
+    outs = [torch.zeros_like(t) for t in d_t]
+    plan.unpack(d_fb, outs)
+    torch.cuda.synchronize()
+    for i in range(256):
+        assert (outs[i].cpu().numpy().view(np.uint16) == want[i]).all(), f"pack/reduce/unpack: tensor {i} of {counts[i]} elements"
+    # fused single pass: the default choice at this size (phased) and the streaming kernel
+    for variant, kernel in ((0, "fusion_reduce_phased_kernel"), (2, "fusion_reduce_kernel")):
+        comp.set_param("variant", variant)
+        try:
+            outs = [torch.zeros_like(t) for t in d_t]
+            plan.reduce(comp.SUM, d_t, d_p, outs, lp_mode=comp.LP_KEEP_PRECISION)
+            torch.cuda.synchronize()
+            assert comp.last_kernel() == kernel
+        finally:
+            comp.set_param("variant", 0)
+        for i in range(256):
+            assert (outs[i].cpu().numpy().view(np.uint16) == want[i]).all(), f"fused ({kernel}): tensor {i}"
+    # and without a plan
+    outs = [torch.zeros_like(t) for t in d_t]
+    comp.fusion_reduce_static(counts, comp.BFLOAT16, 256, comp.SUM, d_t, d_p, outs, lp_mode=comp.LP_KEEP_PRECISION)
+    torch.cuda.synchronize()
+    for i in range(256):
+        assert (outs[i].cpu().numpy().view(np.uint16) == want[i]).all(), f"fused, static table: tensor {i}"
+    plan.close()
+

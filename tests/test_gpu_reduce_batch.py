@@ -68,7 +68,7 @@ def test_every_dtype_and_op_seven_jobs(comp, dtype, op):
 
 @pytest.mark.parametrize("n_jobs", [1, 7, 64, 200])
 def test_job_counts_and_mixed_sizes(comp, n_jobs):
-    """Counts log-uniform over 1 .. 2^20 (and a few empty jobs) in one call; 200 jobs of two inputs need three launches."""
+    """Counts log-uniform over 1 .. 2^20 (and a few empty jobs) in one call; 200 jobs of two inputs need three launches (96 jobs each at most)."""
     rng = np.random.default_rng(7100 + n_jobs)
     counts = [int(c) for c in np.exp(rng.uniform(0, np.log(1 << 20), n_jobs))]
     counts[0] = 1 << 20
