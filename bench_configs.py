@@ -15,7 +15,10 @@
          tensors: pack, unpack and the fused reduce
   copy   ccl_comp_copy at 64 MiB, 512 MiB and 3 GiB, and the bf16 <-> fp32 array converters at 2^28 elements
 
-    python bench_configs.py [--out results/configs.json] [--skip c3,batch,types,align,copy]
+    python bench_configs.py [--out results/configs.json] [--skip c3,batch,types,align,copy] [--only c1,c4] [--c3-k 7]
+
+--only runs just the named sections (c1, c2, c3, batch, types, align, copy, c4, latency), --c3-k just the named sizes of
+the sweep (size = 1 KiB x 4^k): what a profiler run of one kernel wants.
 
 EVERY row is checked before it is timed: the first buffer set goes through the call once and the result is compared,
 bit for bit, with the CPU oracle (oracle/, the checker -- it is never the thing measured) on the same inputs: whole
@@ -53,7 +56,15 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--out", default=os.path.join(ROOT, "results", "configs.json"))
     ap.add_argument("--skip", default="")
+    ap.add_argument("--only", default="")
+    ap.add_argument("--c3-k", default="", help="comma-separated exponents k of the C3 sizes 1 KiB x 4^k (default: all 11)")
     args = ap.parse_args()
+    only = [x for x in args.only.split(",") if x]
+    skip = [x for x in args.skip.split(",") if x]
+    c3_k = [int(x) for x in args.c3_k.split(",") if x] or list(range(11))
+
+    def want(section):
+        return (section in only) if only else (section not in skip)
     import numpy as np
     import torch
     import oneccl_amd.comp as comp
@@ -101,32 +112,34 @@ def main():
         checked[0] += 1
 
     # ---- C1
-    n1 = 16_777_216
-    sets = [[torch.empty(n1, dtype=torch.float32, device="cuda").uniform_(-1, 1) for _ in range(2)] for _ in range(8)]
+    if want("c1"):
+        n1 = 16_777_216
+        sets = [[torch.empty(n1, dtype=torch.float32, device="cuda").uniform_(-1, 1) for _ in range(2)] for _ in range(8)]
 
-    def c1_once():
-        comp.comp_reduce(comp.FLOAT32, comp.SUM, sets[0][1], n1, sets[0][0])
-        return sets[0][0]
-    verify_reduce("C1", O.FLOAT32, O.SUM, [sets[0][0], sets[0][1]], c1_once, n1)
-    us = timed(torch, lambda i: comp.comp_reduce(comp.FLOAT32, comp.SUM, sets[i % 8][1], n1, sets[i % 8][0]), 64, 16)
-    add("C1 fp32 sum, 2 inputs in place, 64 MiB", us, 3 * n1 * 4, f"8 rotating buffer sets; {comp.last_kernel()}")
-    del sets
+        def c1_once():
+            comp.comp_reduce(comp.FLOAT32, comp.SUM, sets[0][1], n1, sets[0][0])
+            return sets[0][0]
+        verify_reduce("C1", O.FLOAT32, O.SUM, [sets[0][0], sets[0][1]], c1_once, n1)
+        us = timed(torch, lambda i: comp.comp_reduce(comp.FLOAT32, comp.SUM, sets[i % 8][1], n1, sets[i % 8][0]), 64, 16)
+        add("C1 fp32 sum, 2 inputs in place, 64 MiB", us, 3 * n1 * 4, f"8 rotating buffer sets; {comp.last_kernel()}")
+        del sets
     # ---- C2
-    n2 = 33_554_432
-    sets = [[torch.empty(n2, dtype=torch.bfloat16, device="cuda").normal_(0, 1) for _ in range(8)] for _ in range(6)]
-    outs = [torch.empty_like(s[0]) for s in sets]
+    if want("c2"):
+        n2 = 33_554_432
+        sets = [[torch.empty(n2, dtype=torch.bfloat16, device="cuda").normal_(0, 1) for _ in range(8)] for _ in range(6)]
+        outs = [torch.empty_like(s[0]) for s in sets]
 
-    def c2_once():
-        comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, sets[0], outs[0], n2, lp_mode=comp.LP_KEEP_PRECISION)
-        return outs[0]
-    verify_reduce("C2", O.BFLOAT16, O.SUM, sets[0], c2_once, n2, keep=1)
-    us = timed(torch, lambda i: comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, sets[i % 6], outs[i % 6], n2,
-                                                  lp_mode=comp.LP_KEEP_PRECISION), 64, 16)
-    add("C2 bf16 sum, 8 inputs, 64 MiB (fp32 acc, RNE once)", us, 9 * n2 * 2, f"6 rotating buffer sets; {comp.last_kernel()}")
-    us = timed(torch, lambda i: comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, sets[0], outs[0], n2,
-                                                  lp_mode=comp.LP_KEEP_PRECISION), 64, 16)
-    add("C2 same, one buffer set (Infinity Cache assisted)", us, 9 * n2 * 2, "")
-    del sets, outs
+        def c2_once():
+            comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, sets[0], outs[0], n2, lp_mode=comp.LP_KEEP_PRECISION)
+            return outs[0]
+        verify_reduce("C2", O.BFLOAT16, O.SUM, sets[0], c2_once, n2, keep=1)
+        us = timed(torch, lambda i: comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, sets[i % 6], outs[i % 6], n2,
+                                                      lp_mode=comp.LP_KEEP_PRECISION), 64, 16)
+        add("C2 bf16 sum, 8 inputs, 64 MiB (fp32 acc, RNE once)", us, 9 * n2 * 2, f"6 rotating buffer sets; {comp.last_kernel()}")
+        us = timed(torch, lambda i: comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, sets[0], outs[0], n2,
+                                                      lp_mode=comp.LP_KEEP_PRECISION), 64, 16)
+        add("C2 same, one buffer set (Infinity Cache assisted)", us, 9 * n2 * 2, "")
+        del sets, outs
 
     c3_cases = [("int8 sum", comp.INT8, comp.SUM, torch.int8, 1), ("int32 sum", comp.INT32, comp.SUM, torch.int32, 4),
                 ("int64 max", comp.INT64, comp.MAX, torch.int64, 8), ("fp16 sum", comp.FLOAT16, comp.SUM, torch.float16, 2),
@@ -140,9 +153,9 @@ def main():
         return lambda: torch.randint(info.min, info.max, (cnt,), dtype=tdt, device="cuda")
 
     # ---- C3
-    if "c3" not in args.skip:
+    if want("c3"):
         for label, dt, op, tdt, esz in c3_cases:
-            for k in range(11):
+            for k in c3_k:
                 size = 1024 * 4 ** k
                 cnt = size // esz
                 nsets = max(1, min(8, (1 << 30) // (5 * size)))
@@ -159,7 +172,7 @@ def main():
                 add(f"C3 {label}, 4 inputs, {size >> 10} KiB per buffer", us, 5 * size, f"{nsets} set(s)")
                 del ss, oo
     # ---- C3's small sizes as 64 independent jobs: one call each against one batched call
-    if "batch" not in args.skip:
+    if want("batch"):
         for label, dt, op, tdt, esz in c3_cases:
             for k in range(7):
                 size = 1024 * 4 ** k
@@ -184,7 +197,7 @@ def main():
                     f"{us_batch / 64:.2f} us per job; as 64 calls through this binding {us_calls / 64:.2f} us per job")
                 del jobs_in, jobs_out, jobs
     # ---- every datatype x op at 512 MiB per buffer, 8 and 4 inputs: is any of them bound by arithmetic?
-    if "types" not in args.skip:
+    if want("types"):
         size = 512 << 20
         tcases = [("int8", comp.INT8, torch.int8, None), ("int16", comp.INT16, torch.int16, None),
                   ("int32", comp.INT32, torch.int32, None), ("int64", comp.INT64, torch.int64, None),
@@ -238,7 +251,7 @@ def main():
         checked[0] += 1
 
     # ---- buffers at different offsets from a 16-byte boundary
-    if "align" not in args.skip:
+    if want("align"):
         na = 33_554_432
         sets = [[torch.empty(na + 64, dtype=torch.bfloat16, device="cuda").normal_(0, 1) for _ in range(9)] for _ in range(6)]
         for label, shifts in (("all aligned", [0] * 9), ("every input at its own alignment", [1, 2, 3, 4, 5, 6, 7, 0, 0]),
@@ -281,7 +294,7 @@ def main():
             plan.close()
             del tens, outs, fb, peers
     # ---- copies and converters
-    if "copy" not in args.skip:
+    if want("copy"):
         for mib in (64, 512, 3072):
             nb = mib << 20
             nsets = 4 if mib == 64 else 1
@@ -333,61 +346,62 @@ def main():
         add("convert fp16 -> fp32, 2^28 elements", us, 6 * nc)
         del f16, f32, f32b, b16
     # ---- C4
-    rng = np.random.default_rng(4)
-    counts = [int(round(math.exp(rng.uniform(math.log(2048), math.log(2_097_152))))) for _ in range(256)]
-    payload = sum(counts) * 2
-    plan = comp.FusionPlan(counts, comp.BFLOAT16, 256)
-    nelem = plan.nbytes // 2
-    tens = [torch.empty(c, dtype=torch.bfloat16, device="cuda").normal_(0, 0.02) for c in counts]
-    outs = [torch.zeros_like(t) for t in tens]
-    fb = torch.zeros(nelem, dtype=torch.bfloat16, device="cuda")
-    peers = [torch.empty(nelem, dtype=torch.bfloat16, device="cuda").normal_(0, 0.02) for _ in range(7)]
-    plan.pack(tens, fb)
-    torch.cuda.synchronize()
-    verify_fusion("C4 pack", plan, counts, 256, tens, None, fb_after_pack=fb, mode="pack")
-    us_pack = timed(torch, lambda i: plan.pack(tens, fb), 50, 10)
-    fb2 = torch.empty_like(fb)
-
-    def c4_reduce_once():
-        comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, [fb] + peers, fb2, nelem, lp_mode=comp.LP_KEEP_PRECISION)
-        return fb2
-    verify_reduce("C4 reduce over the fusion buffer", O.BFLOAT16, O.SUM, [fb] + peers, c4_reduce_once, nelem, keep=1)
-    us_red = timed(torch, lambda i: comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, [fb] + peers, fb2, nelem,
-                                                      lp_mode=comp.LP_KEEP_PRECISION), 50, 10)
-    plan.unpack(fb2, outs)
-    torch.cuda.synchronize()
-    verify_fusion("C4 pack + reduce + unpack", plan, counts, 256, tens, peers, outs_after=outs)
-    us_unpack = timed(torch, lambda i: plan.unpack(fb2, outs), 50, 10)
-
-    def three(i):
+    if want("c4"):
+        rng = np.random.default_rng(4)
+        counts = [int(round(math.exp(rng.uniform(math.log(2048), math.log(2_097_152))))) for _ in range(256)]
+        payload = sum(counts) * 2
+        plan = comp.FusionPlan(counts, comp.BFLOAT16, 256)
+        nelem = plan.nbytes // 2
+        tens = [torch.empty(c, dtype=torch.bfloat16, device="cuda").normal_(0, 0.02) for c in counts]
+        outs = [torch.zeros_like(t) for t in tens]
+        fb = torch.zeros(nelem, dtype=torch.bfloat16, device="cuda")
+        peers = [torch.empty(nelem, dtype=torch.bfloat16, device="cuda").normal_(0, 0.02) for _ in range(7)]
         plan.pack(tens, fb)
-        comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, [fb] + peers, fb, nelem, lp_mode=comp.LP_KEEP_PRECISION)
-        plan.unpack(fb, outs)
-    for o_ in outs:
-        o_.zero_()
-    three(0)
-    torch.cuda.synchronize()
-    verify_fusion("C4 three launches", plan, counts, 256, tens, peers, outs_after=outs)
-    us_three = timed(torch, three, 50, 10)
-    for o_ in outs:
-        o_.zero_()
-    plan.reduce(comp.SUM, tens, peers, outs, lp_mode=comp.LP_KEEP_PRECISION)
-    torch.cuda.synchronize()
-    verify_fusion("C4 fused", plan, counts, 256, tens, peers, outs_after=outs)
-    fused_kernel = comp.last_kernel()
-    us_fused = timed(torch, lambda i: plan.reduce(comp.SUM, tens, peers, outs, lp_mode=comp.LP_KEEP_PRECISION), 50, 10)
-    add(f"C4 pack, 256 tensors, payload {payload:,} B", us_pack, 2 * payload)
-    add("C4 8-input reduce over the fusion buffer", us_red, 9 * payload)
-    add("C4 unpack", us_unpack, 2 * payload)
-    add("C4 pack + reduce + unpack (3 launches)", us_three, 13 * payload)
-    add("C4 fused single pass (tensors + 7 peers -> tensors)", us_fused, 9 * payload,
-        f"{us_three / us_fused:.2f}x faster than the 3-step sequence; {fused_kernel}")
-    plan.close()
+        torch.cuda.synchronize()
+        verify_fusion("C4 pack", plan, counts, 256, tens, None, fb_after_pack=fb, mode="pack")
+        us_pack = timed(torch, lambda i: plan.pack(tens, fb), 50, 10)
+        fb2 = torch.empty_like(fb)
+
+        def c4_reduce_once():
+            comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, [fb] + peers, fb2, nelem, lp_mode=comp.LP_KEEP_PRECISION)
+            return fb2
+        verify_reduce("C4 reduce over the fusion buffer", O.BFLOAT16, O.SUM, [fb] + peers, c4_reduce_once, nelem, keep=1)
+        us_red = timed(torch, lambda i: comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, [fb] + peers, fb2, nelem,
+                                                          lp_mode=comp.LP_KEEP_PRECISION), 50, 10)
+        plan.unpack(fb2, outs)
+        torch.cuda.synchronize()
+        verify_fusion("C4 pack + reduce + unpack", plan, counts, 256, tens, peers, outs_after=outs)
+        us_unpack = timed(torch, lambda i: plan.unpack(fb2, outs), 50, 10)
+
+        def three(i):
+            plan.pack(tens, fb)
+            comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, [fb] + peers, fb, nelem, lp_mode=comp.LP_KEEP_PRECISION)
+            plan.unpack(fb, outs)
+        for o_ in outs:
+            o_.zero_()
+        three(0)
+        torch.cuda.synchronize()
+        verify_fusion("C4 three launches", plan, counts, 256, tens, peers, outs_after=outs)
+        us_three = timed(torch, three, 50, 10)
+        for o_ in outs:
+            o_.zero_()
+        plan.reduce(comp.SUM, tens, peers, outs, lp_mode=comp.LP_KEEP_PRECISION)
+        torch.cuda.synchronize()
+        verify_fusion("C4 fused", plan, counts, 256, tens, peers, outs_after=outs)
+        fused_kernel = comp.last_kernel()
+        us_fused = timed(torch, lambda i: plan.reduce(comp.SUM, tens, peers, outs, lp_mode=comp.LP_KEEP_PRECISION), 50, 10)
+        add(f"C4 pack, 256 tensors, payload {payload:,} B", us_pack, 2 * payload)
+        add("C4 8-input reduce over the fusion buffer", us_red, 9 * payload)
+        add("C4 unpack", us_unpack, 2 * payload)
+        add("C4 pack + reduce + unpack (3 launches)", us_three, 13 * payload)
+        add("C4 fused single pass (tensors + 7 peers -> tensors)", us_fused, 9 * payload,
+            f"{us_three / us_fused:.2f}x faster than the 3-step sequence; {fused_kernel}")
+        plan.close()
 
     # small-message latency from C++ (no Python in the loop); the program checks its own results
     lat = os.path.join(ROOT, "tests", "cpp", "bench_latency")
     lat_lines = []
-    if os.path.exists(lat):
+    if want("latency") and os.path.exists(lat):
         import subprocess
         pr = subprocess.run([lat], capture_output=True, text=True, timeout=300)
         if pr.returncode != 0:

@@ -7,6 +7,7 @@
 
 #include "../../include/mi_ccl_comp.h"
 #include "fusion_kernels.hpp"
+#include "launch_geometry.hpp"
 
 namespace mi {
 
@@ -49,21 +50,43 @@ static size_t fusion_dtype_size(int dtype) {
     return (dtype >= 0 && dtype < MI_CCL_DATATYPE_LAST) ? sz[dtype] : 0;
 }
 
+// Pack and unpack.  A block copies one 4 KiB quarter of a work item with one vector per lane -- a wave issues one load
+// and one store and ends, the shape in which writes run fastest (as in copy_kernel) -- and the four blocks of an item
+// read the same descriptor.  Only one pointer table travels with the launch (the tensors; the fusion buffer is one
+// pointer), so it holds kFusionCopyGroup tensors: the 256 tensors of a typical bucket are one launch.  Measured on the
+// 256-tensor configuration (191 MB of payload): 61.8 us against 68.4 us for 16 KiB per block in two launches, and
+// 58.3 us for a plain copy of as many bytes.
+constexpr int kFusionCopyGroup = 448;
+constexpr uint32_t kFusionCopySub = 4096;         // bytes per block
+static_assert(kFusionChunk % kFusionCopySub == 0 && kFusionCopySub == 16 * kBlock, "an item is a whole number of block-sized quarters");
+struct FusionCopyPtrs {
+    const void* p[kFusionCopyGroup];
+};
+
 // to_fusion != 0: tensors -> fusion buffer (pack); else fusion buffer -> tensors (unpack)
 __global__ void __launch_bounds__(kBlock)
-fusion_copy_kernel(FusionPtrs tensors, unsigned char* fusion_buf, const uint64_t* off, const uint64_t* bytes,
-                   const FusionItem* items, uint32_t nitems, uint32_t t0, int to_fusion) {
-    for (uint32_t it = blockIdx.x; it < nitems; it += gridDim.x) {
-        const FusionItem w = items[it];
-        const uint64_t lo = (uint64_t)w.c * kFusionChunk;
-        const uint64_t left = bytes[w.t] - lo;
-        const uint32_t n = left < kFusionChunk ? (uint32_t)left : kFusionChunk;
-        unsigned char* tp = (unsigned char*)tensors.p[w.t - t0] + lo;
-        unsigned char* fp = fusion_buf + off[w.t] + lo;
-        if (to_fusion)
-            copy_span(tp, fp, n);
-        else
-            copy_span(fp, tp, n);
+fusion_copy_kernel(FusionCopyPtrs tensors, unsigned char* fusion_buf, const uint64_t* off, const uint64_t* bytes,
+                   const FusionItem* items, uint32_t t0, int to_fusion) {
+    constexpr uint32_t kSubs = kFusionChunk / kFusionCopySub;
+    const uint32_t tid = threadIdx.x;
+    const FusionItem w = items[blockIdx.x / kSubs];
+    const uint64_t lo = (uint64_t)w.c * kFusionChunk + (blockIdx.x % kSubs) * kFusionCopySub;
+    const uint64_t total = bytes[w.t];
+    if (lo >= total) return;                        // the item's last quarters may be empty
+    const uint64_t left = total - lo;
+    const uint32_t n = left < kFusionCopySub ? (uint32_t)left : kFusionCopySub;
+    unsigned char* tp = (unsigned char*)tensors.p[w.t - t0] + lo;
+    unsigned char* fp = fusion_buf + off[w.t] + lo;
+    const unsigned char* src = to_fusion ? tp : fp;
+    unsigned char* dst = to_fusion ? fp : tp;
+    // vectors from the destination's first 16-byte boundary on, whatever the source's alignment is
+    uint32_t head = (uint32_t)(-(intptr_t)dst) & 15u;
+    if (head > n) head = n;
+    const uint32_t nvec = (n - head) >> 4, tail = n - head - (nvec << 4);
+    if (tid < nvec) st_loose((u32x4_u*)(dst + head) + tid, ld_loose((const u32x4_u*)(src + head) + tid));
+    if (tid < head + tail) {
+        const uint32_t i = (tid < head) ? tid : head + (nvec << 4) + (tid - head);
+        dst[i] = src[i];
     }
 }
 
@@ -272,22 +295,22 @@ static int fusion_copy(mi_ccl_fusion_plan* plan, const void* const* tensors, voi
     for (size_t t = 0; t < plan->k; t++)
         if (!tensors[t] && plan->counts[t])
             return MI_CCL_INVALID_ARGUMENTS;
-    Tuning tune = current_tuning();
-    for (size_t t0 = 0; t0 < plan->k; t0 += kFusionGroup) {
-        const size_t t1 = (t0 + kFusionGroup < plan->k) ? t0 + kFusionGroup : plan->k;
-        const uint64_t i0 = plan->item_begin[t0], i1 = plan->item_begin[t1];
-        if (i1 == i0)
-            continue;
-        FusionPtrs ptrs;
+    constexpr uint32_t kSubs = kFusionChunk / kFusionCopySub;
+    const uint64_t max_items = hip_block_limit(kBlock) / kSubs;       // items one launch may take
+    for (size_t t0 = 0; t0 < plan->k; t0 += kFusionCopyGroup) {
+        const size_t t1 = (t0 + kFusionCopyGroup < plan->k) ? t0 + kFusionCopyGroup : plan->k;
+        FusionCopyPtrs ptrs;
         for (size_t t = t0; t < t1; t++) ptrs.p[t - t0] = tensors[t];
-        int grid = grid_for(i1 - i0, tune);
-        g_last_kernel = "fusion_copy_kernel";
-        hipLaunchKernelGGL(fusion_copy_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ptrs,
-                           (unsigned char*)fusion_buf, plan->d_off, plan->d_bytes, plan->d_items + i0,
-                           (uint32_t)(i1 - i0), (uint32_t)t0, to_fusion);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess)
-            return fusion_status_of(e);
+        for (uint64_t i0 = plan->item_begin[t0]; i0 < plan->item_begin[t1]; i0 += max_items) {
+            const uint64_t i1 = (i0 + max_items < plan->item_begin[t1]) ? i0 + max_items : plan->item_begin[t1];
+            g_last_kernel = "fusion_copy_kernel";
+            hipLaunchKernelGGL(fusion_copy_kernel, dim3((unsigned)((i1 - i0) * kSubs)), dim3(kBlock), 0, (hipStream_t)stream,
+                               ptrs, (unsigned char*)fusion_buf, plan->d_off, plan->d_bytes, plan->d_items + i0, (uint32_t)t0,
+                               to_fusion);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess)
+                return fusion_status_of(e);
+        }
     }
     return MI_CCL_SUCCESS;
 }

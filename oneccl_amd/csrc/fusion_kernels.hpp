@@ -3,9 +3,10 @@
 // (src/fusion/fusion.cpp:283-362): tensor t lives at fusion_buf + off[t]; off is a running byte offset,
 // optionally rounded up to an alignment.
 //
-// Work is cut into items of kFusionChunk bytes of one tensor; a block takes items grid-stride.  The item
-// list and the per-tensor offset/size tables live in device memory owned by the plan; the tensor pointers
-// of a call travel as kernel arguments, kFusionGroup tensors per launch.
+// Work is cut into items of kFusionChunk bytes of one tensor; a block of the fused reduce takes items grid-stride
+// (a block of pack / unpack takes a quarter of one item).  The item list and the per-tensor offset/size tables live in
+// device memory owned by the plan; the tensor pointers of a call travel as kernel arguments: kFusionGroup tensors
+// per launch of the fused reduce (two tables: inputs and outputs), more for pack and unpack (one table).
 #pragma once
 
 #include "reduce_kernels.hpp"
@@ -41,28 +42,6 @@ struct FusionLaunchArgs {
     hipStream_t stream;
     Tuning tune;
 };
-
-// Copy n <= kFusionChunk bytes with one block: vectors from the destination's first 16-byte boundary on, whatever
-// the source's alignment is.
-__device__ __forceinline__ void copy_span(const unsigned char* src, unsigned char* dst, uint32_t n) {
-    const uint32_t tid = threadIdx.x;
-    uint32_t head = (uint32_t)(-(intptr_t)dst) & 15u;
-    if (head > n) head = n;
-    const uint32_t nvec = (n - head) >> 4, tail = n - head - (nvec << 4);
-    const u32x4_u* s = (const u32x4_u*)(src + head);
-    u32x4_u* o = (u32x4_u*)(dst + head);
-    u32x4 x[4];
-#pragma unroll
-    for (int u = 0; u < 4; u++)
-        if (tid + u * kBlock < nvec) x[u] = ld_loose(s + tid + u * kBlock);
-#pragma unroll
-    for (int u = 0; u < 4; u++)
-        if (tid + u * kBlock < nvec) st_loose(o + tid + u * kBlock, x[u]);
-    if (tid < head + tail) {
-        uint32_t i = (tid < head) ? tid : head + (nvec << 4) + (tid - head);
-        dst[i] = src[i];
-    }
-}
 
 // Elements of a tensor chunk before its output's first 16-byte boundary, where its vectors start (none when the
 // output is not even aligned to its element size).  Inputs that disagree with the output modulo 16 bytes -- the peers'
