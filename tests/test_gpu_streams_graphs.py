@@ -173,3 +173,94 @@ def test_worker_threads_on_disjoint_partitions(comp, variant):
     torch.cuda.synchronize()
     assert not errors, errors
     assert (to_host(out, np.uint16) == want).all()
+
+
+def test_graph_of_batched_reduce_and_allocation_free_fused_reduce(comp):
+    """The two entry points meant for callers that hold a graph: mi_ccl_comp_reduce_batch (its job table travels in the
+    kernel arguments) and mi_ccl_fusion_reduce_static (its table is rebuilt by a kernel in front of the reduce, no
+    allocation, no memset) captured together, replayed four times with eager calls of the same entry points -- which
+    share the static table -- in between; every replay equals the oracle."""
+    import torch
+    rng = np.random.default_rng(11)
+    counts = [70_001, 1, 4096, 300_000, 33]
+    np_t = np.float32
+    jobs_h = [[rng.uniform(-2, 2, c).astype(np_t) for _ in range(3)] for c in counts]
+    jobs_d = [[to_dev(x) for x in j] for j in jobs_h]
+    jobs_o = [torch.zeros(c, dtype=torch.float32, device="cuda") for c in counts]
+    table = comp.BatchJobs([(s, o, c) for s, o, c in zip(jobs_d, jobs_o, counts)])
+    want_jobs = [O.reduce_n(j, O.FLOAT32, O.MAX) for j in jobs_h]
+    offs, total = O.fusion_offsets(counts, 4, 64)
+    nelem = total // 4
+    peers_h = [rng.uniform(-2, 2, nelem).astype(np_t) for _ in range(3)]
+    peers_d = [to_dev(p_) for p_ in peers_h]
+    fused_o = [torch.zeros(c, dtype=torch.float32, device="cuda") for c in counts]
+    want_fused = []
+    for i, c in enumerate(counts):
+        o = int(offs[i]) // 4
+        want_fused.append(O.reduce_n([jobs_h[i][0]] + [p_[o:o + c] for p_ in peers_h], O.FLOAT32, O.SUM))
+    own = [j[0] for j in jobs_d]
+
+    def both():
+        table.reduce(comp.FLOAT32, comp.MAX)
+        comp.fusion_reduce_static(counts, comp.FLOAT32, 64, comp.SUM, own, peers_d, fused_o)
+
+    def check(what):
+        torch.cuda.synchronize()
+        for i in range(len(counts)):
+            assert (to_host(jobs_o[i], np.uint32) == want_jobs[i].view(np.uint32)).all(), f"{what}: job {i}"
+            assert (to_host(fused_o[i], np.uint32) == want_fused[i].view(np.uint32)).all(), f"{what}: fused tensor {i}"
+
+    both()                                  # eager first: the first call on a device looks the static table up
+    check("eager")
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        both()
+    other_counts = [5, 100_000]             # an eager call with another layout overwrites the shared table
+    other = [to_dev(rng.uniform(-1, 1, c).astype(np_t)) for c in other_counts]
+    other_o = [torch.zeros_like(t) for t in other]
+    for rep in range(4):
+        for t in jobs_o + fused_o:
+            t.zero_()
+        comp.fusion_reduce_static(other_counts, comp.FLOAT32, 4, comp.SUM, other, [], other_o)
+        torch.cuda.synchronize()
+        g.replay()
+        check(f"replay {rep}")
+
+
+def test_two_threads_with_different_fp16_implementations(comp):
+    """The float16 implementation travels with the call: two host threads, one reducing under avx512f (a signalling
+    NaN that min hands back is quieted) and one under avx512fp16 (it stays as it is), each on its own stream, never
+    see the other's setting, and the process-wide default is left alone."""
+    import threading
+    import torch
+    snan, one = np.uint16(0x7D01), np.uint16(0x3C00)
+    count = 10_007
+    a = np.full(count, one, np.uint16)          # in
+    b = np.full(count, snan, np.uint16)         # inout: min(in = 1, inout = sNaN) hands inout back
+    want = {3: O.comp_reduce(a, b, O.FLOAT16, O.MIN, fp16_impl=3), 4: O.comp_reduce(a, b, O.FLOAT16, O.MIN, fp16_impl=4)}
+    assert want[3][0] == 0x7F01 and want[4][0] == 0x7D01
+    errors = []
+
+    def worker(impl):
+        try:
+            stream = torch.cuda.Stream()
+            da = to_dev(a)
+            for rep in range(200):
+                db = to_dev(b)
+                comp.comp_reduce(comp.FLOAT16, comp.MIN, da, count, db, fp16_impl=impl, stream=stream)
+                stream.synchronize()
+                got = to_host(db, np.uint16)
+                if not (got == want[impl]).all():
+                    errors.append((impl, rep, hex(int(got[0]))))
+                    return
+        except Exception as e:      # noqa: BLE001
+            errors.append((impl, repr(e)))
+
+    default_before = comp.get_param("fp16_impl")
+    threads = [threading.Thread(target=worker, args=(impl,)) for impl in (3, 4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert comp.get_param("fp16_impl") == default_before
