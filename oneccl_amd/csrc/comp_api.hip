@@ -60,10 +60,16 @@ static uint64_t block_limit() {
 }
 static std::atomic<int> g_num_cus[64];
 
-// Barrier words of the phased kernel: one copy per device (each GPU holds its own instance of a
-// __device__ variable at its own address), looked up once per device.
-static __device__ PhaseSync g_phase_sync;
+// Barrier words of the phased kernels: kPhaseSlots sets per device (each GPU holds its own instance of a __device__
+// variable at its own address, looked up once per device).  Every call takes the next set in turn, so that launches
+// which overlap on one GPU (different streams) do not count each other's arrivals: with one shared set two
+// overlapping launches lose their phase alignment and run at the unaligned speed, about a quarter slower.  (A set
+// comes round again after kPhaseSlots calls; launches that far apart and still overlapping share it, which costs
+// speed only, never correctness.)
+constexpr int kPhaseSlots = 16;
+static __device__ PhaseSync g_phase_sync[kPhaseSlots];
 static std::atomic<PhaseSync*> g_phase_sync_ptr[64];
+static std::atomic<unsigned> g_phase_sync_next[64];
 
 static PhaseSync* phase_sync() {
     int dev = 0;
@@ -77,7 +83,7 @@ static PhaseSync* phase_sync() {
         p = (PhaseSync*)sym;
         g_phase_sync_ptr[dev].store(p, std::memory_order_release);
     }
-    return p;
+    return p + g_phase_sync_next[dev].fetch_add(1, std::memory_order_relaxed) % kPhaseSlots;
 }
 
 static int num_cus() {

@@ -44,7 +44,7 @@ struct Tuning {
     int variant;        // 0 = automatic; 1, 2, 4 = streaming kernel (with that unroll depth where compiled); 8 = phased kernel
     int num_cus;
     long phased_min_bytes;   // automatic choice: phased kernel when (N + 1) * bytes per buffer reaches this
-    struct PhaseSync* sync;  // device-resident barrier words of the current device (may be null)
+    struct PhaseSync* sync;  // the set of device-resident barrier words this call uses (may be null)
     int fp16_impl;           // which CPU implementation's float16 results to reproduce: 2, 3 (through fp32) or 4 (native)
 };
 

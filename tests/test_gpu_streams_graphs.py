@@ -42,7 +42,7 @@ def test_graph_capture_and_replay(comp, variant):
             g.replay()
             torch.cuda.synchronize()
             assert (to_host(out, np.uint16) == want).all(), f"replay {rep}"
-            # an eager launch between replays shares the barrier words with the captured one
+            # an eager launch between replays (it may land on the captured launch's set of barrier words)
             comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, d, out, count, lp_mode=comp.LP_KEEP_PRECISION)
             torch.cuda.synchronize()
             assert (to_host(out, np.uint16) == want).all()
@@ -136,7 +136,7 @@ def test_two_phased_reduces_overlapping_on_two_streams(comp):
 def test_worker_threads_on_disjoint_partitions(comp, variant):
     """What CCL_WORKER_COUNT = W does (parallelizer.cpp:230-241,374-379): W host threads, each with a stream of its
     own, reduce disjoint count/W partitions of the same buffers at the same time through the C ABI.  The result is
-    the one-call result, bit for bit; variant 8 makes every partition a phased launch, so the launches share the
+    the one-call result, bit for bit; variant 8 makes every partition a phased launch, each with its own set of
     barrier words while they overlap."""
     import threading
     import torch
