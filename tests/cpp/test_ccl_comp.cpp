@@ -5,6 +5,7 @@
 // bit for bit against the CPU oracle.  Exit status 0 = all checks passed.
 #include <hip/hip_runtime.h>
 #include <math.h>
+#include <stdint.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -493,6 +494,34 @@ int main() {
                     }
                 }
             }
+        }
+        // another element type and operation: int32 max with a pair stage, three inputs, a chunk of 4,000 elements
+        {
+            const size_t count = 100003;
+            std::vector<std::vector<int32_t>> hl(3, std::vector<int32_t>(count)), hp(3, std::vector<int32_t>(count));
+            uint32_t x = 99;
+            for (int i = 0; i < 3; i++)
+                for (size_t e = 0; e < count; e++) {
+                    x = x * 1664525u + 1013904223u; hl[i][e] = (int32_t)x;
+                    x = x * 1664525u + 1013904223u; hp[i][e] = (int32_t)x;
+                }
+            std::vector<std::unique_ptr<DevBuf<int32_t>>> dl, dp;
+            std::vector<const void*> local, pair;
+            for (int i = 0; i < 3; i++) {
+                dl.emplace_back(new DevBuf<int32_t>(hl[i])); dp.emplace_back(new DevBuf<int32_t>(hp[i]));
+                local.push_back(dl[i]->p); pair.push_back(dp[i]->p);
+            }
+            std::vector<int32_t> want(count);
+            for (size_t e = 0; e < count; e++) {
+                int32_t m = INT32_MIN;
+                for (int i = 0; i < 3; i++) { m = hl[i][e] > m ? hl[i][e] : m; m = hp[i][e] > m ? hp[i][e] : m; }
+                want[e] = m;
+            }
+            ccl_chunked_reducer red(16000, 3);
+            DevBuf<int32_t> out(count);
+            red.run(&sched, local, pair, count, out.p, DT(ccl::datatype::int32), ccl::reduction::max);
+            EXPECT(out.host() == want, "chunked int32 max with a pair stage");
+            EXPECT(red.chunks_of_last_run() == 26, "26 chunks of 4,000 elements");
         }
         bool threw = false;
         try { ccl_chunked_reducer bad(1000, 4); } catch (const ccl::exception&) { threw = true; }

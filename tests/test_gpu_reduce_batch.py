@@ -81,6 +81,14 @@ def test_job_counts_and_mixed_sizes(comp, n_jobs):
         _run(comp, rng, O.BFLOAT16, O.SUM, 8, counts, lp=comp.LP_KEEP_PRECISION, keep=1)
 
 
+def test_more_jobs_than_one_table_holds_with_eight_inputs(comp):
+    """Eight inputs per job leave room for 35 jobs per launch (320 pointers): 100 jobs take three launches."""
+    rng = np.random.default_rng(7150)
+    counts = [int(c) for c in rng.integers(0, 40_000, 100)]
+    _run(comp, rng, O.FLOAT16, O.PROD, 8, counts)
+    _run(comp, rng, O.INT64, O.MIN, 8, counts, in_place_every=2)
+
+
 def test_sixteen_bit_modes_and_nan_patterns(comp):
     rng = np.random.default_rng(7200)
     counts = [33, 8191, 1, 100_003, 16]
