@@ -143,7 +143,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
     const uint32_t lane = tid & 63u;
     bool give_up = false;
     unsigned gen = 0;
-    if (tid == 0) gen = MI_ALOAD(&ps->rel.v);
+    if (tid == 0) gen = phase_generation(ps);
     const uint64_t per_phase = (uint64_t)SLOTS * gridDim.x;
     for (uint64_t p0 = 0; p0 < nitems; p0 += per_phase) {
         // Lane k of every wave fetches the descriptor of this block's k-th item of the phase, so that the chain
