@@ -237,7 +237,11 @@ const char* mi_ccl_last_kernel(void);
  * kernels with that many vectors per lane where a type has them; 8 = the phased kernels at any size; a non-zero value
  * also keeps one-input calls on the general reduce kernels instead of the copy and broadcast kernels -- for tests and
  * measurements),
- * "phased_min_bytes" (scales the sizes from which the phased kernels are used; default 160 MB), "num_cus" (read
+ * "phased_min_bytes" (scales the sizes from which the phased kernels are used; default 160 MB),
+ * "phase_early_loads" / "phase_early_stores" (phased kernels: how many 16-byte loads / stores per lane a block still
+ * has to issue when it reports the end of its read / write phase to the chip-wide barrier, which hides the barrier's
+ * latency; defaults 12 and -1 = chosen per element type, 4 or 16; 0 = report when done; timing only, results do not
+ * depend on them), "num_cus" (read
  * only), "fp16_impl" (what MI_CCL_FP16_DEFAULT stands for: 2, 3 or 4 of enum mi_ccl_fp16_impl above), and
  * "launch_block_limit" (blocks per launch of the copy, broadcast and converter kernels, which cut larger work into
  * several launches; 0 = what HIP allows, 2^24 - 1; smaller values let tests exercise the cutting).

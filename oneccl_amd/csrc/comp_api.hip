@@ -49,6 +49,8 @@ static std::atomic<int> g_max_blocks{ 0 };
 static std::atomic<int> g_xcd_chunked{ 0 };
 static std::atomic<int> g_variant{ 0 };
 static std::atomic<long> g_phased_min_bytes{ 160L << 20 };
+static std::atomic<int> g_phase_early_loads{ 12 };
+static std::atomic<int> g_phase_early_stores{ -1 };
 static std::atomic<int> g_fp16_impl{ MI_CCL_FP16_AVX512F };
 static std::atomic<long> g_launch_block_limit{ 0 };     // 0: what HIP allows; smaller values are for tests of the splitting
 static_assert(kGeomBlock == kBlock, "the geometry header and the kernels agree on the block size");
@@ -108,6 +110,8 @@ Tuning current_tuning() {
     t.num_cus = num_cus();
     t.phased_min_bytes = g_phased_min_bytes.load(std::memory_order_relaxed);
     t.sync = phase_sync();
+    t.early_loads = g_phase_early_loads.load(std::memory_order_relaxed);
+    t.early_stores = g_phase_early_stores.load(std::memory_order_relaxed);
     t.fp16_impl = g_fp16_impl.load(std::memory_order_relaxed);
     return t;
 }
@@ -816,6 +820,14 @@ int mi_ccl_set_param(const char* name, long value) {
         g_phased_min_bytes.store(value);
         return MI_CCL_SUCCESS;
     }
+    if (!strcmp(name, "phase_early_loads") && value >= 0 && value <= 4096) {
+        g_phase_early_loads.store((int)value);
+        return MI_CCL_SUCCESS;
+    }
+    if (!strcmp(name, "phase_early_stores") && value >= -1 && value <= kPhaseU) {
+        g_phase_early_stores.store((int)value);
+        return MI_CCL_SUCCESS;
+    }
     if (!strcmp(name, "fp16_impl") && value >= MI_CCL_FP16_F16C && value <= MI_CCL_FP16_AVX512FP16) {
         g_fp16_impl.store((int)value);
         return MI_CCL_SUCCESS;
@@ -840,6 +852,10 @@ long mi_ccl_get_param(const char* name) {
         return g_variant.load();
     if (!strcmp(name, "phased_min_bytes"))
         return g_phased_min_bytes.load();
+    if (!strcmp(name, "phase_early_loads"))
+        return g_phase_early_loads.load();
+    if (!strcmp(name, "phase_early_stores"))
+        return g_phase_early_stores.load();
     if (!strcmp(name, "fp16_impl"))
         return g_fp16_impl.load();
     if (!strcmp(name, "launch_block_limit"))

@@ -126,7 +126,8 @@ struct FusionPhaseRegs {
 template <class TR, int OP, int NT>
 __global__ void __launch_bounds__(kPhaseBlock)
 fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, const uint64_t* off, const uint64_t* bytes,
-                            const FusionItem* items, uint32_t nitems, uint32_t t0, PhaseSync* ps) {
+                            const FusionItem* items, uint32_t nitems, uint32_t t0, PhaseSync* ps, int early_loads,
+                            int early_stores) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr uint32_t ES = sizeof(E);
@@ -164,7 +165,18 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                 d_head = fusion_head<ES>((const void*)(uintptr_t)d_o);
             }
         }
+        // The block reports its arrival at the barriers a little before it is done (see phase_arrive): in front of the
+        // slot that leaves early_loads or fewer loads per lane to issue (a slot is two vectors of NT inputs), and in
+        // front of the one that leaves early_stores or fewer stores (two per slot).
+        const int nslots = __popcll(__ballot(d_nb != 0));
+        const int lead_r = early_loads > 0 ? (early_loads >= 2 * NT ? early_loads / (2 * NT) : 1) : 0;
+        const int arrive_r = nslots > lead_r ? nslots - lead_r : 0;
+        bool arrived = false;
         for (int k = 0; k < SLOTS; k++) {
+            if (lead_r > 0 && k == arrive_r) {
+                if (tid == 0) phase_arrive(ps);
+                arrived = true;
+            }
             const uint32_t nb = __shfl(d_nb, k, 64);
             if (nb == 0) break;
             const unsigned char* a = (const unsigned char*)(uintptr_t)__shfl(d_a, k, 64);
@@ -206,8 +218,17 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                 }
             }
         }
-        phase_barrier(ps, ++gen, give_up);
+        if (!arrived && tid == 0) phase_arrive(ps);
+        phase_wait(ps, ++gen, give_up);
+        const bool more = p0 + per_phase < nitems;
+        const int lead_w = early_stores / 2;
+        const int arrive_w = nslots > lead_w ? nslots - lead_w : 0;
+        arrived = false;
         for (int k = 0; k < SLOTS; k++) {
+            if (more && lead_w > 0 && k == arrive_w) {
+                if (tid == 0) phase_arrive(ps);
+                arrived = true;
+            }
             const uint32_t nb = __shfl(d_nb, k, 64);
             if (nb == 0) break;
             unsigned char* o = (unsigned char*)(uintptr_t)__shfl(d_o, k, 64);
@@ -235,7 +256,10 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                 if (tid + kPhaseBlock < nvec) st_loose(d + tid + kPhaseBlock, v1);
             }
         }
-        if (p0 + per_phase < nitems) phase_barrier(ps, ++gen, give_up);
+        if (more) {
+            if (!arrived && tid == 0) phase_arrive(ps);
+            phase_wait(ps, ++gen, give_up);
+        }
     }
 }
 
@@ -245,7 +269,8 @@ inline hipError_t launch_fusion_phased(const FusionLaunchArgs& a, const FusionPt
     int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
     g_last_kernel = "fusion_reduce_phased_kernel";
     hipLaunchKernelGGL((fusion_reduce_phased_kernel<TR, OP, NT>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, own, out, pp,
-                       a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0, a.tune.sync);
+                       a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0, a.tune.sync,
+                       a.tune.early_loads, phase_early_stores<TR>(a.tune));
     return hipGetLastError();
 }
 
@@ -264,11 +289,14 @@ inline hipError_t launch_fusion_op(const FusionLaunchArgs& a) {
             out.p[t - t0] = a.out[t];
         }
         hipError_t e = hipSuccess;
-        // large groups (from 320 MB of traffic by default): separate reads from writes in time (at most 16 KiB of
-        // padding per item is over-counted)
+        // large groups with three or more peers (from 320 MB of traffic by default, 480 MB with three peers): separate
+        // reads from writes in time (at most 16 KiB of padding per item is over-counted).  With one or two peers the
+        // phased form measures 5-25 % below the streaming one at every size (its two vectors of so few inputs are
+        // too few loads in flight per lane), so it is only taken when forced.
         const uint64_t traffic = (uint64_t)(a.n_peers + 2) * (i1 - i0) * kFusionChunk;
+        const uint64_t from = (uint64_t)a.tune.phased_min_bytes * (a.n_peers == 3 ? 3u : 2u);
         const bool phased = a.tune.sync && a.tune.num_cus >= kPhaseGroups && a.n_peers >= 1 && a.n_peers <= 7 &&
-                            (a.tune.variant == 8 || (a.tune.variant == 0 && traffic >= 2 * (uint64_t)a.tune.phased_min_bytes));
+                            (a.tune.variant == 8 || (a.tune.variant == 0 && a.n_peers >= 3 && traffic >= from));
         if (phased) {
             switch (a.n_peers) {
                 case 1: e = launch_fusion_phased<TR, OP, 2>(a, own, out, pp, i0, i1, t0); break;

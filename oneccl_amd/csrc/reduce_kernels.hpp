@@ -43,8 +43,10 @@ struct Tuning {
     int xcd_chunked;    // 1: each XCD streams one contiguous eighth of the buffer
     int variant;        // 0 = automatic; 1, 2, 4 = streaming kernel (with that unroll depth where compiled); 8 = phased kernel
     int num_cus;
-    long phased_min_bytes;   // automatic choice: phased kernel when (N + 1) * bytes per buffer reaches this
+    long phased_min_bytes;   // automatic choice: no phased kernel below this much traffic per launch
     struct PhaseSync* sync;  // the set of device-resident barrier words this call uses (may be null)
+    int early_loads;         // phased kernels: loads per lane still to issue when a block reports the end of its reads
+    int early_stores;        // ... and stores per lane still to issue when it reports the end of its writes (< 0: per type)
     int fp16_impl;           // which CPU implementation's float16 results to reproduce: 2, 3 (through fp32) or 4 (native)
 };
 
@@ -627,34 +629,46 @@ struct PhaseSync {
 #define MI_ALOAD(p) __hip_atomic_load((p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 #define MI_AADD(p, x) __hip_atomic_fetch_add((p), (x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 
-// Every block calls this the same number of times per launch (twice per phase, except after the last phase's
-// writes), so the counters stay multiples of their group sizes from launch to launch.  A barrier is complete when
-// `top` has counted kPhaseGroups complete groups more: the last block of a group bumps `top`, and the waiters poll
-// `top` itself (a third word bumped by the last group measured 0.3 % slower: one more dependent atomic between the
-// last arrival and the release).  gen counts barriers: this block waits for top >= gen * kPhaseGroups.
+// A barrier in two halves.  One thread of every block reports the block's arrival (phase_arrive), every block does so
+// the same number of times per launch (twice per phase, except after the last phase's writes), so the counters stay
+// multiples of their group sizes from launch to launch.  A barrier is complete when `top` has counted kPhaseGroups
+// complete groups more: the last block of a group bumps `top`, and the waiters poll `top` itself (a third word bumped
+// by the last group measured 0.3 % slower: one more dependent atomic between the last arrival and the release; the
+// 16 group words polled directly by 16 lanes 1.2 % slower).  gen counts barriers: a block waits for
+// top >= gen * kPhaseGroups (phase_wait, called by all its threads).
+//
+// The halves are apart on purpose.  From the last arrival to the moment the waiting blocks see the release, two
+// dependent atomics and a poll go to memory and back, about 2 us in which HBM would idle.  So a block reports its
+// arrival a little before it is done: with Tuning::early_loads vector loads per lane of the read phase still to
+// issue, and with Tuning::early_stores stores per lane of the write phase still to issue (its first wave, whose
+// thread 0 reports, has then seen all its earlier stores acknowledged, because the returning atomic waits for
+// them).  The release then reaches the blocks about when the slowest of them finishes.  Measured on 8 x 2 GB bf16:
+// 2.619 ms with arrival at the end of each phase, 2.580 with 4 loads, 2.545 with 8, 2.536 with 12 and 2.540 with 16
+// early loads (4 early stores each; 8 or 12 early stores measure 0.2-0.5 % slower than 4).
 __device__ __forceinline__ unsigned phase_generation(const PhaseSync* ps) {
     return MI_ALOAD(&ps->top.v) / kPhaseGroups;     // at kernel start: the barriers completed so far
 }
-__device__ __forceinline__ void phase_barrier(PhaseSync* ps, unsigned gen, bool& give_up) {
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const unsigned per = gridDim.x / kPhaseGroups;
-        const unsigned old = MI_AADD(&ps->grp[blockIdx.x % kPhaseGroups].v, 1u);
-        if ((old + 1u) % per == 0u) {
-            MI_AADD(&ps->top.v, 1u);
-        }
-        if (!give_up) {
-            const long long t0 = wall_clock64();
-            while ((int)(MI_ALOAD(&ps->top.v) - gen * kPhaseGroups) < 0) {
-                __builtin_amdgcn_s_sleep(1);
-                if (wall_clock64() - t0 > kPhaseSpinTicks) {
-                    give_up = true;
-                    break;
-                }
+__device__ __forceinline__ void phase_arrive(PhaseSync* ps) {
+    const unsigned per = gridDim.x / kPhaseGroups;
+    const unsigned old = MI_AADD(&ps->grp[blockIdx.x % kPhaseGroups].v, 1u);
+    if ((old + 1u) % per == 0u) {
+        MI_AADD(&ps->top.v, 1u);
+    }
+}
+// No data crosses the barrier (a lane only ever reads back the LDS slots it wrote itself), so the waves of a block
+// are held by a bare s_barrier: nothing has to wait for the block's outstanding stores.
+__device__ __forceinline__ void phase_wait(PhaseSync* ps, unsigned gen, bool& give_up) {
+    if (threadIdx.x == 0 && !give_up) {
+        const long long t0 = wall_clock64();
+        while ((int)(MI_ALOAD(&ps->top.v) - gen * kPhaseGroups) < 0) {
+            __builtin_amdgcn_s_sleep(1);
+            if (wall_clock64() - t0 > kPhaseSpinTicks) {
+                give_up = true;
+                break;
             }
         }
     }
-    __syncthreads();
+    __builtin_amdgcn_s_barrier();
 }
 
 // G vectors per lane at once: all G x N loads are issued before the first is used, so that a lane keeps about
@@ -704,7 +718,8 @@ __device__ __forceinline__ void reduce_group_guarded(const u32x4_u* const (&s)[N
 
 template <class TR, int OP, int UNROLL>
 __device__ __forceinline__ void reduce_rt_tile(const SrcTable& src, int n, uint32_t head, const uint64_t (&idx)[UNROLL],
-                                               uint64_t nvec, u32x4 (&out)[UNROLL]) {
+                                               uint64_t nvec, u32x4 (&out)[UNROLL], PhaseSync* arrive_ps = nullptr,
+                                               int arrive_j = 0) {
     typedef typename TR::elem_t E;
     Accs<TR> a[UNROLL];
     const u32x4_u* s0 = (const u32x4_u*)((const unsigned char*)src.p[0] + head * sizeof(E));
@@ -713,6 +728,7 @@ __device__ __forceinline__ void reduce_rt_tile(const SrcTable& src, int n, uint3
     for (int j = 1; j < n; j++) {
         const u32x4_u* sj = (const u32x4_u*)((const unsigned char*)src.p[j] + head * sizeof(E));
         u32x4 x[UNROLL];
+        if (j == arrive_j && threadIdx.x == 0) phase_arrive(arrive_ps);     // arrive_j == 0: never
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) x[u] = (idx[u] < nvec) ? ld_loose(sj + idx[u]) : u32x4{ 0, 0, 0, 0 };
 #pragma unroll
@@ -768,13 +784,34 @@ struct MultiPhaseRegs {
     static constexpr int groups = 6;
 };
 
+// Stores per lane still to issue when a block reports the end of its write phase (Tuning::early_stores < 0 asks for
+// this).  Every plain type measures 0.7-1 % faster with 16 than with 4 (8 x 1 GiB and 4 x 1 GiB); the two bfloat16
+// families, whose lanes spend longer between their loads, are within 0.4 % from 4 to 20 and best at 4.
+template <class TR>
+struct PhaseEarlyStores {
+    static constexpr int value = 16;
+};
+template <bool RNE, bool VEC_SEM>
+struct PhaseEarlyStores<Bf16PairwiseTraits<RNE, VEC_SEM>> {
+    static constexpr int value = 4;
+};
+template <bool RNE>
+struct PhaseEarlyStores<Bf16KeepTraits<RNE>> {
+    static constexpr int value = 4;
+};
+template <class TR>
+inline int phase_early_stores(const Tuning& t) {
+    const int v = t.early_stores >= 0 ? t.early_stores : PhaseEarlyStores<TR>::value;
+    return v < kPhaseU ? v : kPhaseU;
+}
+
 // The phased form of the same: kPhaseU vectors per lane in LDS and 4 x MultiPhaseRegs::groups in registers are
 // reduced while HBM sees only reads, then stored to every destination while it sees only writes.  The register
 // groups are unrolled (a register file has no run-time index); the loop over the inputs inside each stays a loop.
 template <class TR, int OP>
 __global__ void __launch_bounds__(kPhaseBlock)
 reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uint64_t nvec, uint32_t tail,
-                           PhaseSync* ps) {
+                           PhaseSync* ps, int early_loads, int early_stores) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr int G = 4;                                // vectors per lane and input in flight
@@ -803,17 +840,30 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
                 for (int g = 0; g < G; g++) rs[q * G + g] = v[g];
             }
         }
+        bool arrived = false;       // thread 0 has reported this block's arrival at the end of the read phase
         for (int q = 0; q < LG; q++) {
             uint64_t idx[G];
             u32x4 v[G];
 #pragma unroll
             for (int g = 0; g < G; g++) idx[g] = pos(p0, (RG + q) * G + g);
             if (idx[0] >= nvec) break;      // slabs grow with q: nothing further for this lane in this phase
-            reduce_rt_tile<TR, OP, G>(src, n, head, idx, nvec, v);
+            // the arrival goes in front of the first load that leaves early_loads or fewer still to issue
+            const int rem = (LG - q) * n * G;
+            int arrive_j = 0;
+            if (!arrived) {
+                const int j = rem > early_loads ? (rem - early_loads + G - 1) / G : 0;
+                if (j == 0 && threadIdx.x == 0) phase_arrive(ps);
+                arrive_j = j < n ? j : 0;
+                arrived = j < n;
+            }
+            reduce_rt_tile<TR, OP, G>(src, n, head, idx, nvec, v, ps, arrive_j);
 #pragma unroll
             for (int g = 0; g < G; g++) stage[(q * G + g) * kPhaseBlock + threadIdx.x] = v[g];
         }
-        phase_barrier(ps, ++gen, give_up);
+        if (!arrived && threadIdx.x == 0) phase_arrive(ps);
+        phase_wait(ps, ++gen, give_up);
+        const bool more = p0 + per_phase < nvec;
+        const int arrive_u = more ? kPhaseU - early_stores : -1;    // kPhaseU: after the last store
         for (int k = 0; k < m; k++) {
             u32x4_u* d = (u32x4_u*)((unsigned char*)dst.p[k] + head * sizeof(E));
 #pragma unroll
@@ -823,10 +873,14 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
             }
             for (int u = 0; u < kPhaseU; u++) {
                 const uint64_t i = pos(p0, G * RG + u);
+                if (u == arrive_u && k == m - 1 && threadIdx.x == 0) phase_arrive(ps);
                 if (i < nvec) st_loose(d + i, stage[u * kPhaseBlock + threadIdx.x]);
             }
         }
-        if (p0 + per_phase < nvec) phase_barrier(ps, ++gen, give_up);
+        if (more) {
+            if (arrive_u == kPhaseU && threadIdx.x == 0) phase_arrive(ps);
+            phase_wait(ps, ++gen, give_up);
+        }
     }
     if (blockIdx.x == 0 && (head | tail)) reduce_multi_edges<TR, OP>(src, n, dst, m, head, nvec, tail);
 }
@@ -884,16 +938,27 @@ inline hipError_t launch_fixed_unroll(const LaunchArgs& a, uint32_t head, uint64
     return launch_fixed<TR, OP, N, kDefault>(a, head, nvec, tail);
 }
 
-// The phased form pays for its barriers from a few hundred MB of traffic, later the fewer inputs there are (less to
-// interleave per write).  Measured crossovers against the streaming kernels, in traffic per launch: 240 MB with 4 or
-// more inputs, 0.8 GB with 3, about 4 GB with 1 or 2; 320 MB with more than one destination.
-// Tuning::phased_min_bytes scales them all (default 160 MB); Tuning::variant 8 forces the phased form.
-inline bool wants_phased(const LaunchArgs& a, uint64_t nvec) {
+// When the phased form pays.  A phase costs a fixed few microseconds on top of its traffic, so what counts is how
+// full the phases are: fill = result bytes / (phases x what one phase holds, 88 MiB on 256 CUs).  Measured against
+// the streaming kernels (fp32 sum, one destination, rotating buffer sets): with 2 inputs the phased form wins at
+// fill 0.97 (+1 to +8 % from 256 MiB of traffic up) and loses at 0.73; with 3 it wins at 0.73 (+2-3 %) and loses at
+// 0.55; with 4 it wins at 0.58 and loses at 0.44; with 8 it wins from 0.32 (+3 %) and is even at 0.24: about 2 / n.
+// Long buffers have fill near 1 and are always phased (+8 % with 2 inputs, +17 % with 8 at 4 GiB of traffic).
+// Several destinations: from 2 x phased_min_bytes of traffic (default 320 MB).  One input stays with the copy and
+// broadcast kernels.  Tuning::phased_min_bytes is a lower bound on the traffic in every case (default 160 MB);
+// Tuning::variant 8 forces the phased form.
+inline bool wants_phased(const LaunchArgs& a, uint64_t nvec, int reg_groups) {
     if (a.tune.sync == nullptr || a.tune.num_cus < kPhaseGroups) return false;
     if (a.tune.variant != 0) return a.tune.variant == 8;
     const uint64_t traffic = (uint64_t)(a.n + a.m) * nvec * 16u;
-    const unsigned halves = a.m > 1 ? 4u : a.n >= 4 ? 3u : a.n == 3 ? 10u : a.n == 2 ? 60u : 50u;
-    return 2 * traffic >= (uint64_t)a.tune.phased_min_bytes * halves;
+    if (a.n < 2 || traffic < (uint64_t)a.tune.phased_min_bytes * (a.m > 1 ? 2u : 1u)) return false;
+    if (a.m > 1) return true;
+    const uint64_t grid = (uint64_t)(a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
+    const uint64_t per_phase = grid * kPhaseBlock * (uint64_t)(4 * reg_groups + kPhaseU);     // vectors
+    const uint64_t phases = (nvec + per_phase - 1) / per_phase;
+    const double fill = (double)nvec / (double)(phases * per_phase);
+    const double need = 2.0 / a.n < 0.9 ? 2.0 / a.n : 0.9;
+    return fill >= need;
 }
 
 // Elements before the first vector: the vectors start on a 16-byte boundary of as many buffers as possible (of the
@@ -923,11 +988,11 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
     if (head > a.count) head = a.count;
     const uint64_t nvec = (a.count - head) / VEC;
     const uint32_t tail = (uint32_t)(a.count - head - nvec * VEC);
-    if (wants_phased(a, nvec)) {
+    if (wants_phased(a, nvec, MultiPhaseRegs<TR>::groups)) {
         int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
         g_last_kernel = "reduce_multi_phased_kernel";
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
-                           a.m, (uint32_t)head, nvec, tail, a.tune.sync);
+                           a.m, (uint32_t)head, nvec, tail, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune));
         return hipGetLastError();
     }
     constexpr int UNROLL = 4;
@@ -948,7 +1013,7 @@ inline hipError_t launch_op(const LaunchArgs& a) {
     if (head > a.count) head = a.count;
     const uint64_t nvec = (a.count - head) / VEC;
     const uint32_t tail = (uint32_t)(a.count - head - nvec * VEC);
-    if (wants_phased(a, nvec)) return launch_multi_op<TR, OP>(a);         // the phased kernel takes any number of inputs
+    if (wants_phased(a, nvec, MultiPhaseRegs<TR>::groups)) return launch_multi_op<TR, OP>(a);     // the phased kernel takes any number of inputs
     // five or more inputs in the range between latency-bound and phased (64 to 240 MB of traffic): taking the inputs
     // one after the other, as the run-time-count streaming kernel does, measures 5-12 % above loading them together
     if (a.n >= 5 && a.tune.variant == 0 && (uint64_t)(a.n + 1) * nvec * 16u >= (uint64_t)a.tune.phased_min_bytes / 5 * 2)

@@ -218,16 +218,26 @@ def test_fused_reduce_over_several_phases(comp, dtype, op, n_peers, lp, impl, al
     d_t = [to_dev(t) for t in tensors]
     d_p = [to_dev(p) for p in peers]
     outs = [to_dev(np.zeros(c + 4, np_t)) for c in counts]
-    comp.set_param("variant", 8)
-    try:
-        plan.reduce(op, d_t, d_p, outs, lp_mode=lp, bf16_impl=impl)
-        torch.cuda.synchronize()
-    finally:
-        comp.set_param("variant", 0)
+    want = []
     for i, c in enumerate(counts):
         o = int(offs[i]) // esz
-        want = O.reduce_n([tensors[i]] + [p[o:o + c] for p in peers], dtype, op, keep=lp, bf16_impl=impl)
-        g = to_host(outs[i], np_t)
-        assert_same(g[:c], want, dtype, f"tensor {i} of {c} elements")
-        assert not g[c:].view(np.uint8).any(), "wrote past the tensor"
+        want.append(O.reduce_n([tensors[i]] + [p[o:o + c] for p in peers], dtype, op, keep=lp, bf16_impl=impl))
+    # the default, then other points at which a block reports its arrival at the barrier: timing only, same bits
+    for loads, stores in ((12, -1), (0, 0), (4096, 20), (40, 3)):
+        for o in outs:
+            o.zero_()
+        comp.set_param("variant", 8)
+        comp.set_param("phase_early_loads", loads)
+        comp.set_param("phase_early_stores", stores)
+        try:
+            plan.reduce(op, d_t, d_p, outs, lp_mode=lp, bf16_impl=impl)
+            torch.cuda.synchronize()
+        finally:
+            comp.set_param("variant", 0)
+            comp.set_param("phase_early_loads", 12)
+            comp.set_param("phase_early_stores", -1)
+        for i, c in enumerate(counts):
+            g = to_host(outs[i], np_t)
+            assert_same(g[:c], want[i], dtype, f"tensor {i} of {c} elements, early loads {loads} stores {stores}")
+            assert not g[c:].view(np.uint8).any(), "wrote past the tensor"
     plan.close()

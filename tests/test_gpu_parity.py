@@ -422,6 +422,43 @@ def test_phased_kernel_parity(comp, dtype, op, n):
         comp.set_param("variant", 0)
 
 
+@pytest.mark.parametrize("dtype,op,n,m", [(O.BFLOAT16, O.SUM, 8, 1), (O.FLOAT32, O.SUM, 2, 1), (O.INT32, O.MAX, 1, 1),
+                                          (O.FLOAT16, O.SUM, 3, 2), (O.INT8, O.SUM, 16, 1)])
+def test_phased_kernel_early_arrival_settings(comp, dtype, op, n, m):
+    """A block of the phased kernel reports its arrival at the chip-wide barrier a few loads / stores before it is done
+    ("phase_early_loads", "phase_early_stores").  The barrier aligns the blocks in time only, so every setting, from
+    "when done" to "before the first staged load", must give the oracle's bits: three full phases and a partial one."""
+    import torch
+    rng = np.random.default_rng(900 + dtype + n)
+    esz = O.DTYPE_SIZE[dtype]
+    keep = 1 if dtype == O.BFLOAT16 else 0
+    per_phase = comp.get_param("num_cus") * 512 * 44 * (16 // esz)      # elements one phase covers
+    count = 3 * per_phase + per_phase // 5 + 3
+    srcs = make_inputs(rng, dtype, count, op, n)
+    want = O.reduce_n(srcs, dtype, op, keep=keep, threads=16)
+    d = [to_dev(s) for s in srcs]
+    assert comp.get_param("phase_early_loads") == 12 and comp.get_param("phase_early_stores") == -1
+    comp.set_param("variant", 8)
+    try:
+        for loads, stores in ((12, -1), (0, 0), (4, 20), (1000, 1), (4096, 7), (13, 19)):
+            comp.set_param("phase_early_loads", loads)
+            comp.set_param("phase_early_stores", stores)
+            outs = [torch.zeros_like(d[0]) for _ in range(m)]
+            comp.comp_reduce_write_n(dtype, op, d, outs, count, lp_mode=comp.LP_KEEP_PRECISION if keep else 0)
+            torch.cuda.synchronize()
+            assert comp.last_kernel() == "reduce_multi_phased_kernel"
+            for o in outs:
+                assert_same(to_host(o, O.NP_STORAGE[dtype]), want, dtype, f"early loads {loads} stores {stores}", srcs, op,
+                            keep=keep)
+        for bad in (("phase_early_loads", -1), ("phase_early_loads", 4097), ("phase_early_stores", -2), ("phase_early_stores", 21)):
+            with pytest.raises(comp.CclError):
+                comp.set_param(*bad)
+    finally:
+        comp.set_param("variant", 0)
+        comp.set_param("phase_early_loads", 12)
+        comp.set_param("phase_early_stores", -1)
+
+
 @pytest.mark.parametrize("variant", [0, 1, 8])
 @pytest.mark.parametrize("dtype,op,n,m", [(O.BFLOAT16, O.SUM, 8, 1), (O.INT8, O.MAX, 5, 1), (O.FLOAT16, O.MIN, 3, 2),
                                           (O.FLOAT64, O.SUM, 2, 1), (O.INT32, O.PROD, 11, 3), (O.UINT16, O.SUM, 1, 2)])
