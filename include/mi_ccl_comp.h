@@ -241,7 +241,9 @@ const char* mi_ccl_last_kernel(void);
  * "phase_early_loads" / "phase_early_stores" (phased kernels: how many 16-byte loads / stores per lane a block still
  * has to issue when it reports the end of its read / write phase to the chip-wide barrier, which hides the barrier's
  * latency; defaults 12 and -1 = chosen per element type, 4 or 16; 0 = report when done; timing only, results do not
- * depend on them), "num_cus" (read
+ * depend on them), "phase_spin_ticks" (phased kernels: the longest a block waits at one barrier, in 100 MHz ticks,
+ * before it goes on alone and stops waiting for the rest of the launch; default 20000 = 200 us; 0 = never wait, which
+ * costs speed only and is what the tests of that path use), "num_cus" (read
  * only), "fp16_impl" (what MI_CCL_FP16_DEFAULT stands for: 2, 3 or 4 of enum mi_ccl_fp16_impl above), and
  * "launch_block_limit" (blocks per launch of the copy, broadcast and converter kernels, which cut larger work into
  * several launches; 0 = what HIP allows, 2^24 - 1; smaller values let tests exercise the cutting).

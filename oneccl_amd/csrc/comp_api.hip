@@ -51,6 +51,7 @@ static std::atomic<int> g_variant{ 0 };
 static std::atomic<long> g_phased_min_bytes{ 160L << 20 };
 static std::atomic<int> g_phase_early_loads{ 12 };
 static std::atomic<int> g_phase_early_stores{ -1 };
+static std::atomic<long> g_phase_spin_ticks{ kPhaseSpinTicks };
 static std::atomic<int> g_fp16_impl{ MI_CCL_FP16_AVX512F };
 static std::atomic<long> g_launch_block_limit{ 0 };     // 0: what HIP allows; smaller values are for tests of the splitting
 static_assert(kGeomBlock == kBlock, "the geometry header and the kernels agree on the block size");
@@ -112,6 +113,7 @@ Tuning current_tuning() {
     t.sync = phase_sync();
     t.early_loads = g_phase_early_loads.load(std::memory_order_relaxed);
     t.early_stores = g_phase_early_stores.load(std::memory_order_relaxed);
+    t.spin_ticks = g_phase_spin_ticks.load(std::memory_order_relaxed);
     t.fp16_impl = g_fp16_impl.load(std::memory_order_relaxed);
     return t;
 }
@@ -828,6 +830,10 @@ int mi_ccl_set_param(const char* name, long value) {
         g_phase_early_stores.store((int)value);
         return MI_CCL_SUCCESS;
     }
+    if (!strcmp(name, "phase_spin_ticks") && value >= 0 && value <= 100000000) {
+        g_phase_spin_ticks.store(value);
+        return MI_CCL_SUCCESS;
+    }
     if (!strcmp(name, "fp16_impl") && value >= MI_CCL_FP16_F16C && value <= MI_CCL_FP16_AVX512FP16) {
         g_fp16_impl.store((int)value);
         return MI_CCL_SUCCESS;
@@ -856,6 +862,8 @@ long mi_ccl_get_param(const char* name) {
         return g_phase_early_loads.load();
     if (!strcmp(name, "phase_early_stores"))
         return g_phase_early_stores.load();
+    if (!strcmp(name, "phase_spin_ticks"))
+        return g_phase_spin_ticks.load();
     if (!strcmp(name, "fp16_impl"))
         return g_fp16_impl.load();
     if (!strcmp(name, "launch_block_limit"))

@@ -8,6 +8,7 @@
 #include "../../include/mi_ccl_comp.h"
 #include "fusion_kernels.hpp"
 #include "launch_geometry.hpp"
+#include "launch_geometry.hpp"
 
 namespace mi {
 
@@ -56,8 +57,14 @@ static size_t fusion_dtype_size(int dtype) {
 // pointer), so it holds kFusionCopyGroup tensors: the 256 tensors of a typical bucket are one launch.  Measured on the
 // 256-tensor configuration (191 MB of payload): 61.8 us against 68.4 us for 16 KiB per block in two launches, and
 // 58.3 us for a plain copy of as many bytes.
+//
+// The quarters are cut where the DESTINATION crosses a 128-byte line, not at multiples of 4 KiB of the tensor: in a
+// tightly packed fusion buffer behind an odd-sized tensor the two differ, and quarters cut by tensor offset would each
+// start and end inside a line (and inside a vector: up to 15 single-byte stores at either end) that the neighbouring
+// block writes too.  Quarter 0 is short by what the destination lacks to its first line boundary, the tensor's last
+// quarter takes the rest (at most 127 bytes more than 4 KiB, so a few lanes copy a second vector).
 constexpr int kFusionCopyGroup = 448;
-constexpr uint32_t kFusionCopySub = 4096;         // bytes per block
+constexpr uint32_t kFusionCopySub = kCopyQuarter;  // bytes per block
 static_assert(kFusionChunk % kFusionCopySub == 0 && kFusionCopySub == 16 * kBlock, "an item is a whole number of block-sized quarters");
 struct FusionCopyPtrs {
     const void* p[kFusionCopyGroup];
@@ -70,20 +77,19 @@ fusion_copy_kernel(FusionCopyPtrs tensors, unsigned char* fusion_buf, const uint
     constexpr uint32_t kSubs = kFusionChunk / kFusionCopySub;
     const uint32_t tid = threadIdx.x;
     const FusionItem w = items[blockIdx.x / kSubs];
-    const uint64_t lo = (uint64_t)w.c * kFusionChunk + (blockIdx.x % kSubs) * kFusionCopySub;
-    const uint64_t total = bytes[w.t];
-    if (lo >= total) return;                        // the item's last quarters may be empty
-    const uint64_t left = total - lo;
-    const uint32_t n = left < kFusionCopySub ? (uint32_t)left : kFusionCopySub;
-    unsigned char* tp = (unsigned char*)tensors.p[w.t - t0] + lo;
-    unsigned char* fp = fusion_buf + off[w.t] + lo;
-    const unsigned char* src = to_fusion ? tp : fp;
-    unsigned char* dst = to_fusion ? fp : tp;
+    unsigned char* tp = (unsigned char*)tensors.p[w.t - t0];
+    unsigned char* fp = fusion_buf + off[w.t];
+    const CopyQuarter cq = copy_quarter(bytes[w.t], (uint64_t)(uintptr_t)(to_fusion ? fp : tp),
+                                        (uint64_t)w.c * kSubs + blockIdx.x % kSubs);
+    const uint32_t n = cq.n;                        // at most 4 KiB + 127
+    if (n == 0) return;                             // the last item's last quarters may be empty
+    const unsigned char* src = (to_fusion ? tp : fp) + cq.lo;
+    unsigned char* dst = (to_fusion ? fp : tp) + cq.lo;
     // vectors from the destination's first 16-byte boundary on, whatever the source's alignment is
     uint32_t head = (uint32_t)(-(intptr_t)dst) & 15u;
     if (head > n) head = n;
     const uint32_t nvec = (n - head) >> 4, tail = n - head - (nvec << 4);
-    if (tid < nvec) st_loose((u32x4_u*)(dst + head) + tid, ld_loose((const u32x4_u*)(src + head) + tid));
+    for (uint32_t v = tid; v < nvec; v += kBlock) st_loose((u32x4_u*)(dst + head) + v, ld_loose((const u32x4_u*)(src + head) + v));
     if (tid < head + tail) {
         const uint32_t i = (tid < head) ? tid : head + (nvec << 4) + (tid - head);
         dst[i] = src[i];

@@ -127,7 +127,7 @@ template <class TR, int OP, int NT>
 __global__ void __launch_bounds__(kPhaseBlock)
 fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, const uint64_t* off, const uint64_t* bytes,
                             const FusionItem* items, uint32_t nitems, uint32_t t0, PhaseSync* ps, int early_loads,
-                            int early_stores) {
+                            int early_stores, long spin_ticks) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr uint32_t ES = sizeof(E);
@@ -219,7 +219,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
             }
         }
         if (!arrived && tid == 0) phase_arrive(ps);
-        phase_wait(ps, ++gen, give_up);
+        phase_wait(ps, ++gen, give_up, spin_ticks);
         const bool more = p0 + per_phase < nitems;
         const int lead_w = early_stores / 2;
         const int arrive_w = nslots > lead_w ? nslots - lead_w : 0;
@@ -258,7 +258,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
         }
         if (more) {
             if (!arrived && tid == 0) phase_arrive(ps);
-            phase_wait(ps, ++gen, give_up);
+            phase_wait(ps, ++gen, give_up, spin_ticks);
         }
     }
 }
@@ -270,7 +270,7 @@ inline hipError_t launch_fusion_phased(const FusionLaunchArgs& a, const FusionPt
     g_last_kernel = "fusion_reduce_phased_kernel";
     hipLaunchKernelGGL((fusion_reduce_phased_kernel<TR, OP, NT>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, own, out, pp,
                        a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0, a.tune.sync,
-                       a.tune.early_loads, phase_early_stores<TR>(a.tune));
+                       a.tune.early_loads, phase_early_stores<TR>(a.tune), a.tune.spin_ticks);
     return hipGetLastError();
 }
 

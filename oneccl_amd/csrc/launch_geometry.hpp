@@ -129,4 +129,26 @@ MI_GEOM_HD inline BcastLane bcast_lane(uint32_t blk, uint32_t tid, uint32_t sect
     return l;
 }
 
+// ---- pack / unpack: the 4 KiB quarters of one tensor, cut where the destination crosses a 128-byte line -------------
+// Quarter q of a tensor of `total` bytes whose destination starts at address dst_addr covers bytes [lo, lo + n) of
+// the tensor: quarter 0 ends at the destination's first line boundary at or before 4 KiB, every further quarter starts
+// on a line boundary and is 4 KiB, the last one takes what is left (n <= 4 KiB + 127).  n == 0: no such quarter.
+constexpr uint32_t kCopyQuarter = 4096;
+constexpr uint32_t kCopyLine = 128;
+struct CopyQuarter {
+    uint64_t lo;
+    uint32_t n;
+};
+MI_GEOM_HD inline CopyQuarter copy_quarter(uint64_t total, uint64_t dst_addr, uint64_t q) {
+    const uint64_t nq = (total + kCopyQuarter - 1) / kCopyQuarter;
+    CopyQuarter r = { 0, 0 };
+    if (q >= nq) return r;
+    const uint64_t lack = (0 - dst_addr) & (kCopyLine - 1);     // bytes to the destination's first line boundary
+    const uint64_t back = lack ? kCopyLine - lack : 0;
+    r.lo = q ? q * kCopyQuarter - back : 0;
+    const uint64_t hi = (q + 1 == nq) ? total : (q + 1) * kCopyQuarter - back;
+    r.n = (uint32_t)(hi - r.lo);
+    return r;
+}
+
 }  // namespace mi

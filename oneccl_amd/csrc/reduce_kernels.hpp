@@ -47,6 +47,7 @@ struct Tuning {
     struct PhaseSync* sync;  // the set of device-resident barrier words this call uses (may be null)
     int early_loads;         // phased kernels: loads per lane still to issue when a block reports the end of its reads
     int early_stores;        // ... and stores per lane still to issue when it reports the end of its writes (< 0: per type)
+    long spin_ticks;         // phased kernels: longest wait at one barrier, in 100 MHz ticks, before a block goes on alone
     int fp16_impl;           // which CPU implementation's float16 results to reproduce: 2, 3 (through fp32) or 4 (native)
 };
 
@@ -615,7 +616,7 @@ reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint
 constexpr int kPhaseBlock = 512;                  // 8 wavefronts, one block per CU
 constexpr int kPhaseU = 20;                       // vectors per lane per phase staged in LDS: 20 x 16 B x 512 lanes = 160 KiB
 constexpr int kPhaseGroups = 16;                  // arrival counters (same-address atomics serialise)
-constexpr long long kPhaseSpinTicks = 20000;      // 100 MHz ticks: 200 us
+constexpr long kPhaseSpinTicks = 20000;           // default bound on one wait, in 100 MHz ticks: 200 us
 
 struct __attribute__((aligned(256))) PhaseWord {
     unsigned v;
@@ -657,12 +658,12 @@ __device__ __forceinline__ void phase_arrive(PhaseSync* ps) {
 }
 // No data crosses the barrier (a lane only ever reads back the LDS slots it wrote itself), so the waves of a block
 // are held by a bare s_barrier: nothing has to wait for the block's outstanding stores.
-__device__ __forceinline__ void phase_wait(PhaseSync* ps, unsigned gen, bool& give_up) {
+__device__ __forceinline__ void phase_wait(PhaseSync* ps, unsigned gen, bool& give_up, long spin_ticks) {
     if (threadIdx.x == 0 && !give_up) {
         const long long t0 = wall_clock64();
         while ((int)(MI_ALOAD(&ps->top.v) - gen * kPhaseGroups) < 0) {
             __builtin_amdgcn_s_sleep(1);
-            if (wall_clock64() - t0 > kPhaseSpinTicks) {
+            if (wall_clock64() - t0 >= spin_ticks) {
                 give_up = true;
                 break;
             }
@@ -811,7 +812,7 @@ inline int phase_early_stores(const Tuning& t) {
 template <class TR, int OP>
 __global__ void __launch_bounds__(kPhaseBlock)
 reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uint64_t nvec, uint32_t tail,
-                           PhaseSync* ps, int early_loads, int early_stores) {
+                           PhaseSync* ps, int early_loads, int early_stores, long spin_ticks) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr int G = 4;                                // vectors per lane and input in flight
@@ -861,7 +862,7 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
             for (int g = 0; g < G; g++) stage[(q * G + g) * kPhaseBlock + threadIdx.x] = v[g];
         }
         if (!arrived && threadIdx.x == 0) phase_arrive(ps);
-        phase_wait(ps, ++gen, give_up);
+        phase_wait(ps, ++gen, give_up, spin_ticks);
         const bool more = p0 + per_phase < nvec;
         const int arrive_u = more ? kPhaseU - early_stores : -1;    // kPhaseU: after the last store
         for (int k = 0; k < m; k++) {
@@ -879,7 +880,7 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
         }
         if (more) {
             if (arrive_u == kPhaseU && threadIdx.x == 0) phase_arrive(ps);
-            phase_wait(ps, ++gen, give_up);
+            phase_wait(ps, ++gen, give_up, spin_ticks);
         }
     }
     if (blockIdx.x == 0 && (head | tail)) reduce_multi_edges<TR, OP>(src, n, dst, m, head, nvec, tail);
@@ -992,7 +993,7 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
         int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
         g_last_kernel = "reduce_multi_phased_kernel";
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
-                           a.m, (uint32_t)head, nvec, tail, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune));
+                           a.m, (uint32_t)head, nvec, tail, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune), a.tune.spin_ticks);
         return hipGetLastError();
     }
     constexpr int UNROLL = 4;

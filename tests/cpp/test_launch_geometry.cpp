@@ -124,6 +124,26 @@ int main() {
                 for (int m : { 1, 2, 3, 7, 16 })
                     for (uint32_t max_sect : { 8u, 16u, 4096u }) check_bcast(addr, bytes, m, max_sect, limit, true);
             }
+    // pack / unpack quarters: they tile the tensor exactly, none is longer than 4 KiB + 127, every quarter but the
+    // first starts on a 128-byte line of the destination, and none exists beyond ceil(total / 4 KiB)
+    for (uint64_t total : { 1ull, 2ull, 127ull, 128ull, 129ull, 4095ull, 4096ull, 4097ull, 4223ull, 4224ull, 8191ull, 8192ull, 16383ull, 16384ull,
+                            16385ull, 100003ull, 4194304ull, 4194306ull, 12345678ull })
+        for (uint64_t mis = 0; mis < 128; mis += (total < 20000 ? 1 : 7)) {
+            const uint64_t dst = 0x7f0000100000ull + mis;
+            const uint64_t nq = (total + kCopyQuarter - 1) / kCopyQuarter;
+            uint64_t next = 0;
+            for (uint64_t q = 0; q < nq; q++) {
+                const CopyQuarter c = copy_quarter(total, dst, q);
+                EXPECT(c.n > 0 && c.n <= kCopyQuarter + kCopyLine - 1);
+                EXPECT(c.lo == next);
+                EXPECT(q == 0 || ((dst + c.lo) & (kCopyLine - 1)) == 0);
+                EXPECT(q + 1 == nq || c.n <= kCopyQuarter);
+                next = c.lo + c.n;
+            }
+            EXPECT(next == total);
+            for (uint64_t q = nq; q < nq + 4; q++) EXPECT(copy_quarter(total, dst, q).n == 0);
+        }
+    EXPECT(copy_quarter(0, 0x1000, 0).n == 0);
     printf("%d checks, %d failed\n", checks, failed);
     return failed ? 1 : 0;
 }

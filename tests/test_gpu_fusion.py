@@ -81,6 +81,31 @@ def test_pack_reduce_unpack_and_fused(comp, align, dtype):
         g = to_host(outs[i], np_t)
         assert_same(g[:c], want[i], dtype, f"3-step tensor {i}")
         assert (g[c:] == 0).all(), "unpack wrote past the tensor"
+    # unpack into tensors that start at odd element offsets inside larger allocations (the copy is cut where the
+    # destination crosses cache lines, which then differs from tensor to tensor): nothing outside the tensor is written
+    holders_u, d_u = [], []
+    for i, c in enumerate(counts):
+        sh = i % 5
+        h = to_dev(np.zeros(sh + c + 8, np_t))
+        holders_u.append(h)
+        d_u.append(h.data_ptr() + sh * esz)
+    plan.unpack(d_fb, d_u)
+    torch.cuda.synchronize()
+    for i, c in enumerate(counts):
+        sh = i % 5
+        g = to_host(holders_u[i], np_t)
+        assert_same(g[sh:sh + c], want[i], dtype, f"unpack to shifted tensor {i}")
+        assert (g[:sh] == 0).all() and (g[sh + c:] == 0).all(), "unpack wrote outside the shifted tensor"
+    # ... and pack once more into a fusion buffer that itself starts 3 elements into its allocation
+    d_fb2 = to_dev(np.zeros(nelem + 3 + 8, np_t))
+    plan.pack(d_t, d_fb2.data_ptr() + 3 * esz)
+    torch.cuda.synchronize()
+    got2 = to_host(d_fb2, np_t)
+    assert (got2[:3] == 0).all() and (got2[3 + nelem:] == 0).all(), "pack wrote outside the fusion buffer"
+    got2 = got2[3:3 + nelem].view(np.uint8)
+    for i, c in enumerate(counts):
+        o = int(offs[i])
+        assert (got2[o:o + c * esz] == fb[o:o + c * esz]).all(), f"pack into a shifted buffer, tensor {i}"
 
     # GPU, fused single pass, out of place (streaming kernel, then the phased one forced on) and in place
     for variant in (2, 8):

@@ -459,6 +459,35 @@ def test_phased_kernel_early_arrival_settings(comp, dtype, op, n, m):
         comp.set_param("phase_early_stores", -1)
 
 
+def test_phased_kernel_when_no_block_waits(comp):
+    """The bound on a block's wait at the chip-wide barrier set to zero from the host: every block goes on alone after
+    its first poll, the phases of different blocks overlap freely, and the result is still the oracle's (the barrier
+    carries no data).  Every block still reports all its arrivals, so the launches that follow, with the default
+    bound again, find the barrier words consistent and give the same bits."""
+    import torch
+    rng = np.random.default_rng(77)
+    dtype, n = O.BFLOAT16, 8
+    per_phase = comp.get_param("num_cus") * 512 * 44 * 8
+    count = 4 * per_phase + 12345
+    srcs = make_inputs(rng, dtype, count, O.SUM, n)
+    want = O.reduce_n(srcs, dtype, O.SUM, keep=1, threads=16)
+    d = [to_dev(s) for s in srcs]
+    assert comp.get_param("phase_spin_ticks") == 20000
+    comp.set_param("variant", 8)
+    try:
+        for ticks in (0, 0, 20000, 20000):
+            comp.set_param("phase_spin_ticks", ticks)
+            out = torch.zeros_like(d[0])
+            for _ in range(17):         # more calls than there are sets of barrier words: every set is used both ways
+                comp.comp_reduce_n(dtype, O.SUM, d, out, count, lp_mode=comp.LP_KEEP_PRECISION)
+            torch.cuda.synchronize()
+            assert comp.last_kernel() == "reduce_multi_phased_kernel"
+            assert_same(to_host(out, np.uint16), want, dtype, f"wait bound {ticks} ticks", srcs, O.SUM, keep=1)
+    finally:
+        comp.set_param("variant", 0)
+        comp.set_param("phase_spin_ticks", 20000)
+
+
 @pytest.mark.parametrize("variant", [0, 1, 8])
 @pytest.mark.parametrize("dtype,op,n,m", [(O.BFLOAT16, O.SUM, 8, 1), (O.INT8, O.MAX, 5, 1), (O.FLOAT16, O.MIN, 3, 2),
                                           (O.FLOAT64, O.SUM, 2, 1), (O.INT32, O.PROD, 11, 3), (O.UINT16, O.SUM, 1, 2)])
