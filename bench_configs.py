@@ -122,6 +122,8 @@ def main():
         verify_reduce("C1", O.FLOAT32, O.SUM, [sets[0][0], sets[0][1]], c1_once, n1)
         us = timed(torch, lambda i: comp.comp_reduce(comp.FLOAT32, comp.SUM, sets[i % 8][1], n1, sets[i % 8][0]), 64, 16)
         add("C1 fp32 sum, 2 inputs in place, 64 MiB", us, 3 * n1 * 4, f"8 rotating buffer sets; {comp.last_kernel()}")
+        us = timed(torch, lambda i: comp.comp_reduce(comp.FLOAT32, comp.SUM, sets[0][1], n1, sets[0][0]), 64, 16)
+        add("C1 same, one buffer set (Infinity Cache assisted)", us, 3 * n1 * 4, "")
         del sets
     # ---- C2
     if want("c2"):
