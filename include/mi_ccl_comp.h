@@ -129,8 +129,9 @@ int mi_ccl_comp_reduce_write_n(int dtype, int op, const void* const* srcs, int n
  * nothing is allocated.  Replaces read_reduce_write (n = 2: even[i] = pair[i] + local[i] for every peer i in one kernel,
  * src/coll/algorithms/reduce_scatter/sycl/reduce_scatter_large_sycl_impl.hpp:22-66), reduce_read_write_kernel_{1..7}
  * (src/kernels/kernels.cl:156-177) and, with n = 1, copy_data (N copies in one kernel, used at :216-224 of the same
- * file); it is also the small-message path: 64 reduces of a few KiB cost one launch, not 64.  lp_mode:
- * MI_CCL_LP_PAIRWISE or MI_CCL_LP_KEEP_PRECISION (bfloat16). */
+ * file); it is also the small-message path: 64 reduces of a few KiB cost one launch, not 64.  A job that moves
+ * "phased_min_bytes" (160 MB) or more, (n + 1) x its bytes, gets a launch of its own in the kernel form its size calls
+ * for (still nothing allocated on the device).  lp_mode: MI_CCL_LP_PAIRWISE or MI_CCL_LP_KEEP_PRECISION (bfloat16). */
 int mi_ccl_comp_reduce_batch(int dtype, int op, const void* const* srcs, int n, void* const* dsts,
                              const size_t* counts, int n_jobs, int lp_mode, int bf16_impl, int fp16_impl,
                              void* stream);

@@ -6,6 +6,7 @@
 #include <string.h>
 
 #include <atomic>
+#include <vector>
 #include <cctype>
 
 #include "../../include/mi_ccl_comp.h"
@@ -647,6 +648,37 @@ int mi_ccl_comp_reduce_batch(int dtype, int op, const void* const* srcs, int n, 
     a.tune = current_tuning();
     if (fp16_impl != MI_CCL_FP16_DEFAULT)
         a.tune.fp16_impl = fp16_impl;
+    // A job that moves as much as a launch of its own would be phased for (the chunks of a large reduce-scatter:
+    // hundreds of MB each) goes through the single-reduce path, which picks the kernel form for its size; one more
+    // launch is nothing against it.  The others share the batch launch.
+    const uint64_t big = (uint64_t)a.tune.phased_min_bytes;
+    int n_big = 0;
+    if (a.tune.variant == 0)
+        for (int j = 0; j < n_jobs; j++) n_big += (uint64_t)(n + 1) * counts[j] * esz >= big;
+    if (n_big == 0)
+        return status_of(dispatch_batch(dtype, keep, bf16_impl, a));
+    std::vector<const void*> s_small;
+    std::vector<void*> d_small;
+    std::vector<size_t> c_small;
+    for (int j = 0; j < n_jobs; j++) {
+        if ((uint64_t)(n + 1) * counts[j] * esz >= big) {
+            const int rc = reduce_n_impl(dtype, op, srcs + (size_t)j * n, n, dsts + j, 1, counts[j], lp_mode, bf16_impl,
+                                         fp16_impl, stream);
+            if (rc != MI_CCL_SUCCESS)
+                return rc;
+        }
+        else if (counts[j]) {
+            s_small.insert(s_small.end(), srcs + (size_t)j * n, srcs + (size_t)(j + 1) * n);
+            d_small.push_back(dsts[j]);
+            c_small.push_back(counts[j]);
+        }
+    }
+    if (c_small.empty())
+        return MI_CCL_SUCCESS;
+    a.srcs = s_small.data();
+    a.dsts = d_small.data();
+    a.counts = c_small.data();
+    a.n_jobs = (int)c_small.size();
     return status_of(dispatch_batch(dtype, keep, bf16_impl, a));
 }
 

@@ -89,6 +89,20 @@ def test_more_jobs_than_one_table_holds_with_eight_inputs(comp):
     _run(comp, rng, O.INT64, O.MIN, 8, counts, in_place_every=2)
 
 
+def test_large_jobs_mixed_with_small_ones(comp):
+    """Jobs that move 160 MB or more get launches of their own (the phased kernel for the two largest here), the rest
+    share one: the chunks of a large reduce-scatter beside a few stragglers, in one call, every job against the oracle.
+    All jobs large, and only the middle one large, as well."""
+    rng = np.random.default_rng(7170)
+    big2 = (340 << 20) // 4           # two fp32 inputs: 3 x 340 MiB of traffic, four nearly full phases
+    _run(comp, rng, O.FLOAT32, O.SUM, 2, [1000, big2, 0, 77, big2 + 5, 1 << 20, 14 << 20], in_place_every=2)
+    assert comp.last_kernel() == "reduce_batch_kernel"
+    _run(comp, rng, O.FLOAT32, O.SUM, 2, [14 << 20, 14 << 20 | 1], mixed_align=False)
+    assert comp.last_kernel() == "reduce_vec_kernel"
+    _run(comp, rng, O.BFLOAT16, O.SUM, 4, [5, 40 << 20, 9], lp=comp.LP_KEEP_PRECISION, keep=1)
+    _run(comp, rng, O.INT8, O.MAX, 1, [3, 200 << 20, 4099])
+
+
 def test_sixteen_bit_modes_and_nan_patterns(comp):
     rng = np.random.default_rng(7200)
     counts = [33, 8191, 1, 100_003, 16]
