@@ -105,8 +105,9 @@ inline hipError_t launch_batch_op(const BatchLaunchArgs& a) {
         for (; j0 + nj < a.n_jobs && nj < per_launch; nj++) {
             const int j = j0 + nj;
             const uint64_t count = a.counts[j];
-            // the vectors of a job start on a 16-byte boundary of as many of its buffers as possible (vector_head)
+            // the vectors of a job start on the 16-byte boundary of the buffer that makes the loose accesses cheapest (vector_head)
             LaunchArgs one;
+            one.tune = a.tune;
             one.srcs = a.srcs + (size_t)j * a.n;
             one.n = a.n;
             one.dst = a.dsts[j];

@@ -15,6 +15,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#define MI_HD_INLINE __host__ __device__ inline
+
 namespace mi {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -497,8 +499,8 @@ __device__ __forceinline__ u32x4 vec_finish(const Accs<TR>& a) {
 // Streaming 128-bit accesses through pointers that promise no alignment (the instruction is the same one).  The
 // memory pipeline takes a vector access at any byte address (a wave's 1 KiB then touches one cache line more), so
 // buffers that disagree modulo 16 bytes -- tensors behind an odd-sized one in a tightly packed fusion buffer, a
-// peer's chunk at an odd offset -- still move as vectors.  The host starts the vectors on a 16-byte boundary of as
-// many buffers as it can.
+// peer's chunk at an odd offset -- still move as vectors.  The host starts the vectors on the 16-byte boundary of the
+// buffer that makes the loose accesses cheapest (vector_head).
 typedef u32x4 u32x4_u __attribute__((aligned(1)));
 __device__ __forceinline__ u32x4 ld_loose(const u32x4_u* p) { return __builtin_nontemporal_load(p); }
 __device__ __forceinline__ void st_loose(u32x4_u* p, u32x4 v) { __builtin_nontemporal_store(v, p); }
@@ -962,18 +964,34 @@ inline bool wants_phased(const LaunchArgs& a, uint64_t nvec, int reg_groups) {
     return fill >= need;
 }
 
-// Elements before the first vector: the vectors start on a 16-byte boundary of as many buffers as possible (of the
-// first destination among equals; eight aligned inputs and a loose output measure 6.6 TB/s where the reverse measures
-// 5.2).  The buffers that disagree are read and written as loose vectors.  No head when that boundary is not a
-// multiple of the element size.
+// Elements before the first vector.  The vectors start on a 16-byte boundary of one of the buffers; the buffers that
+// disagree with it are read and written as loose vectors, and what that costs depends on which they are.  Measured
+// with the phased kernel on 8 x 1 GiB bf16 (7.14 TB/s with everything aligned): seven inputs 4 bytes off the grid
+// 7.00 (-2 %: a loose read on a 4-byte boundary is nearly free), eight inputs 2 bytes off 5.66 (-21 %: off the 4-byte
+// boundary a loose read is dear), the output alone off the grid, by 4 or by 6 bytes, 6.67-6.80 (-5 to -7 %).  So every
+// candidate boundary is priced -- 1 per input that is off it by a multiple of 4 bytes, 8 per input off it otherwise,
+// 16 per output off it -- and the cheapest wins, the first destination's among equals.  (A plain majority, the rule
+// before, put the grid on seven peers 4 bytes off and paid for a loose output: 6.67 against 7.00.)  No head when that
+// boundary is not a multiple of the element size.
+MI_HD_INLINE unsigned loose_read_cost(unsigned off) {
+    return (off & 15u) == 0 ? 0u : (off & 3u) == 0 ? 1u : 8u;
+}
 template <class E>
 inline uint64_t vector_head(const LaunchArgs& a) {
-    int votes[16] = { 0 };
-    for (int j = 0; j < a.n; j++) votes[(uintptr_t)a.srcs[j] & 15u]++;
-    for (int k = 0; k < a.m; k++) votes[(uintptr_t)(a.dsts ? a.dsts[k] : a.dst) & 15u]++;
-    uintptr_t mis = (uintptr_t)(a.dsts ? a.dsts[0] : a.dst) & 15u;
-    for (uintptr_t c = 0; c < 16; c++)
-        if (votes[c] > votes[mis]) mis = c;
+    unsigned in_mis[kMaxSrcs], out_mis[kMaxDsts];
+    for (int j = 0; j < a.n; j++) in_mis[j] = (unsigned)((uintptr_t)a.srcs[j] & 15u);
+    for (int k = 0; k < a.m; k++) out_mis[k] = (unsigned)((uintptr_t)(a.dsts ? a.dsts[k] : a.dst) & 15u);
+    auto price = [&](unsigned c) {
+        unsigned p = 0;
+        for (int j = 0; j < a.n; j++) p += loose_read_cost(in_mis[j] - c);
+        for (int k = 0; k < a.m; k++) p += out_mis[k] == c ? 0u : 16u;
+        return p;
+    };
+    unsigned mis = out_mis[0], best = price(mis);
+    for (int k = 1; k < a.m; k++)
+        if (price(out_mis[k]) < best) best = price(mis = out_mis[k]);
+    for (int j = 0; j < a.n; j++)
+        if (price(in_mis[j]) < best) best = price(mis = in_mis[j]);
     return (mis % sizeof(E)) == 0 ? ((16u - mis) & 15u) / sizeof(E) : 0;
 }
 
