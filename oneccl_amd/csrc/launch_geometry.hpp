@@ -1,5 +1,6 @@
-// Launch geometry of the copy-shaped kernels (copy, broadcast, array converters): plain host arithmetic, kept apart
-// from the kernels so that it can be compiled and tested without a GPU.
+// Launch geometry of the copy-shaped kernels (copy, broadcast, array converters, pack / unpack) and the host's choices
+// for a reduce (where its vectors start, whether its phased form pays): plain arithmetic, kept apart from the kernels
+// so that it can be compiled and tested without a GPU.
 //
 // These kernels give every lane one group of elements (one 16-byte vector, or the 4 or 8 elements that make one) and
 // every block one tile of kGeomBlock groups.  HIP refuses a launch whose gridDim.x * blockDim.x reaches 2^32, i.e. more
@@ -127,6 +128,53 @@ MI_GEOM_HD inline BcastLane bcast_lane(uint32_t blk, uint32_t tid, uint32_t sect
     l.dst = k;
     l.vec = ((uint64_t)sect * sect_tiles + t) * kGeomBlock + tid;
     return l;
+}
+
+// ---- where the 16-byte vectors of a reduce start -----------------------------------------------------------------
+// The vectors start on a 16-byte boundary of one of the buffers; every buffer that disagrees with it is read or
+// written as loose vectors, and what that costs depends on which they are.  Measured with the phased kernel on
+// 8 x 1 GiB bf16 (7.14 TB/s with everything aligned): seven inputs 4 bytes off the grid 7.00 (-2 %: a loose read on a
+// 4-byte boundary is nearly free), eight inputs 2 bytes off 5.66 (-21 %: off the 4-byte boundary a loose read is
+// dear), the output alone off the grid, by 4 or by 6 bytes, 6.67-6.80 (-5 to -7 %).  So every candidate boundary is
+// priced -- 1 per input that is off it by a multiple of 4 bytes, 8 per input off it otherwise, 16 per output off it --
+// and the cheapest wins, the first destination's among equals.  (A plain majority, the rule before, put the grid on
+// seven peers 4 bytes off and paid for a loose output: 6.67 against 7.00.)
+inline unsigned loose_read_price(unsigned off) {
+    return (off & 15u) == 0 ? 0u : (off & 3u) == 0 ? 1u : 8u;
+}
+constexpr unsigned kLooseWritePrice = 16;
+inline unsigned grid_price(unsigned c, const unsigned* in_mis, int n, const unsigned* out_mis, int m) {
+    unsigned p = 0;
+    for (int j = 0; j < n; j++) p += loose_read_price(in_mis[j] - c);
+    for (int k = 0; k < m; k++) p += ((out_mis[k] - c) & 15u) == 0 ? 0u : kLooseWritePrice;
+    return p;
+}
+// in_mis / out_mis: the buffers' addresses modulo 16; returns the address modulo 16 at which the vectors start
+inline unsigned vector_grid(const unsigned* in_mis, int n, const unsigned* out_mis, int m) {
+    unsigned mis = out_mis[0] & 15u, best = grid_price(mis, in_mis, n, out_mis, m);
+    for (int k = 1; k < m; k++) {
+        const unsigned p = grid_price(out_mis[k], in_mis, n, out_mis, m);
+        if (p < best) { best = p; mis = out_mis[k] & 15u; }
+    }
+    for (int j = 0; j < n; j++) {
+        const unsigned p = grid_price(in_mis[j], in_mis, n, out_mis, m);
+        if (p < best) { best = p; mis = in_mis[j] & 15u; }
+    }
+    return mis;
+}
+
+// ---- when the phased form of a reduce pays -----------------------------------------------------------------------
+// A phase costs a fixed few microseconds on top of its traffic, so what counts is how full the phases are:
+// fill = result vectors / (phases x what one phase holds).  Measured against the streaming kernels (fp32 sum, one
+// destination, rotating buffer sets): with 2 inputs the phased form wins at fill 0.97 (+1 to +8 % from 256 MiB of
+// traffic up) and loses at 0.73; with 3 it wins at 0.73 (+2-3 %) and loses at 0.55; with 4 it wins at 0.58 and loses at
+// 0.44; with 8 it wins from 0.32 (+3 %) and is even at 0.24: about 2 / n.
+inline bool phases_full_enough(uint64_t nvec, uint64_t vectors_per_phase, int n_inputs) {
+    if (nvec == 0 || vectors_per_phase == 0 || n_inputs < 1) return false;
+    const uint64_t phases = (nvec + vectors_per_phase - 1) / vectors_per_phase;
+    const double fill = (double)nvec / (double)(phases * vectors_per_phase);
+    const double need = 2.0 / n_inputs < 0.9 ? 2.0 / n_inputs : 0.9;
+    return fill >= need;
 }
 
 // ---- pack / unpack: the 4 KiB quarters of one tensor, cut where the destination crosses a 128-byte line -------------

@@ -15,7 +15,7 @@
 #include <stddef.h>
 #include <stdint.h>
 
-#define MI_HD_INLINE __host__ __device__ inline
+#include "launch_geometry.hpp"
 
 namespace mi {
 
@@ -941,15 +941,10 @@ inline hipError_t launch_fixed_unroll(const LaunchArgs& a, uint32_t head, uint64
     return launch_fixed<TR, OP, N, kDefault>(a, head, nvec, tail);
 }
 
-// When the phased form pays.  A phase costs a fixed few microseconds on top of its traffic, so what counts is how
-// full the phases are: fill = result bytes / (phases x what one phase holds, 88 MiB on 256 CUs).  Measured against
-// the streaming kernels (fp32 sum, one destination, rotating buffer sets): with 2 inputs the phased form wins at
-// fill 0.97 (+1 to +8 % from 256 MiB of traffic up) and loses at 0.73; with 3 it wins at 0.73 (+2-3 %) and loses at
-// 0.55; with 4 it wins at 0.58 and loses at 0.44; with 8 it wins from 0.32 (+3 %) and is even at 0.24: about 2 / n.
-// Long buffers have fill near 1 and are always phased (+8 % with 2 inputs, +17 % with 8 at 4 GiB of traffic).
-// Several destinations: from 2 x phased_min_bytes of traffic (default 320 MB).  One input stays with the copy and
-// broadcast kernels.  Tuning::phased_min_bytes is a lower bound on the traffic in every case (default 160 MB);
-// Tuning::variant 8 forces the phased form.
+// When the phased form pays: from Tuning::phased_min_bytes of traffic per launch (default 160 MB), with two or more
+// inputs and one destination when its phases are full enough (phases_full_enough: long buffers always are: +8 % with
+// 2 inputs, +17 % with 8 at 4 GiB of traffic), with several destinations from twice that traffic.  One input stays with
+// the copy and broadcast kernels.  Tuning::variant 8 forces the phased form.
 inline bool wants_phased(const LaunchArgs& a, uint64_t nvec, int reg_groups) {
     if (a.tune.sync == nullptr || a.tune.num_cus < kPhaseGroups) return false;
     if (a.tune.variant != 0) return a.tune.variant == 8;
@@ -957,41 +952,18 @@ inline bool wants_phased(const LaunchArgs& a, uint64_t nvec, int reg_groups) {
     if (a.n < 2 || traffic < (uint64_t)a.tune.phased_min_bytes * (a.m > 1 ? 2u : 1u)) return false;
     if (a.m > 1) return true;
     const uint64_t grid = (uint64_t)(a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
-    const uint64_t per_phase = grid * kPhaseBlock * (uint64_t)(4 * reg_groups + kPhaseU);     // vectors
-    const uint64_t phases = (nvec + per_phase - 1) / per_phase;
-    const double fill = (double)nvec / (double)(phases * per_phase);
-    const double need = 2.0 / a.n < 0.9 ? 2.0 / a.n : 0.9;
-    return fill >= need;
+    return phases_full_enough(nvec, grid * kPhaseBlock * (uint64_t)(4 * reg_groups + kPhaseU), a.n);
 }
 
-// Elements before the first vector.  The vectors start on a 16-byte boundary of one of the buffers; the buffers that
-// disagree with it are read and written as loose vectors, and what that costs depends on which they are.  Measured
-// with the phased kernel on 8 x 1 GiB bf16 (7.14 TB/s with everything aligned): seven inputs 4 bytes off the grid
-// 7.00 (-2 %: a loose read on a 4-byte boundary is nearly free), eight inputs 2 bytes off 5.66 (-21 %: off the 4-byte
-// boundary a loose read is dear), the output alone off the grid, by 4 or by 6 bytes, 6.67-6.80 (-5 to -7 %).  So every
-// candidate boundary is priced -- 1 per input that is off it by a multiple of 4 bytes, 8 per input off it otherwise,
-// 16 per output off it -- and the cheapest wins, the first destination's among equals.  (A plain majority, the rule
-// before, put the grid on seven peers 4 bytes off and paid for a loose output: 6.67 against 7.00.)  No head when that
-// boundary is not a multiple of the element size.
-MI_HD_INLINE unsigned loose_read_cost(unsigned off) {
-    return (off & 15u) == 0 ? 0u : (off & 3u) == 0 ? 1u : 8u;
-}
+// Elements before the first vector: the vectors start on the 16-byte boundary that makes the loose accesses of the
+// buffers that disagree with it cheapest (vector_grid).  No head when that boundary is not a multiple of the element
+// size.
 template <class E>
 inline uint64_t vector_head(const LaunchArgs& a) {
     unsigned in_mis[kMaxSrcs], out_mis[kMaxDsts];
     for (int j = 0; j < a.n; j++) in_mis[j] = (unsigned)((uintptr_t)a.srcs[j] & 15u);
     for (int k = 0; k < a.m; k++) out_mis[k] = (unsigned)((uintptr_t)(a.dsts ? a.dsts[k] : a.dst) & 15u);
-    auto price = [&](unsigned c) {
-        unsigned p = 0;
-        for (int j = 0; j < a.n; j++) p += loose_read_cost(in_mis[j] - c);
-        for (int k = 0; k < a.m; k++) p += out_mis[k] == c ? 0u : 16u;
-        return p;
-    };
-    unsigned mis = out_mis[0], best = price(mis);
-    for (int k = 1; k < a.m; k++)
-        if (price(out_mis[k]) < best) best = price(mis = out_mis[k]);
-    for (int j = 0; j < a.n; j++)
-        if (price(in_mis[j]) < best) best = price(mis = in_mis[j]);
+    const unsigned mis = vector_grid(in_mis, a.n, out_mis, a.m);
     return (mis % sizeof(E)) == 0 ? ((16u - mis) & 15u) / sizeof(E) : 0;
 }
 

@@ -144,6 +144,46 @@ int main() {
             for (uint64_t q = nq; q < nq + 4; q++) EXPECT(copy_quarter(total, dst, q).n == 0);
         }
     EXPECT(copy_quarter(0, 0x1000, 0).n == 0);
+    // where a reduce's vectors start: the measured cases, then every choice against a brute-force minimum
+    {
+        const unsigned peers4[8] = { 0, 4, 4, 4, 4, 4, 4, 4 }, in2[8] = { 2, 2, 2, 2, 2, 2, 2, 2 }, al[8] = { 0 };
+        const unsigned spread[8] = { 0, 2, 4, 6, 8, 10, 12, 14 };
+        const unsigned o0[1] = { 0 }, o6[1] = { 6 };
+        EXPECT(vector_grid(peers4, 8, o0, 1) == 0);     // seven peers 4 bytes off: loose reads on 4-byte boundaries are cheap
+        EXPECT(vector_grid(in2, 8, o0, 1) == 2);        // eight inputs 2 bytes off: dearer than one loose output
+        EXPECT(vector_grid(al, 8, o6, 1) == 0);         // the output alone off: it stays loose
+        EXPECT(vector_grid(al, 8, o0, 1) == 0);
+        EXPECT(vector_grid(spread, 8, o0, 1) == 0);
+        EXPECT(vector_grid(in2, 1, o0, 1) == 0);        // one input 2 bytes off costs less than a loose output
+        EXPECT(vector_grid(in2, 2, o0, 1) == 0 && vector_grid(in2, 3, o0, 1) == 2);
+        uint64_t x = 88172645463325252ull;
+        for (int it = 0; it < 20000; it++) {
+            unsigned in[8], out[3];
+            x ^= x << 13; x ^= x >> 7; x ^= x << 17;
+            const int n = 1 + (int)(x % 8), m = 1 + (int)((x >> 8) % 3);
+            const unsigned gran = 1u << ((x >> 16) % 4);        // 1-, 2-, 4- and 8-byte elements
+            for (int j = 0; j < n; j++) in[j] = (unsigned)((x >> (20 + 4 * j)) & 15u) / gran * gran;
+            for (int k = 0; k < m; k++) out[k] = (unsigned)((x >> (52 + 4 * k)) & 15u) / gran * gran;
+            const unsigned g = vector_grid(in, n, out, m);
+            bool is_one = false;
+            unsigned best = ~0u;
+            for (int j = 0; j < n; j++) { is_one |= in[j] == g; const unsigned p = grid_price(in[j], in, n, out, m); if (p < best) best = p; }
+            for (int k = 0; k < m; k++) { is_one |= out[k] == g; const unsigned p = grid_price(out[k], in, n, out, m); if (p < best) best = p; }
+            EXPECT(is_one && grid_price(g, in, n, out, m) == best);
+            EXPECT(grid_price(out[0], in, n, out, m) > best || g == out[0]);    // the first destination's among equals
+        }
+    }
+    // whether the phased form pays: the measured crossovers (one phase holds 88 MiB of results on 256 CUs)
+    {
+        const uint64_t per = 256ull * 512 * 44;
+        auto mib = [](uint64_t m) { return (m << 20) / 16; };
+        EXPECT(phases_full_enough(mib(85), per, 2) && !phases_full_enough(mib(128), per, 2) && phases_full_enough(mib(170), per, 2));
+        EXPECT(phases_full_enough(mib(64), per, 3) && !phases_full_enough(mib(96), per, 3) && phases_full_enough(mib(128), per, 3));
+        EXPECT(phases_full_enough(mib(51), per, 4) && !phases_full_enough(mib(38), per, 4));
+        EXPECT(phases_full_enough(mib(28), per, 8) && !phases_full_enough(mib(21), per, 8));
+        for (int n = 2; n <= 64; n++) EXPECT(phases_full_enough(mib(2000), per, n));    // long buffers always
+        EXPECT(!phases_full_enough(0, per, 8) && !phases_full_enough(100, 0, 8));
+    }
     printf("%d checks, %d failed\n", checks, failed);
     return failed ? 1 : 0;
 }
