@@ -241,7 +241,8 @@ const char* mi_ccl_last_kernel(void);
  * "phased_min_bytes" (scales the sizes from which the phased kernels are used; default 160 MB),
  * "phase_early_loads" / "phase_early_stores" (phased kernels: how many 16-byte loads / stores per lane a block still
  * has to issue when it reports the end of its read / write phase to the chip-wide barrier, which hides the barrier's
- * latency; defaults 12 and -1 = chosen per element type, 4 or 16; 0 = report when done; timing only, results do not
+ * latency; defaults 12 and -1 = chosen per element type, 4 or 16, and 0 with three or more destinations; 0 = report
+ * when the whole block is done and its stores are acknowledged; timing only, results do not
  * depend on them), "phase_spin_ticks" (phased kernels: the longest a block waits at one barrier, in 100 MHz ticks,
  * before it goes on alone and stops waiting for the rest of the launch; default 20000 = 200 us; 0 = never wait, which
  * costs speed only and is what the tests of that path use), "num_cus" (read

@@ -218,6 +218,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                 }
             }
         }
+        if (lead_r == 0) __syncthreads();           // "when done" means the whole block, and its loads have landed
         if (!arrived && tid == 0) phase_arrive(ps);
         phase_wait(ps, ++gen, give_up, spin_ticks);
         const bool more = p0 + per_phase < nitems;
@@ -257,6 +258,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
             }
         }
         if (more) {
+            if (lead_w == 0) __syncthreads();       // "when done": every wave's stores have been acknowledged
             if (!arrived && tid == 0) phase_arrive(ps);
             phase_wait(ps, ++gen, give_up, spin_ticks);
         }
@@ -270,7 +272,7 @@ inline hipError_t launch_fusion_phased(const FusionLaunchArgs& a, const FusionPt
     g_last_kernel = "fusion_reduce_phased_kernel";
     hipLaunchKernelGGL((fusion_reduce_phased_kernel<TR, OP, NT>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, own, out, pp,
                        a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0, a.tune.sync,
-                       a.tune.early_loads, phase_early_stores<TR>(a.tune), a.tune.spin_ticks);
+                       a.tune.early_loads, phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks);
     return hipGetLastError();
 }
 

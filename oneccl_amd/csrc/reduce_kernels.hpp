@@ -802,9 +802,13 @@ template <bool RNE>
 struct PhaseEarlyStores<Bf16KeepTraits<RNE>> {
     static constexpr int value = 4;
 };
+// With three or more destinations a block stores several hundred vectors per lane and phase, its waves drift apart,
+// and an early report from one of them lets the next reads start under far too many outstanding writes: there the
+// block reports when every wave's stores have been acknowledged (8 -> 8 at 1 GiB: 6.27 against 5.79 TB/s, 4 -> 4: 6.20
+// against 5.87; 8 -> 2 and 2 -> 2 still gain 0.5-2 % from the early report).
 template <class TR>
-inline int phase_early_stores(const Tuning& t) {
-    const int v = t.early_stores >= 0 ? t.early_stores : PhaseEarlyStores<TR>::value;
+inline int phase_early_stores(const Tuning& t, int n_dsts) {
+    const int v = t.early_stores >= 0 ? t.early_stores : n_dsts >= 3 ? 0 : PhaseEarlyStores<TR>::value;
     return v < kPhaseU ? v : kPhaseU;
 }
 
@@ -863,6 +867,7 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
 #pragma unroll
             for (int g = 0; g < G; g++) stage[(q * G + g) * kPhaseBlock + threadIdx.x] = v[g];
         }
+        if (early_loads == 0) __syncthreads();      // "when done" means the whole block, and its loads have landed
         if (!arrived && threadIdx.x == 0) phase_arrive(ps);
         phase_wait(ps, ++gen, give_up, spin_ticks);
         const bool more = p0 + per_phase < nvec;
@@ -881,7 +886,10 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
             }
         }
         if (more) {
-            if (arrive_u == kPhaseU && threadIdx.x == 0) phase_arrive(ps);
+            if (arrive_u == kPhaseU) {
+                __syncthreads();                    // "when done": every wave's stores have been acknowledged
+                if (threadIdx.x == 0) phase_arrive(ps);
+            }
             phase_wait(ps, ++gen, give_up, spin_ticks);
         }
     }
@@ -983,7 +991,7 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
         int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
         g_last_kernel = "reduce_multi_phased_kernel";
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
-                           a.m, (uint32_t)head, nvec, tail, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune), a.tune.spin_ticks);
+                           a.m, (uint32_t)head, nvec, tail, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune, a.m), a.tune.spin_ticks);
         return hipGetLastError();
     }
     constexpr int UNROLL = 4;
