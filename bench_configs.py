@@ -13,11 +13,13 @@
   align  buffers that disagree modulo 16 bytes: 8-input bf16 sum at 64 MiB per buffer with every input at its own
          alignment, and with only the output off; the reference's tight fusion layout (alignment 1) of 400 odd-sized
          tensors: pack, unpack and the fused reduce
+  write  a reduce stored to several buffers, and one buffer written to several (the all-gather write side), at 64 MiB
+         and 1 GiB per buffer
   copy   ccl_comp_copy at 64 MiB, 512 MiB and 3 GiB, and the bf16 <-> fp32 array converters at 2^28 elements
 
-    python bench_configs.py [--out results/configs.json] [--skip c3,batch,types,align,copy] [--only c1,c4] [--c3-k 7]
+    python bench_configs.py [--out results/configs.json] [--skip c3,batch,types,align,write,copy] [--only c1,c4] [--c3-k 7]
 
---only runs just the named sections (c1, c2, c3, batch, types, align, copy, c4, latency), --c3-k just the named sizes of
+--only runs just the named sections (c1, c2, c3, batch, types, align, write, copy, c4, latency), --c3-k just the named sizes of
 the sweep (size = 1 KiB x 4^k): what a profiler run of one kernel wants.
 
 EVERY row is checked before it is timed: the first buffer set goes through the call once and the result is compared,
@@ -297,6 +299,27 @@ def main():
             add(f"align: fused reduce against 7 peers, {label}-sized", us, 9 * payload, comp.last_kernel())
             plan.close()
             del tens, outs, fb, peers
+    # ---- several destinations (the write side: a reduce stored to M buffers, one buffer written to M)
+    if want("write"):
+        for n, m, mib in ((8, 8, 1024), (8, 2, 1024), (4, 4, 1024), (2, 2, 1024), (1, 7, 1024), (1, 2, 1024), (8, 8, 64), (2, 2, 64), (1, 7, 64), (1, 2, 64)):
+            cnt = (mib << 20) // 2
+            nsets = 1 if mib >= 512 else max(1, min(4, (3 << 30) // ((n + m) * (mib << 20))))
+            srcs = [[torch.empty(cnt, dtype=torch.bfloat16, device="cuda").normal_(0, 1) for _ in range(n)] for _ in range(nsets)]
+            dsts = [[torch.zeros(cnt, dtype=torch.bfloat16, device="cuda") for _ in range(m)] for _ in range(nsets)]
+            lp = comp.LP_KEEP_PRECISION if n > 1 else comp.LP_PAIRWISE
+            for k in range(m):
+                def once(k=k):
+                    for d in dsts[0]:
+                        d.zero_()
+                    comp.comp_reduce_write_n(comp.BFLOAT16, comp.SUM, srcs[0], dsts[0], cnt, lp_mode=lp)
+                    return dsts[0][k]
+                if k in (0, m - 1):
+                    verify_reduce(f"write {n}->{m} {mib} MiB, destination {k}", O.BFLOAT16, O.SUM, srcs[0], once, cnt, keep=1 if n > 1 else 0)
+            us = timed(torch, lambda i: comp.comp_reduce_write_n(comp.BFLOAT16, comp.SUM, srcs[i % nsets], dsts[i % nsets], cnt, lp_mode=lp),
+                       10 if mib >= 512 else 40, 3)
+            add(f"write: bf16 sum of {n} input{'s' if n > 1 else ''} stored to {m} buffers, {mib} MiB each", us, (n + m) * cnt * 2,
+                f"{nsets} set(s); {comp.last_kernel()}")
+            del srcs, dsts
     # ---- copies and converters
     if want("copy"):
         for mib in (64, 512, 3072):
