@@ -7,7 +7,7 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libmi_ccl_comp.so")
+LIB_PATH = os.environ.get("MI_CCL_COMP_LIB") or os.path.join(HERE, "libmi_ccl_comp.so")     # another build, for A/B runs
 
 # ccl::datatype (include/oneapi/ccl/types.hpp:52-69)
 INT8, UINT8, INT16, UINT16, INT32, UINT32, INT64, UINT64, FLOAT16, FLOAT32, FLOAT64, BFLOAT16 = range(12)

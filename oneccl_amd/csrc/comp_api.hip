@@ -276,7 +276,8 @@ static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void
 
 // Vectors from the output's first 16-byte boundary on; the input is read as loose vectors (any alignment).  One
 // vector per lane and one 4 KiB tile per block, however large the copy: short-lived blocks over a compact window of
-// addresses measure 6.45-6.5 TB/s from 512 MiB up, four vectors per lane 5.9 and the phased one-input reduce 5.9.
+// addresses measure 6.45-6.5 TB/s from 512 MiB up (6.6-6.7 with device-scope stores, st_loose_device_scope), four
+// vectors per lane 5.9 and the phased one-input reduce 5.9.
 template <bool NT>
 __global__ void __launch_bounds__(kBlock)
 copy_kernel(const unsigned char* in, unsigned char* out, uint32_t head, uint64_t nvec, uint32_t tail) {
@@ -284,7 +285,7 @@ copy_kernel(const unsigned char* in, unsigned char* out, uint32_t head, uint64_t
     u32x4* d = (u32x4*)(out + head);
     for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += (uint64_t)gridDim.x * kBlock) {
         if (NT)
-            __builtin_nontemporal_store(ld_loose(s + i), d + i);
+            st_loose_device_scope((u32x4_u*)(d + i), ld_loose(s + i));
         else
             d[i] = *(s + i);
     }
