@@ -107,7 +107,6 @@ inline hipError_t launch_batch_op(const BatchLaunchArgs& a) {
             const uint64_t count = a.counts[j];
             // the vectors of a job start on the 16-byte boundary of the buffer that makes the loose accesses cheapest (vector_head)
             LaunchArgs one;
-            one.tune = a.tune;
             one.srcs = a.srcs + (size_t)j * a.n;
             one.n = a.n;
             one.dst = a.dsts[j];
