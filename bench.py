@@ -336,6 +336,16 @@ def main():
 
     ms_per_step = (t1 - t0) / args.steps * 1e3
     kernel_ms = ev0.elapsed_time(ev1) / args.steps
+    # median and minimum of single launches, each between its own pair of events, after the timed region (not part of
+    # `value` or `kernel_ms`; an event pair per launch adds a few microseconds of its own to short launches)
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for i, (a, b) in enumerate(pairs):
+        a.record(stream)
+        step(i)
+        b.record(stream)
+    torch.cuda.synchronize()
+    singles = sorted(a.elapsed_time(b) for a, b in pairs)
+    launch_ms_median = singles[len(singles) // 2] if len(singles) % 2 else 0.5 * (singles[len(singles) // 2 - 1] + singles[len(singles) // 2])
     kernel = "hipMemcpyDtoDAsync" if probe == "memcpy" else comp.last_kernel()
     value = algo_bytes / (ms_per_step * 1e-3) / 1e9
     achieved = algo_bytes / (kernel_ms * 1e-3) / 1e9
@@ -360,7 +370,8 @@ def main():
                    "parity": "bit-exact vs oracle on the CPU-baseline sample" if base else "not checked in this run"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(args.workload, kernel),
-                     "kernel_ms": round(kernel_ms, 4), "kernel": kernel},
+                     "kernel_ms": round(kernel_ms, 4), "kernel": kernel,
+                     "single_launch_ms_median": round(launch_ms_median, 4), "single_launch_ms_min": round(singles[0], 4)},
         "cpu_baseline": base,
     }
     print(json.dumps(out))
