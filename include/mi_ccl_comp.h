@@ -233,7 +233,8 @@ const char* mi_ccl_last_kernel(void);
 
 /* Launch-shape knobs, the counterpart of CCL_KERNEL_GROUP_SIZE / CCL_KERNEL_MEM_ALIGN
  * (src/common/env/env.cpp:251-253).  Names: "waves_per_cu" (blocks per CU the streaming kernels' grid is capped
- * at; default 256, i.e. one tile per block up to 65,536 blocks), "max_blocks" (cap on the grid; 0 = no cap), "xcd_chunked" (0/1: give each of the 8 XCDs one
+ * at; default 256, i.e. one tile per block up to 65,536 blocks), "max_blocks" (cap on the grid of the streaming kernels, for callers that want CUs left free for other work; 0 = no
+ * cap; while a cap is set the phased kernels, which take one block on every CU, are not chosen), "xcd_chunked" (0/1: give each of the 8 XCDs one
  * contiguous share of the buffer), "variant" (kernel form: 0 = chosen by size and shape; 1, 2, 4 = the streaming
  * kernels with that many vectors per lane where a type has them; 8 = the phased kernels at any size; a non-zero value
  * also keeps one-input calls on the general reduce kernels instead of the copy and broadcast kernels -- for tests and

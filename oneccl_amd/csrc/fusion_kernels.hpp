@@ -298,7 +298,7 @@ inline hipError_t launch_fusion_op(const FusionLaunchArgs& a) {
         const uint64_t traffic = (uint64_t)(a.n_peers + 2) * (i1 - i0) * kFusionChunk;
         const uint64_t from = (uint64_t)a.tune.phased_min_bytes * (a.n_peers == 3 ? 3u : 2u);
         const bool phased = a.tune.sync && a.tune.num_cus >= kPhaseGroups && a.n_peers >= 1 && a.n_peers <= 7 &&
-                            (a.tune.variant == 8 || (a.tune.variant == 0 && a.n_peers >= 3 && traffic >= from));
+                            (a.tune.variant == 8 || (a.tune.variant == 0 && a.tune.max_blocks == 0 && a.n_peers >= 3 && traffic >= from));
         if (phased) {
             switch (a.n_peers) {
                 case 1: e = launch_fusion_phased<TR, OP, 2>(a, own, out, pp, i0, i1, t0); break;

@@ -964,6 +964,7 @@ inline hipError_t launch_fixed_unroll(const LaunchArgs& a, uint32_t head, uint64
 inline bool wants_phased(const LaunchArgs& a, uint64_t nvec, int reg_groups) {
     if (a.tune.sync == nullptr || a.tune.num_cus < kPhaseGroups) return false;
     if (a.tune.variant != 0) return a.tune.variant == 8;
+    if (a.tune.max_blocks > 0) return false;        // a caller that caps the grid keeps CUs free: the phased form takes them all
     const uint64_t traffic = (uint64_t)(a.n + a.m) * nvec * 16u;
     if (a.n < 2 || traffic < (uint64_t)a.tune.phased_min_bytes * (a.m > 1 ? 2u : 1u)) return false;
     if (a.m > 1) return true;

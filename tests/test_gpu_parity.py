@@ -459,6 +459,27 @@ def test_phased_kernel_early_arrival_settings(comp, dtype, op, n, m):
         comp.set_param("phase_early_stores", -1)
 
 
+def test_grid_cap_keeps_the_streaming_kernels(comp):
+    """"max_blocks" caps the grid for callers that want CUs left free; the phased kernels take one block on every CU, so
+    while a cap is set a large reduce stays with the (grid-striding) streaming kernels -- same bits either way."""
+    import torch
+    rng = np.random.default_rng(78)
+    count = 40 << 20                 # 8 x 80 MiB of bf16: phased without a cap
+    srcs = make_inputs(rng, O.BFLOAT16, count, O.SUM, 8)
+    want = O.reduce_n(srcs, O.BFLOAT16, O.SUM, keep=1, threads=16)
+    d = [to_dev(s) for s in srcs]
+    try:
+        for cap, kernel in ((0, "reduce_multi_phased_kernel"), (64, "reduce_multi_kernel"), (1, "reduce_multi_kernel")):
+            comp.set_param("max_blocks", cap)
+            out = torch.zeros_like(d[0])
+            comp.comp_reduce_n(O.BFLOAT16, O.SUM, d, out, count, lp_mode=comp.LP_KEEP_PRECISION)
+            torch.cuda.synchronize()
+            assert comp.last_kernel() == kernel, (cap, comp.last_kernel())
+            assert_same(to_host(out, np.uint16), want, O.BFLOAT16, f"grid cap {cap}", srcs, O.SUM, keep=1)
+    finally:
+        comp.set_param("max_blocks", 0)
+
+
 def test_phased_kernel_when_no_block_waits(comp):
     """The bound on a block's wait at the chip-wide barrier set to zero from the host: every block goes on alone after
     its first poll, the phases of different blocks overlap freely, and the result is still the oracle's (the barrier
