@@ -128,17 +128,20 @@ __device__ __forceinline__ uint32_t f32_step_bits(uint32_t in, uint32_t io) {
 // element traits: elem_t (storage), acc_t (what is carried between steps), init / step / finish
 
 // Integers and fp32/fp64 (CCL_REDUCE, comp.cpp:31-58).  Integer sum/prod are done on the unsigned type of
-// the same width (two's-complement wrap).  min/max: ties and unordered operands return `in`.
+// the same width (two's-complement wrap); 8- and 16-bit operands are lifted to `unsigned` first, because the
+// language would promote them to a signed int, which 65535 * 65535 overflows.  min/max: ties and unordered
+// operands return `in`.
 template <class T, class U>
 struct PlainTraits {
     typedef T elem_t;
     typedef T acc_t;
+    typedef decltype(U() + 0u) W;       // unsigned for the narrow types, U itself from 32 bits up
     static constexpr int VEC = 16 / sizeof(T);
     static __device__ __forceinline__ acc_t init(elem_t x) { return x; }
     template <int OP>
     static __device__ __forceinline__ acc_t step(elem_t in, acc_t io) {
-        if (OP == OP_SUM) return (T)((U)io + (U)in);
-        if (OP == OP_PROD) return (T)((U)io * (U)in);
+        if (OP == OP_SUM) return (T)(U)((W)(U)io + (W)(U)in);
+        if (OP == OP_PROD) return (T)(U)((W)(U)io * (W)(U)in);
         if (OP == OP_MIN) return (io < in) ? io : in;
         return (in < io) ? io : in;
     }

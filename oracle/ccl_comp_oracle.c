@@ -167,7 +167,9 @@ static inline float f32_step(float in, float io, int op, int vec_sem) {
 
 /* CCL_REDUCE(type), comp.cpp:31-58.  Sum and product of integers are done on the unsigned type of
  * the same width: the reference's signed `+=`/`*=` wraps in practice and that is the defined result
- * here. */
+ * here.  ORC_UWIDE lifts an 8- or 16-bit operand to `unsigned` first (C would promote it to a signed
+ * int, and 65535 * 65535 overflows one); wider types stay as they are. */
+#define ORC_UWIDE(x) ((x) + 0u)
 #define DEFINE_REDUCE_INT(name, T, U)                                                \
     static void name(const void* in_, size_t n, void* io_, int op) {                 \
         const T* in = (const T*)in_;                                                 \
@@ -175,10 +177,10 @@ static inline float f32_step(float in, float io, int op, int vec_sem) {
         size_t i;                                                                    \
         switch (op) {                                                                \
             case ORC_SUM:                                                            \
-                for (i = 0; i < n; i++) io[i] = (T)(U)((U)io[i] + (U)in[i]);         \
+                for (i = 0; i < n; i++) io[i] = (T)(U)(ORC_UWIDE((U)io[i]) + ORC_UWIDE((U)in[i])); \
                 break;                                                               \
             case ORC_PROD:                                                           \
-                for (i = 0; i < n; i++) io[i] = (T)(U)((U)io[i] * (U)in[i]);         \
+                for (i = 0; i < n; i++) io[i] = (T)(U)(ORC_UWIDE((U)io[i]) * ORC_UWIDE((U)in[i])); \
                 break;                                                               \
             case ORC_MIN:                                                            \
                 for (i = 0; i < n; i++) io[i] = STD_MIN(in[i], io[i]);               \

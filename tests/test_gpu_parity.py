@@ -367,6 +367,33 @@ def test_all_pairs_of_16bit_values_sum_and_prod(comp, dtype, impl):
             assert_same(to_host(db, np.uint16), want, dtype, f"op={op} rows from {r0}", [b, a], op, bf16_impl=impl, fp16_impl=3)
 
 
+@pytest.mark.parametrize("dtype", [O.INT16, O.UINT16])
+def test_all_pairs_of_16bit_integers_sum_and_prod(comp, dtype):
+    """Every (in, inout) pair of 16-bit integer patterns -- 2^32 pairs -- through the GPU kernel: the wrapped sum and
+    product (65535 x 65535 overflows a signed int, so both sides multiply in unsigned).  Checked against the oracle
+    and against the closed form on 32-bit unsigned integers, which shares no code with either."""
+    import torch
+    np_t = O.NP_STORAGE[dtype]
+    allv = np.arange(65536, dtype=np.uint16)
+    rows = 512
+    a = np.tile(allv, rows)
+    da = to_dev(a.view(np_t))
+    a32 = a.astype(np.uint32)
+    for op in (O.SUM, O.PROD):
+        for r0 in range(0, 65536, rows):
+            b = np.repeat(allv[r0:r0 + rows], 65536)
+            db = to_dev(b.view(np_t))
+            comp.comp_reduce(dtype, op, da, a.size, db)
+            torch.cuda.synchronize()
+            got = to_host(db, np_t).view(np.uint16)
+            b32 = b.astype(np.uint32)
+            closed = ((b32 + a32) if op == O.SUM else (b32 * a32)).astype(np.uint16)     # modulo 2^32, then modulo 2^16
+            assert (got == closed).all(), (dtype, op, r0, "closed form")
+            if r0 % (16 * rows) == 0 or r0 + rows == 65536:
+                want = O.reduce_n([b.view(np_t), a.view(np_t)], dtype, op, threads=16)
+                assert (got == want.view(np.uint16)).all(), (dtype, op, r0, "oracle")
+
+
 def test_arguments_and_errors(comp):
     import torch
     L = comp.lib()

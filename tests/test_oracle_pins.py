@@ -250,6 +250,23 @@ def test_int_ops_vs_python_big_integers(dtype, op):
         assert int(got[i]) == w, (dtype, op, x, y)
 
 
+@pytest.mark.parametrize("dtype", [O.INT16, O.UINT16, O.INT8, O.UINT8])
+def test_narrow_int_products_wrap_where_a_signed_int_would_overflow(dtype):
+    """Every value of the type times a set of rows that includes the largest magnitudes (65535 x 65535 = 0xFFFE0001 does
+    not fit a signed int, which is what the operands of a 16-bit multiply are promoted to): the wrapped product on
+    32-bit unsigned integers is the expected result."""
+    np_t = O.NP_STORAGE[dtype]
+    bits = np.iinfo(np_t).bits
+    allv = np.arange(1 << bits, dtype=np.uint32)
+    rows = np.unique(np.concatenate([np.array([0, 1, 2, 0x7FFF, 0x8000, 0x8001, 0xB504, 0xB505, 0xFFFE, 0xFFFF], np.uint32) & ((1 << bits) - 1),
+                                     np.random.default_rng(16).integers(0, 1 << bits, 54, dtype=np.uint32)]))
+    a = np.tile(allv, rows.size)
+    b = np.repeat(rows, allv.size)
+    u_t = np.uint16 if bits == 16 else np.uint8
+    got = O.comp_reduce(a.astype(u_t).view(np_t), b.astype(u_t).view(np_t), dtype, O.PROD)
+    assert (got.view(u_t) == (a * b).astype(u_t)).all()
+
+
 @pytest.mark.parametrize("dtype,np_t", [(O.FLOAT32, np.float32), (O.FLOAT64, np.float64)])
 def test_fp_sum_prod_are_single_ieee_ops_in_chain_order(dtype, np_t):
     rng = np.random.default_rng(3)
