@@ -200,15 +200,18 @@ int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* ow
 
 /* The same fused reduce for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc): no plan, and no hipMalloc, hipFree or other allocating call -- the work
- * table that a plan keeps in memory of its own lives in an array inside the library (about 1 MiB per GPU, held until
- * the process ends) and is rewritten by a small kernel on `stream` in front of the reduce of every call.  The layout
- * is given directly: counts[k] elements of `dtype`, starts rounded up to `align` bytes (as mi_ccl_fusion_offsets).
- * Same results as mi_ccl_fusion_reduce on a plan of the same layout.  Limits: k <= MI_CCL_FUSION_STATIC_MAX_TENSORS and
- * at most MI_CCL_FUSION_STATIC_MAX_ITEMS pieces of 16 KiB (a tensor takes ceil(bytes / 16384) of them: 2 GiB of payload
- * when the tensors are multiples of 16 KiB); beyond either the call returns out_of_resource and does nothing.  All
- * calls on one GPU share the one table: calls on the same stream are ordered, calls that overlap on different
- * streams of one GPU race (results undefined).  The first call on a GPU looks the array's address up; make that call
- * outside a capture.  This entry point has no counterpart in the reference. */
+ * table that a plan keeps in memory of its own lives in an array inside the library (four tables of about 1 MiB per
+ * GPU, held until the process ends); a call takes the next table in turn and a small kernel on `stream` rewrites it in
+ * front of the reduce.  The layout is given directly: counts[k] elements of `dtype`, starts rounded up to `align` bytes
+ * (as mi_ccl_fusion_offsets).  Same results as mi_ccl_fusion_reduce on a plan of the same layout.  Limits:
+ * k <= MI_CCL_FUSION_STATIC_MAX_TENSORS and at most MI_CCL_FUSION_STATIC_MAX_ITEMS pieces of 16 KiB (a tensor takes
+ * ceil(bytes / 16384) of them: 2 GiB of payload when the tensors are multiples of 16 KiB); beyond either the call returns
+ * out_of_resource and does nothing.  Calls on the same stream are ordered.  A table comes round again with the fourth
+ * call after it on that GPU: up to four calls may overlap on different streams (or sit in graphs that replay side by
+ * side); a call that is still running when the fourth call after it starts races with it (results undefined) -- keep
+ * at most four in flight per GPU, or order them on one stream; a call captured into a graph keeps, in every replay,
+ * the table it took at capture, so order a graph's replays with whatever else may reach that table.  The first call on a GPU looks the array's address up;
+ * make that call outside a capture.  This entry point has no counterpart in the reference. */
 #define MI_CCL_FUSION_STATIC_MAX_TENSORS 1024
 #define MI_CCL_FUSION_STATIC_MAX_ITEMS 131072
 int mi_ccl_fusion_reduce_static(const size_t* counts, size_t k, int dtype, size_t align, int op,

@@ -5,6 +5,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
+
 #include "../../include/mi_ccl_comp.h"
 
 namespace {
@@ -49,6 +51,11 @@ ccl::env_data parse_env() {
         if (!enum_by_name(fp16_env_impl_names, v, e.fp16_impl_type))
             fail(std::string("unsupported FP16 impl type: ") + v);
     }
+    if (const char* v = getenv("MI_CCL_CHECK_POINTERS")) {
+        if (strlen(v) != 1 || v[0] < '0' || v[0] > '2')
+            fail(std::string("unexpected MI_CCL_CHECK_POINTERS value (0, 1 or 2): ") + v);
+        e.check_pointers = v[0] - '0';
+    }
     return e;
 }
 
@@ -73,18 +80,102 @@ int bf16_impl() {
     return (int)ccl::global_data::env().bf16_impl_type;
 }
 
-// ccl::reduction::custom: the callback is host code, so both buffers are staged to the host and the result is
-// copied back, blocking, exactly as the reference does for device USM buffers (comp.cpp:163-194).
+// ---- which memory a pointer names ----------------------------------------------------------------------------
+// The reference looks at both pointers before it picks a path (sycl::get_pointer_type, src/comp/comp.cpp:147-161).
+// Here every path is a kernel, and a kernel that is handed pageable host memory takes a GPU memory fault, so the
+// functions below refuse such a pointer before anything is enqueued.  Memory the GPU can reach (device, managed,
+// pinned host) is accepted.  The answer is remembered per allocation and per thread (hipMemGetAddressRange gives the
+// allocation's extent), so a steady-state call costs a search of a short sorted list; env().check_pointers = 2 asks
+// the runtime on every call (for callers that free and map memory between calls), 0 switches the check off.
+struct known_range {
+    uintptr_t lo, hi;
+};
+thread_local std::vector<known_range> t_known;      // sorted by lo, disjoint
+thread_local known_range t_last = { 0, 0 };         // the range of the most recent hit: neighbours in one table mostly share it
+
+bool gpu_can_reach(const void* p, uintptr_t* lo, uintptr_t* hi) {
+    hipPointerAttribute_t a;
+    memset(&a, 0, sizeof(a));
+    if (hipPointerGetAttributes(&a, p) != hipSuccess) {
+        (void)hipGetLastError();        // the runtime's answer for memory it has never seen; not an error of this thread's
+        return false;
+    }
+    if (a.type == hipMemoryTypeUnregistered)
+        return false;
+    *lo = *hi = 0;
+    hipDeviceptr_t base = nullptr;
+    size_t size = 0;
+    if (hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)p) == hipSuccess && size) {
+        *lo = (uintptr_t)base;
+        *hi = *lo + size;
+    }
+    else {
+        (void)hipGetLastError();
+    }
+    return true;
+}
+
+void require_gpu_memory(const void* p, size_t bytes, const char* fn, const char* arg) {
+    const int mode = ccl::global_data::env().check_pointers;
+    if (mode == 0 || !p || !bytes)
+        return;                         // null pointers are the C ABI's to refuse
+    const uintptr_t a = (uintptr_t)p;
+    if (mode == 1) {
+        if (a >= t_last.lo && a + bytes <= t_last.hi)
+            return;
+        auto it = std::upper_bound(t_known.begin(), t_known.end(), a,
+                                   [](uintptr_t v, const known_range& r) { return v < r.lo; });
+        if (it != t_known.begin() && a < (it - 1)->hi) {
+            if (a + bytes > (it - 1)->hi)
+                fail(std::string(fn) + ": " + arg + " runs past the end of its allocation");
+            t_last = *(it - 1);
+            return;
+        }
+    }
+    uintptr_t lo = 0, hi = 0;
+    if (!gpu_can_reach(p, &lo, &hi))
+        fail(std::string(fn) + ": " + arg + " is not memory the GPU can reach (pageable host memory?); this build "
+             "reduces device buffers only");
+    if (hi > lo) {
+        if (a + bytes > hi)
+            fail(std::string(fn) + ": " + arg + " runs past the end of its allocation");
+        if (mode == 1) {
+            if (t_known.size() >= 256)
+                t_known.clear();
+            t_last = known_range{ 0, 0 };
+            // a new allocation may cover addresses of remembered ones that have been freed since: drop those
+            t_known.erase(std::remove_if(t_known.begin(), t_known.end(),
+                                         [&](const known_range& r) { return r.lo < hi && lo < r.hi; }),
+                          t_known.end());
+            t_known.insert(std::upper_bound(t_known.begin(), t_known.end(), lo,
+                                            [](uintptr_t v, const known_range& r) { return v < r.lo; }),
+                           known_range{ lo, hi });
+        }
+    }
+}
+
+bool is_gpu_memory(const void* p) {
+    uintptr_t lo, hi;
+    return gpu_can_reach(p, &lo, &hi);
+}
+
+// ccl::reduction::custom: the callback is host code.  With two host buffers it is called on them as they are
+// (comp.cpp:84-88, the reference's host path); when either buffer is GPU memory both are staged to the host and the
+// result is copied back, blocking, exactly as the reference does for device USM buffers (comp.cpp:163-194).
 void custom_on_host(ccl_sched* sched, const void* in_buf, size_t in_count, void* inout_buf, size_t* out_count,
                     const ccl_datatype& dtype, ccl::reduction_fn fn, const ccl::fn_context* context) {
+    if (ccl::global_data::env().check_pointers != 0 && !is_gpu_memory(in_buf) && !is_gpu_memory(inout_buf)) {
+        fn(in_buf, in_count, inout_buf, out_count, dtype.idx(), context);
+        return;
+    }
     hipStream_t s = (hipStream_t)stream_of(sched);
     const size_t bytes = in_count * dtype.size();
     std::vector<unsigned char> h_in(bytes), h_io(bytes);
-    check_hip(hipMemcpyAsync(h_in.data(), in_buf, bytes, hipMemcpyDeviceToHost, s), "custom reduction: copy in");
-    check_hip(hipMemcpyAsync(h_io.data(), inout_buf, bytes, hipMemcpyDeviceToHost, s), "custom reduction: copy in");
+    check_hip(hipMemcpyAsync(h_in.data(), in_buf, bytes, hipMemcpyDefault, s), "custom reduction: copy in");
+    check_hip(hipMemcpyAsync(h_io.data(), inout_buf, bytes, hipMemcpyDefault, s), "custom reduction: copy in");
     check_hip(hipStreamSynchronize(s), "custom reduction: sync");
     fn(h_in.data(), in_count, h_io.data(), out_count, dtype.idx(), context);
-    check_hip(hipMemcpyAsync(inout_buf, h_io.data(), bytes, hipMemcpyHostToDevice, s), "custom reduction: copy out");
+    check_hip(hipMemcpyAsync(inout_buf, h_io.data(), bytes, hipMemcpyDefault, s), "custom reduction: copy out");
     check_hip(hipStreamSynchronize(s), "custom reduction: sync");
 }
 
@@ -183,7 +274,14 @@ std::set<ccl_fp16_impl_type> ccl_fp16_get_impl_types() {
     return { ccl_fp16_f16c, ccl_fp16_avx512f, ccl_fp16_avx512fp16 };
 }
 
+void ccl_comp_forget_pointers() {
+    t_known.clear();
+    t_last = known_range{ 0, 0 };
+}
+
 ccl::status ccl_comp_copy(const void* in_buf, void* out_buf, size_t bytes, bool use_nontemporal, ccl_sched* sched) {
+    require_gpu_memory(in_buf, bytes, "ccl_comp_copy", "in_buf");
+    require_gpu_memory(out_buf, bytes, "ccl_comp_copy", "out_buf");
     return to_status(mi_ccl_comp_copy(in_buf, out_buf, bytes, use_nontemporal ? 1 : 0, stream_of(sched)),
                      "ccl_comp_copy");
 }
@@ -204,6 +302,8 @@ ccl::status ccl_comp_reduce(ccl_sched* sched, const void* in_buf, size_t in_coun
         *out_count = in_count;
     if (!fp16_mode(dtype))
         return ccl::status::success;        // float16 without an implementation selected: inout stays as it is
+    require_gpu_memory(in_buf, in_count * dtype.size(), "ccl_comp_reduce", "in_buf");
+    require_gpu_memory(inout_buf, in_count * dtype.size(), "ccl_comp_reduce", "inout_buf");
     return to_status(mi_ccl_comp_reduce((int)dtype.idx(), (int)reduction, in_buf, in_count, inout_buf,
                                         bf16_impl(), fp16_impl_or_default(), stream_of(sched)),
                      "ccl_comp_reduce");
@@ -229,6 +329,10 @@ ccl::status ccl_comp_batch_reduce(const void* in_buf, const std::vector<size_t>&
         *out_count = in_count;
     if (!fp16_mode(dtype))
         return ccl::status::success;        // every pairwise call of the chain leaves inout as it is
+    require_gpu_memory(inout_buf, in_count * dtype.size(), "ccl_comp_batch_reduce", "inout_buf");
+    for (size_t i = 1; i < offsets.size(); i++)
+        require_gpu_memory((const char*)in_buf + dtype.size() * offsets[i], in_count * dtype.size(), "ccl_comp_batch_reduce",
+                           "a slice of in_buf");
     return to_status(mi_ccl_comp_batch_reduce(in_buf, offsets.data(), offsets.size(), in_count, inout_buf,
                                               (int)dtype.idx(), (int)reduction, bf16_keep_precision_mode,
                                               bf16_impl(), fp16_impl_or_default(), stream_of(sched)),
@@ -239,6 +343,8 @@ void ccl_bf16_reduce(const void* in_buf, size_t in_cnt, void* inout_buf, size_t*
                      ccl_sched* sched) {
     if (out_cnt)
         *out_cnt = in_cnt;                                             // bf16.cpp:94-96
+    require_gpu_memory(in_buf, in_cnt * 2, "ccl_bf16_reduce", "in_buf");
+    require_gpu_memory(inout_buf, in_cnt * 2, "ccl_bf16_reduce", "inout_buf");
     to_status(mi_ccl_bf16_reduce(in_buf, in_cnt, inout_buf, (int)reduction_op,
                                  (int)ccl::global_data::env().bf16_impl_type, stream_of(sched)),
               "ccl_bf16_reduce");
@@ -250,45 +356,63 @@ void ccl_fp16_reduce(const void* in_buf, size_t in_cnt, void* inout_buf, size_t*
         *out_cnt = in_cnt;                                             // fp16.cpp:48-50
     if (!fp16_mode(ccl_datatype_storage::instance().get(ccl::datatype::float16)))
         return;
+    require_gpu_memory(in_buf, in_cnt * 2, "ccl_fp16_reduce", "in_buf");
+    require_gpu_memory(inout_buf, in_cnt * 2, "ccl_fp16_reduce", "inout_buf");
     to_status(mi_ccl_fp16_reduce(in_buf, in_cnt, inout_buf, (int)reduction_op, fp16_impl(), stream_of(sched)),
               "ccl_fp16_reduce");
 }
 
 void ccl_convert_fp32_to_bf16_arrays(void* fp32_buf, void* bf16_buf, size_t count, ccl_sched* sched) {
+    require_gpu_memory(fp32_buf, count * 4, "ccl_convert_fp32_to_bf16_arrays", "fp32_buf");
+    require_gpu_memory(bf16_buf, count * 2, "ccl_convert_fp32_to_bf16_arrays", "bf16_buf");
     to_status(mi_ccl_convert_fp32_to_bf16_arrays(fp32_buf, bf16_buf, count,
                                                  (int)ccl::global_data::env().bf16_impl_type, stream_of(sched)),
               "ccl_convert_fp32_to_bf16_arrays");
 }
 
 void ccl_convert_bf16_to_fp32_arrays(void* bf16_buf, float* fp32_buf, size_t count, ccl_sched* sched) {
+    require_gpu_memory(bf16_buf, count * 2, "ccl_convert_bf16_to_fp32_arrays", "bf16_buf");
+    require_gpu_memory(fp32_buf, count * 4, "ccl_convert_bf16_to_fp32_arrays", "fp32_buf");
     to_status(mi_ccl_convert_bf16_to_fp32_arrays(bf16_buf, fp32_buf, count, stream_of(sched)),
               "ccl_convert_bf16_to_fp32_arrays");
 }
 
 void ccl_convert_fp32_to_bf16(const void* src, void* dst, ccl_sched* sched) {
+    require_gpu_memory(src, 16 * 4, "ccl_convert_fp32_to_bf16", "src");
+    require_gpu_memory(dst, 16 * 2, "ccl_convert_fp32_to_bf16", "dst");
     // bf16.cpp:113-123: the avx512bf store when that implementation is selected, the truncating one otherwise
     const int impl = ccl::global_data::env().bf16_impl_type == ccl_bf16_avx512bf ? MI_CCL_BF16_AVX512BF : MI_CCL_BF16_AVX512F;
     to_status(mi_ccl_convert_fp32_to_bf16_arrays(src, dst, 16, impl, stream_of(sched)), "ccl_convert_fp32_to_bf16");
 }
 
 void ccl_convert_bf16_to_fp32(const void* src, void* dst, ccl_sched* sched) {
+    require_gpu_memory(src, 16 * 2, "ccl_convert_bf16_to_fp32", "src");
+    require_gpu_memory(dst, 16 * 4, "ccl_convert_bf16_to_fp32", "dst");
     to_status(mi_ccl_convert_bf16_to_fp32_arrays(src, dst, 16, stream_of(sched)), "ccl_convert_bf16_to_fp32");
 }
 
 void ccl_convert_fp32_to_fp16(const void* src, void* dst, ccl_sched* sched) {
+    require_gpu_memory(src, 8 * 4, "ccl_convert_fp32_to_fp16", "src");
+    require_gpu_memory(dst, 8 * 2, "ccl_convert_fp32_to_fp16", "dst");
     to_status(mi_ccl_convert_fp32_to_fp16_arrays(src, dst, 8, stream_of(sched)), "ccl_convert_fp32_to_fp16");
 }
 
 void ccl_convert_fp16_to_fp32(const void* src, void* dst, ccl_sched* sched) {
+    require_gpu_memory(src, 8 * 2, "ccl_convert_fp16_to_fp32", "src");
+    require_gpu_memory(dst, 8 * 4, "ccl_convert_fp16_to_fp32", "dst");
     to_status(mi_ccl_convert_fp16_to_fp32_arrays(src, dst, 8, stream_of(sched)), "ccl_convert_fp16_to_fp32");
 }
 
 void ccl_convert_fp32_to_fp16_arrays(const void* fp32_buf, void* fp16_buf, size_t count, ccl_sched* sched) {
+    require_gpu_memory(fp32_buf, count * 4, "ccl_convert_fp32_to_fp16_arrays", "fp32_buf");
+    require_gpu_memory(fp16_buf, count * 2, "ccl_convert_fp32_to_fp16_arrays", "fp16_buf");
     to_status(mi_ccl_convert_fp32_to_fp16_arrays(fp32_buf, fp16_buf, count, stream_of(sched)),
               "ccl_convert_fp32_to_fp16_arrays");
 }
 
 void ccl_convert_fp16_to_fp32_arrays(const void* fp16_buf, float* fp32_buf, size_t count, ccl_sched* sched) {
+    require_gpu_memory(fp16_buf, count * 2, "ccl_convert_fp16_to_fp32_arrays", "fp16_buf");
+    require_gpu_memory(fp32_buf, count * 4, "ccl_convert_fp16_to_fp32_arrays", "fp32_buf");
     to_status(mi_ccl_convert_fp16_to_fp32_arrays(fp16_buf, fp32_buf, count, stream_of(sched)),
               "ccl_convert_fp16_to_fp32_arrays");
 }
@@ -304,6 +428,8 @@ ccl::status ccl_comp_reduce_n(ccl_sched* sched, const void* own_buf, const std::
     srcs.reserve(peer_bufs.size() + 1);
     srcs.push_back(own_buf);
     srcs.insert(srcs.end(), peer_bufs.begin(), peer_bufs.end());
+    for (const void* p : srcs) require_gpu_memory(p, count * dtype.size(), "ccl_comp_reduce_n", "an input buffer");
+    require_gpu_memory(out_buf, count * dtype.size(), "ccl_comp_reduce_n", "out_buf");
     int lp = bf16_keep_precision_mode ? MI_CCL_LP_KEEP_PRECISION : MI_CCL_LP_PAIRWISE;
     return to_status(mi_ccl_comp_reduce_n((int)dtype.idx(), (int)reduction, srcs.data(), (int)srcs.size(), out_buf,
                                           count, lp, bf16_impl(), fp16_impl_or_default(), stream_of(sched)),
@@ -321,6 +447,8 @@ ccl::status ccl_comp_reduce_write_n(ccl_sched* sched, const void* own_buf, const
     srcs.reserve(peer_bufs.size() + 1);
     srcs.push_back(own_buf);
     srcs.insert(srcs.end(), peer_bufs.begin(), peer_bufs.end());
+    for (const void* p : srcs) require_gpu_memory(p, count * dtype.size(), "ccl_comp_reduce_write_n", "an input buffer");
+    for (const void* p : out_bufs) require_gpu_memory(p, count * dtype.size(), "ccl_comp_reduce_write_n", "an output buffer");
     int lp = bf16_keep_precision_mode ? MI_CCL_LP_KEEP_PRECISION : MI_CCL_LP_PAIRWISE;
     return to_status(mi_ccl_comp_reduce_write_n((int)dtype.idx(), (int)reduction, srcs.data(), (int)srcs.size(),
                                                 out_bufs.data(), (int)out_bufs.size(), count, lp,
@@ -337,6 +465,13 @@ ccl::status ccl_comp_reduce_batch(ccl_sched* sched, const std::vector<const void
         fail("custom reduction is not available for the batched device reduce");
     if (n_inputs < 1 || counts.size() != dsts.size() || srcs.size() != dsts.size() * (size_t)n_inputs)
         fail("ccl_comp_reduce_batch: srcs must hold n_inputs pointers per job, dsts and counts one entry per job");
+    for (size_t j = 0; j < dsts.size(); j++) {
+        if (!counts[j])
+            continue;                       // an empty job's pointers are not looked at
+        for (int k = 0; k < n_inputs; k++)
+            require_gpu_memory(srcs[j * n_inputs + k], counts[j] * dtype.size(), "ccl_comp_reduce_batch", "an input buffer");
+        require_gpu_memory(dsts[j], counts[j] * dtype.size(), "ccl_comp_reduce_batch", "an output buffer");
+    }
     int lp = bf16_keep_precision_mode ? MI_CCL_LP_KEEP_PRECISION : MI_CCL_LP_PAIRWISE;
     return to_status(mi_ccl_comp_reduce_batch((int)dtype.idx(), (int)reduction, srcs.data(), n_inputs, dsts.data(),
                                               counts.data(), (int)dsts.size(), lp, bf16_impl(), fp16_impl_or_default(),

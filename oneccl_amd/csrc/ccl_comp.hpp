@@ -11,7 +11,10 @@
 //   * an unknown dtype or reduction throws ccl::exception where the reference calls CCL_FATAL
 //     (std::terminate, src/comp/comp.cpp:56,113).
 //   * ccl::reduction::custom runs the user's host callback on host copies of the two buffers, as the
-//     reference does for device buffers (src/comp/comp.cpp:163-194).
+//     reference does for device buffers (src/comp/comp.cpp:163-194), and on the buffers themselves when both
+//     are host memory (src/comp/comp.cpp:84-88).
+//   * a buffer of pageable host memory is refused with ccl::exception before anything is enqueued (the
+//     reference reduces it on the host; here every path is a kernel): see env_data::check_pointers.
 #pragma once
 
 #include <stddef.h>
@@ -102,6 +105,12 @@ namespace ccl {
 struct env_data {
     ccl_bf16_impl_type bf16_impl_type = ccl_bf16_avx512bf;
     ccl_fp16_impl_type fp16_impl_type = ccl_fp16_avx512f;
+    // What the functions below do about a buffer that is not GPU memory (the reference classifies its pointers,
+    // src/comp/comp.cpp:147-161, and reduces host buffers on the host; here every path is a kernel, and a kernel
+    // handed pageable host memory is a GPU memory fault): 1 = refuse it with ccl::exception before anything is
+    // enqueued, remembering per thread which allocations have been seen (the default; MI_CCL_CHECK_POINTERS);
+    // 2 = the same, asking the runtime on every call; 0 = no check, for callers that guarantee device memory.
+    int check_pointers = 1;
 };
 struct global_data {
     static env_data& env();
@@ -163,6 +172,10 @@ struct ccl_sched {
     void renew();                               // every entry back to not_started, for the next run of the schedule
     void* alloc_buffer(size_t bytes);           // device memory owned by the schedule (sched_base.cpp alloc_buffer)
 };
+
+// Drops what this thread remembers about allocations it has seen (env_data::check_pointers = 1): for a caller that
+// frees device memory and may get the same addresses back as host memory.
+void ccl_comp_forget_pointers();
 
 // src/comp/comp.hpp:23-51
 ccl::status ccl_comp_copy(const void* in_buf, void* out_buf, size_t bytes, bool use_nontemporal = false,

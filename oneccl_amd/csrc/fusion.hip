@@ -3,11 +3,11 @@
 
 #include <atomic>
 #include <new>
+#include <stdexcept>
 #include <vector>
 
 #include "../../include/mi_ccl_comp.h"
 #include "fusion_kernels.hpp"
-#include "launch_geometry.hpp"
 #include "launch_geometry.hpp"
 
 namespace mi {
@@ -136,8 +136,14 @@ struct StaticFusionTable {
     uint64_t bytes[MI_CCL_FUSION_STATIC_MAX_TENSORS];
     FusionItem items[MI_CCL_FUSION_STATIC_MAX_ITEMS];
 };
-static __device__ __align__(256) unsigned char scratch[sizeof(StaticFusionTable)];
+// kStaticSlots tables per GPU, taken in turn by the calls on that GPU: a call's table is rewritten by the call that
+// comes kStaticSlots calls later, so up to that many calls may be in flight on different streams (or sit in graphs
+// that replay side by side) before two of them share a table.
+constexpr int kStaticSlots = 4;
+static __device__ __align__(256) unsigned char scratch[kStaticSlots * sizeof(StaticFusionTable)];
+static_assert(sizeof(StaticFusionTable) % 256 == 0, "every table of the array starts on a 256-byte boundary");
 static std::atomic<StaticFusionTable*> g_scratch_ptr[64];
+static std::atomic<unsigned> g_scratch_next[64];
 
 static hipError_t scratch_table(StaticFusionTable** out) {
     int dev = 0;
@@ -155,7 +161,7 @@ static hipError_t scratch_table(StaticFusionTable** out) {
         p = (StaticFusionTable*)ptr;
         g_scratch_ptr[dev].store(p, std::memory_order_release);
     }
-    *out = p;
+    *out = p + g_scratch_next[dev].fetch_add(1, std::memory_order_relaxed) % kStaticSlots;
     return hipSuccess;
 }
 
@@ -221,16 +227,8 @@ int mi_ccl_fusion_offsets(const size_t* counts, size_t k, size_t dtype_size, siz
     return MI_CCL_SUCCESS;
 }
 
-int mi_ccl_fusion_plan_create(const size_t* counts, size_t k, int dtype, size_t align, mi_ccl_fusion_plan** plan) {
-    if (!plan)
-        return MI_CCL_INVALID_ARGUMENTS;
-    *plan = nullptr;
-    const size_t esz = fusion_dtype_size(dtype);
-    if (esz == 0 || k == 0 || !counts || align == 0 || (align & (align - 1)) != 0)
-        return MI_CCL_INVALID_ARGUMENTS;
-    mi_ccl_fusion_plan* p = new (std::nothrow) mi_ccl_fusion_plan;
-    if (!p)
-        return MI_CCL_OUT_OF_RESOURCE;
+// The host tables of a plan are std::vectors, so building one may throw; the entry point below turns that into a status.
+static int plan_build(mi_ccl_fusion_plan* p, const size_t* counts, size_t k, int dtype, size_t esz, size_t align) {
     p->k = k;
     p->dtype = dtype;
     p->esz = esz;
@@ -244,10 +242,8 @@ int mi_ccl_fusion_plan_create(const size_t* counts, size_t k, int dtype, size_t 
         p->item_begin[t] = items.size();
         const uint64_t bytes = (uint64_t)counts[t] * esz;
         const uint64_t chunks = (bytes + kFusionChunk - 1) / kFusionChunk;
-        if (chunks > 0xffffffffull || t > 0xffffffffull || items.size() + chunks > 0x7fffffffull) {
-            delete p;
+        if (chunks > 0xffffffffull || t > 0xffffffffull || items.size() + chunks > 0x7fffffffull)
             return MI_CCL_INVALID_ARGUMENTS;
-        }
         for (uint64_t c = 0; c < chunks; c++) items.push_back(FusionItem{ (uint32_t)t, (uint32_t)c });
     }
     p->item_begin[k] = items.size();
@@ -259,21 +255,44 @@ int mi_ccl_fusion_plan_create(const size_t* counts, size_t k, int dtype, size_t 
     const size_t table_bytes = 2 * k * sizeof(uint64_t) + (items.size() ? items.size() : 1) * sizeof(FusionItem);
     hipError_t e = hipMalloc(&p->d_table, table_bytes);
     if (e != hipSuccess) {
-        delete p;
+        p->d_table = nullptr;
         return fusion_status_of(e);
     }
     e = hipMemcpy(p->d_table, host.data(), 2 * k * sizeof(uint64_t), hipMemcpyHostToDevice);
     if (e == hipSuccess && !items.empty())
         e = hipMemcpy((char*)p->d_table + 2 * k * sizeof(uint64_t), items.data(), items.size() * sizeof(FusionItem),
                       hipMemcpyHostToDevice);
-    if (e != hipSuccess) {
-        (void)hipFree(p->d_table);
-        delete p;
+    if (e != hipSuccess)
         return fusion_status_of(e);
-    }
     p->d_off = (const uint64_t*)p->d_table;
     p->d_bytes = p->d_off + k;
     p->d_items = (const FusionItem*)(p->d_bytes + k);
+    return MI_CCL_SUCCESS;
+}
+
+int mi_ccl_fusion_plan_create(const size_t* counts, size_t k, int dtype, size_t align, mi_ccl_fusion_plan** plan) {
+    if (!plan)
+        return MI_CCL_INVALID_ARGUMENTS;
+    *plan = nullptr;
+    const size_t esz = fusion_dtype_size(dtype);
+    if (esz == 0 || k == 0 || !counts || align == 0 || (align & (align - 1)) != 0)
+        return MI_CCL_INVALID_ARGUMENTS;
+    mi_ccl_fusion_plan* p = new (std::nothrow) mi_ccl_fusion_plan;
+    if (!p)
+        return MI_CCL_OUT_OF_RESOURCE;
+    int rc;
+    try {
+        rc = plan_build(p, counts, k, dtype, esz, align);
+    }
+    catch (const std::exception&) {     // bad_alloc, length_error: out of host memory for the tables
+        rc = MI_CCL_OUT_OF_RESOURCE;
+    }
+    if (rc != MI_CCL_SUCCESS) {
+        if (p->d_table)
+            (void)hipFree(p->d_table);
+        delete p;
+        return rc;
+    }
     *plan = p;
     return MI_CCL_SUCCESS;
 }

@@ -4,13 +4,16 @@
 // Prints one line per size: GPU-clock time per call of 2000 back-to-back calls, host time to enqueue one call, and
 // the round trip of one call followed by a stream synchronisation.  Then the case fusion exists for: 1,024 small bf16
 // gradient tensors reduced against 7 peers, one call per tensor against the fusion manager (requests queued one by
-// one, fused up to 256 per launch: pack, one 8-input reduce over the fusion buffer, unpack).
+// one, fused up to 256 per launch: pack, one 8-input reduce over the fusion buffer, unpack).  Also: the same small
+// reduces as nodes of a HIP graph (64 per graph, time per node of a replay), and what the C++ layer's check of its
+// buffer arguments costs per call (ccl::env_data::check_pointers 0 / 1 / 2).
 #include <hip/hip_runtime.h>
 #include <stdio.h>
 #include <chrono>
 #include <memory>
 #include <vector>
 #include "../../include/mi_ccl_comp.h"
+#include "../../oneccl_amd/csrc/ccl_comp.hpp"
 #include "../../oneccl_amd/csrc/ccl_fusion.hpp"
 #define CK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("HIP error %s line %d\n", hipGetErrorString(e), __LINE__); return 1; } } while (0)
 int main() {
@@ -40,6 +43,64 @@ int main() {
                std::chrono::duration<double, std::micro>(t2 - t0).count() / iters,
                std::chrono::duration<double, std::micro>(t4 - t3).count() / 200);
         for (int i = 0; i < 5; i++) CK(hipFree(b[i]));
+    }
+    // The same small reduces captured into a HIP graph: 64 nodes (rotating over 4 output buffers), replayed 50 times.
+    for (size_t bytes : {1024ul, 16384ul, 65536ul, 262144ul, 1048576ul, 4194304ul}) {
+        void* b[8];
+        for (int i = 0; i < 8; i++) { CK(hipMalloc(&b[i], bytes)); CK(hipMemset(b[i], i < 4 ? i + 1 : 0, bytes)); }
+        const void* srcs[4] = { b[0], b[1], b[2], b[3] };
+        mi_ccl_comp_reduce_n(MI_CCL_INT32, MI_CCL_SUM, srcs, 4, b[4], bytes / 4, 0, 2, 0, s);   // warm, outside the capture
+        CK(hipStreamSynchronize(s));
+        const int nodes = 64, replays = 50;
+        hipGraph_t g; hipGraphExec_t ge;
+        CK(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+        for (int i = 0; i < nodes; i++) mi_ccl_comp_reduce_n(MI_CCL_INT32, MI_CCL_SUM, srcs, 4, b[4 + (i & 3)], bytes / 4, 0, 2, 0, s);
+        CK(hipStreamEndCapture(s, &g));
+        CK(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0));
+        CK(hipGraphLaunch(ge, s)); CK(hipStreamSynchronize(s));
+        std::vector<uint32_t> h(bytes / 4);
+        CK(hipMemcpy(h.data(), b[7], bytes, hipMemcpyDeviceToHost));
+        for (uint32_t v : h) if (v != 0x0a0a0a0au) { printf("WRONG RESULT (graph replay, %zu B)\n", bytes); return 1; }
+        hipEvent_t e0, e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
+        CK(hipEventRecord(e0, s));
+        for (int r = 0; r < replays; r++) CK(hipGraphLaunch(ge, s));
+        CK(hipEventRecord(e1, s));
+        CK(hipStreamSynchronize(s));
+        float ms; CK(hipEventElapsedTime(&ms, e0, e1));
+        auto t0 = std::chrono::steady_clock::now();
+        for (int r = 0; r < 20; r++) { CK(hipGraphLaunch(ge, s)); CK(hipStreamSynchronize(s)); }
+        auto t1 = std::chrono::steady_clock::now();
+        printf("%8zu B x4 as graph nodes: %.2f us per node (64 nodes per graph, 50 replays back to back); one replay + sync %.1f us\n", bytes,
+               ms * 1e3 / replays / nodes, std::chrono::duration<double, std::micro>(t1 - t0).count() / 20);
+        CK(hipGraphExecDestroy(ge)); CK(hipGraphDestroy(g));
+        for (int i = 0; i < 8; i++) CK(hipFree(b[i]));
+    }
+    // What the C++ layer's look at its buffer arguments costs: host time to enqueue one 1 KiB ccl_comp_reduce with
+    // the check off (0), remembered per allocation (1, the default) and asked of the runtime every time (2); the
+    // smallest of five runs of 20,000 calls each.
+    {
+        void *a, *b;
+        CK(hipMalloc(&a, 1024)); CK(hipMalloc(&b, 1024)); CK(hipMemset(a, 0, 1024)); CK(hipMemset(b, 0, 1024));
+        ccl_sched sched; sched.stream = s;
+        const ccl_datatype& i32 = ccl_datatype_storage::instance().get(ccl::datatype::int32);
+        double best[3] = { 1e9, 1e9, 1e9 };
+        for (int run = 0; run < 5; run++)
+            for (int mode = 0; mode < 3; mode++) {
+                ccl::global_data::env().check_pointers = mode;
+                for (int i = 0; i < 200; i++) ccl_comp_reduce(&sched, a, 256, b, nullptr, i32, ccl::reduction::sum, nullptr);
+                CK(hipStreamSynchronize(s));
+                const int iters = 20000;
+                auto t0 = std::chrono::steady_clock::now();
+                for (int i = 0; i < iters; i++) ccl_comp_reduce(&sched, a, 256, b, nullptr, i32, ccl::reduction::sum, nullptr);
+                auto t1 = std::chrono::steady_clock::now();
+                CK(hipStreamSynchronize(s));
+                const double us = std::chrono::duration<double, std::micro>(t1 - t0).count() / iters;
+                if (us < best[mode]) best[mode] = us;
+            }
+        ccl::global_data::env().check_pointers = 1;
+        printf("ccl_comp_reduce, 1 KiB, host enqueue per call: pointer check off %.3f us, remembered (default) %.3f us (+%.3f), runtime query every call %.3f us (+%.3f)\n",
+               best[0], best[1], best[1] - best[0], best[2], best[2] - best[0]);
+        CK(hipFree(a)); CK(hipFree(b));
     }
     // Many small reduces: 64 independent 4-input int32 sums as 64 calls and as ONE call of mi_ccl_comp_reduce_batch
     // (one launch).  Input k of every job holds the byte k + 1, so every output word must be 0x0a0a0a0a.

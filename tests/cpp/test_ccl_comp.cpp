@@ -17,6 +17,7 @@
 #include "../../oneccl_amd/csrc/ccl_comp.hpp"
 #include "../../oneccl_amd/csrc/ccl_fusion.hpp"
 #include "../../oneccl_amd/csrc/ccl_pipeline.hpp"
+#include "../../include/mi_ccl_comp.h"
 #include "../../oracle/ccl_comp_oracle.h"
 
 #define CK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { printf("HIP error %s at line %d\n", hipGetErrorString(e_), __LINE__); exit(2); } } while (0)
@@ -526,6 +527,86 @@ int main() {
         bool threw = false;
         try { ccl_chunked_reducer bad(1000, 4); } catch (const ccl::exception&) { threw = true; }
         EXPECT(threw, "a chunk size that is not a multiple of 16 bytes must throw");
+    }
+    // Pageable host memory is refused before anything is enqueued: the reference classifies its pointers and reduces
+    // host buffers on the host (comp.cpp:147-161); here a kernel on such a pointer would be a GPU memory fault.  Every
+    // call below must throw and must not launch: the thread's last kernel stays the copy that went before.
+    {
+        const size_t count = 4096;
+        std::vector<float> h_a(count, 1.0f), h_b(count, 2.0f);
+        DevBuf<float> d_a(std::vector<float>(count, 3.0f)), d_b(std::vector<float>(count, 4.0f)), d_c(count);
+        const ccl_datatype& f32 = DT(ccl::datatype::float32);
+        const ccl_datatype& b16 = DT(ccl::datatype::bfloat16);
+        for (int mode : { 1, 2 }) {
+            ccl::global_data::env().check_pointers = mode;
+            ccl_comp_copy(d_a.p, d_c.p, count * 4, true, &sched);
+            EXPECT(std::string(mi_ccl_last_kernel()) == "copy_kernel", "marker launch");
+            int refused = 0, tried = 0;
+            auto must_refuse = [&](const char* what, auto&& call) {
+                tried++;
+                try { call(); printf("FAIL: %s did not throw\n", what); }
+                catch (const ccl::exception& e) {
+                    if (strstr(e.what(), "not memory the GPU can reach")) refused++;
+                    else printf("FAIL: %s threw something else: %s\n", what, e.what());
+                }
+            };
+            const std::vector<size_t> offs = { 0, count / 2 };
+            must_refuse("reduce, host in", [&] { ccl_comp_reduce(&sched, h_a.data(), count, d_b.p, nullptr, f32, ccl::reduction::sum, nullptr); });
+            must_refuse("reduce, host inout", [&] { ccl_comp_reduce(&sched, d_a.p, count, h_b.data(), nullptr, f32, ccl::reduction::sum, nullptr); });
+            must_refuse("reduce, both host", [&] { ccl_comp_reduce(&sched, h_a.data(), count, h_b.data(), nullptr, f32, ccl::reduction::max, nullptr); });
+            must_refuse("batch reduce, host buffer", [&] { ccl_comp_batch_reduce(h_a.data(), offs, count / 2, h_a.data(), nullptr, f32, ccl::reduction::sum, nullptr, nullptr, 0, nullptr, nullptr, &sched); });
+            must_refuse("batch reduce, host slices", [&] { ccl_comp_batch_reduce(h_a.data(), offs, count / 2, d_b.p, nullptr, f32, ccl::reduction::sum, nullptr, nullptr, 0, nullptr, nullptr, &sched); });
+            must_refuse("copy, host in", [&] { ccl_comp_copy(h_a.data(), d_b.p, count * 4, false, &sched); });
+            must_refuse("copy, host out", [&] { ccl_comp_copy(d_a.p, h_b.data(), count * 4, true, &sched); });
+            must_refuse("reduce_n, host peer", [&] { ccl_comp_reduce_n(&sched, d_a.p, { d_b.p, h_a.data() }, count, d_c.p, f32, ccl::reduction::sum); });
+            must_refuse("reduce_n, host out", [&] { ccl_comp_reduce_n(&sched, d_a.p, { d_b.p }, count, h_b.data(), f32, ccl::reduction::sum); });
+            must_refuse("reduce_write_n, host out", [&] { ccl_comp_reduce_write_n(&sched, d_a.p, { d_b.p }, count, { d_c.p, h_b.data() }, f32, ccl::reduction::sum); });
+            must_refuse("reduce_batch, host input", [&] { ccl_comp_reduce_batch(&sched, { d_a.p, d_b.p, d_a.p, h_a.data() }, 2, { d_c.p, d_c.p }, { 16, 16 }, f32, ccl::reduction::sum); });
+            must_refuse("bf16 reduce, host in", [&] { ccl_bf16_reduce(h_a.data(), count, d_b.p, nullptr, ccl::reduction::sum, &sched); });
+            must_refuse("fp16 reduce, host inout", [&] { ccl_fp16_reduce(d_a.p, count, h_b.data(), nullptr, ccl::reduction::sum, &sched); });
+            must_refuse("fp32 -> bf16, host source", [&] { ccl_convert_fp32_to_bf16_arrays(h_a.data(), d_b.p, count, &sched); });
+            must_refuse("bf16 -> fp32, host destination", [&] { ccl_convert_bf16_to_fp32_arrays(d_a.p, h_b.data(), count, &sched); });
+            (void)b16;
+            EXPECT(refused == tried, "mode %d: %d of %d calls on pageable host memory were refused", mode, refused, tried);
+            EXPECT(std::string(mi_ccl_last_kernel()) == "copy_kernel", "mode %d: a refused call launched %s", mode, mi_ccl_last_kernel());
+            CK(hipStreamSynchronize(stream));
+            bool untouched = true;
+            for (size_t i = 0; i < count; i++) untouched = untouched && h_a[i] == 1.0f && h_b[i] == 2.0f;
+            std::vector<float> ga = d_a.host(), gb = d_b.host();
+            for (size_t i = 0; i < count; i++) untouched = untouched && ga[i] == 3.0f && gb[i] == 4.0f;
+            EXPECT(untouched, "mode %d: refused calls left every buffer as it was", mode);
+            // a device buffer that is too short for the count is refused too (its allocation's extent is known)
+            bool threw = false;
+            try { ccl_comp_reduce(&sched, d_a.p, count * 1024, d_b.p, nullptr, f32, ccl::reduction::sum, nullptr); }
+            catch (const ccl::exception& e) { threw = strstr(e.what(), "runs past the end") != nullptr; }
+            EXPECT(threw, "mode %d: a count beyond the allocation must throw", mode);
+            EXPECT(std::string(mi_ccl_last_kernel()) == "copy_kernel", "mode %d: the oversized call launched %s", mode, mi_ccl_last_kernel());
+            // pinned host memory is memory the GPU can reach: accepted, and the result is right
+            float* pinned = nullptr;
+            CK(hipHostMalloc((void**)&pinned, count * 4, hipHostMallocDefault));
+            for (size_t i = 0; i < count; i++) pinned[i] = (float)i;
+            ccl_comp_reduce(&sched, pinned, count, d_b.p, nullptr, f32, ccl::reduction::sum, nullptr);
+            gb = d_b.host();
+            bool ok = true;
+            for (size_t i = 0; i < count; i++) ok = ok && gb[i] == 4.0f + (float)i;
+            EXPECT(ok, "mode %d: pinned host input", mode);
+            CK(hipMemcpy(d_b.p, std::vector<float>(count, 4.0f).data(), count * 4, hipMemcpyHostToDevice));
+            CK(hipHostFree(pinned));
+            ccl_comp_forget_pointers();
+        }
+        // custom reduction on two host buffers: the callback runs on them as they are (comp.cpp:84-88)
+        std::vector<int32_t> ha(100), hb(100);
+        for (int i = 0; i < 100; i++) { ha[i] = i; hb[i] = 5; }
+        size_t oc = 0;
+        ccl_comp_reduce(&sched, ha.data(), 100, hb.data(), &oc, DT(ccl::datatype::int32), ccl::reduction::custom, custom_sum_i32);
+        bool ok = oc == 100;
+        for (int i = 0; i < 100; i++) ok = ok && hb[i] == 10 + i;
+        EXPECT(ok, "custom reduction on host buffers");
+        // the check switched off: a good call still works (nothing is ever launched on a bad pointer here)
+        ccl::global_data::env().check_pointers = 0;
+        ccl_comp_reduce(&sched, d_a.p, count, d_b.p, nullptr, f32, ccl::reduction::sum, nullptr);
+        EXPECT(d_b.host()[17] == 7.0f, "check_pointers = 0");
+        ccl::global_data::env().check_pointers = 1;
     }
     CK(hipStreamDestroy(stream));
     printf("%d checks, %d failed\n", g_checks, g_fail);

@@ -1,7 +1,7 @@
 """mi_ccl_fusion_reduce_static, the fused reduce that allocates nothing (its work table lives in an array inside the
 library): called through the C ABI, its output must equal, bit for bit, that of mi_ccl_fusion_reduce on a plan of
-the same layout -- on two calls in a row, the second with a smaller input, so that what the first call left in the
-shared table cannot leak into the second.  Also: the limits are refused with out_of_resource, and once the first
+the same layout -- on two calls in a row, the second with a smaller input, and on a run of calls long enough that a
+table which held a larger layout is used again, so that what an earlier call left in a table cannot leak into a later one.  Also: the limits are refused with out_of_resource, and once the first
 call on the device has looked the table's address up, a call makes no device allocation (the free-memory figure of
 the device does not move)."""
 import numpy as np
@@ -77,6 +77,43 @@ def test_static_entry_point_equals_plan_entry_point_twice_in_a_row(comp, variant
     small = [1, 4097, 0, 8192, 33, 70_001]
     _case(comp, rng, small, O.FLOAT32, O.MAX, 2, 1, comp.LP_PAIRWISE, variant)
     _case(comp, rng, [5], O.INT8, O.PROD, 0, 1, comp.LP_PAIRWISE, variant)
+
+
+def test_static_entry_point_reuses_a_table_that_held_a_larger_layout(comp):
+    """The library keeps four tables per GPU and hands them out in turn, so the fifth call gets the table of the first:
+    a large layout first, then smaller ones until every table has come round again."""
+    rng = np.random.default_rng(77)
+    big = [int(c) for c in np.exp(rng.uniform(np.log(3), np.log(200_000), 200))]
+    _case(comp, rng, big, O.BFLOAT16, O.SUM, 3, 1, comp.LP_KEEP_PRECISION, 0)
+    for r in range(5):
+        _case(comp, rng, [17 + r, 4099, 2], O.INT16, O.MIN, 2, 2, comp.LP_PAIRWISE, 0)
+
+
+def test_static_entry_point_calls_that_overlap_on_two_streams(comp):
+    """Two calls with different layouts issued back to back on two streams (they may run side by side): each has a
+    table of its own, so each must equal the plan entry point's result on the same inputs."""
+    import torch
+    rng = np.random.default_rng(78)
+    cases = []
+    for counts, dtype, n_peers in (([300_001, 5, 1_000_003], O.FLOAT32, 3), ([777, 2_000_001], O.INT32, 2)):
+        np_t, esz = O.NP_STORAGE[dtype], O.DTYPE_SIZE[dtype]
+        _, total = O.fusion_offsets(counts, esz, 4)
+        tens = [to_dev(make_inputs(rng, dtype, c, O.SUM, 1)[0]) for c in counts]
+        peers = [to_dev(make_inputs(rng, dtype, total // esz + 8, O.SUM, 1)[0]) for _ in range(n_peers)]
+        plan = comp.FusionPlan(counts, dtype, 4)
+        want = [torch.zeros_like(t) for t in tens]
+        plan.reduce(comp.SUM, tens, peers, want)
+        plan.close()
+        cases.append((counts, dtype, tens, peers, want, [torch.zeros_like(t) for t in tens]))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for rep in range(3):
+        for (counts, dtype, tens, peers, want, got), st in zip(cases, streams):
+            comp.fusion_reduce_static(counts, dtype, 4, comp.SUM, tens, peers, got, stream=st)
+    torch.cuda.synchronize()
+    for counts, dtype, tens, peers, want, got in cases:
+        for g, w in zip(got, want):
+            assert torch.equal(g, w)
 
 
 def test_static_entry_point_limits_and_errors(comp):
