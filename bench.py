@@ -241,6 +241,132 @@ def cpu_baseline(torch, comp, w, bufs, sample_elems):
                 **({"reference_pairwise": ref_leg} if ref_leg else {})), out, s
 
 
+# The other benchmark configurations, timed after the headline's timed region of a default run (they do not enter
+# `value`, `ms_per_step` or `roofline`): name -> what is run.
+OTHER_WORKLOADS = ("c1_fp32", "c2_bf16", "c5_fp32", "c4_fused", "c4_three_step")
+OTHER_KEYS = ("ms", "GBps", "frac", "kernel", "traffic", "algorithmic_bytes", "steps", "checked")
+
+
+def other_entry(name, ms, algo_bytes, kernel, steps, checked):
+    """One entry of the JSON line's "other_workloads" object: time per call, algorithmic GB/s, fraction of the HBM
+    peak, the kernel that ran, its measured HBM traffic where profiles/measured_traffic.json holds it for that
+    kernel, and what the result was compared with before it was timed."""
+    gbs = algo_bytes / (ms * 1e-3) / 1e9
+    return {"ms": round(ms, 4), "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4), "kernel": kernel,
+            "traffic": measured_traffic(name, kernel.split(" + ")[0]), "algorithmic_bytes": int(algo_bytes),
+            "steps": int(steps), "checked": checked}
+
+
+def other_workloads(torch, comp, stream, steps, warmup):
+    """C1, C2, the fp32 form of C5 and C4 (fused and as pack + reduce + unpack) on the same GPU: each is compared bit
+    for bit with the CPU oracle on its first buffer set (whole buffers up to 64 MiB, beyond that the first 16 MiB and
+    the last 1 MiB of every buffer; C4 tensor by tensor), then timed with HIP events over `steps` back-to-back calls
+    that rotate over the workload's buffer sets."""
+    import math
+    import numpy as np
+    import oracle_lib as O
+    res = {}
+
+    def timed(fn, k, w):
+        for i in range(w):
+            fn(i)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(k):
+            fn(i)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / k
+
+    def bits(t, lo, hi):
+        v = t[lo:hi]
+        return (v.view(torch.int16).cpu().numpy().view(np.uint16) if v.element_size() == 2
+                else v.view(torch.int32).cpu().numpy().view(np.uint32))
+
+    def check_reduce(name, odt, srcs, run_once, count, keep):
+        esz = O.DTYPE_SIZE[odt]
+        spans = [(0, count)] if count * esz <= (64 << 20) else [(0, (16 << 20) // esz), (count - (1 << 20) // esz, count)]
+        want = [(lo, hi, O.reduce_n([bits(s_, lo, hi).view(O.NP_STORAGE[odt]) for s_ in srcs], odt, O.SUM, keep=keep, threads=16))
+                for lo, hi in spans]                  # inputs are read before the call: the output may be one of them
+        out = run_once()
+        torch.cuda.synchronize()
+        for lo, hi, w_ in want:
+            if not (bits(out, lo, hi) == w_.view(bits(out, lo, lo).dtype)).all():
+                sys.exit(f"{name}: GPU result differs from the oracle in elements [{lo}, {hi})")
+        return "bit-exact vs oracle: " + ("every element" if len(spans) == 1 else "first 16 MiB and last 1 MiB of the buffers")
+
+    for name in ("c1_fp32", "c2_bf16", "c5_fp32"):
+        w = WORKLOADS[name]
+        dt, odt = (comp.BFLOAT16, O.BFLOAT16) if w["dtype"] == "bfloat16" else (comp.FLOAT32, O.FLOAT32)
+        lp = comp.LP_KEEP_PRECISION if w["keep"] else comp.LP_PAIRWISE
+        n, count = w["n"], w["count"]
+        sets = [make_buffers(torch, w, 4321 + i) for i in range(w["sets"])]
+        outs = [s_[0] if w.get("in_place") else torch.empty_like(s_[0]) for s_ in sets]
+
+        def call(i, sets=sets, outs=outs, dt=dt, lp=lp, count=count):
+            comp.comp_reduce_n(dt, comp.SUM, sets[i % len(sets)], outs[i % len(sets)], count, lp_mode=lp, stream=stream)
+
+        def once(call=call, outs=outs):
+            call(0)
+            return outs[0]
+        checked = check_reduce(name, odt, sets[0], once, count, 1 if w["keep"] else 0)
+        k = steps if count > 100_000_000 else max(steps, 64)
+        ms = timed(call, k, max(warmup, 5))
+        res[name] = other_entry(name, ms, (n + 1) * count * (2 if dt == comp.BFLOAT16 else 4), comp.last_kernel(), k, checked)
+        del sets, outs
+        torch.cuda.empty_cache()
+
+    # C4: 256 bf16 tensors, counts log-uniform over [2,048, 2,097,152], 256-byte aligned offsets, 7 peer fusion buffers
+    rng = np.random.default_rng(4)
+    counts = [int(round(math.exp(rng.uniform(math.log(2048), math.log(2_097_152))))) for _ in range(256)]
+    payload = sum(counts) * 2
+    plan = comp.FusionPlan(counts, comp.BFLOAT16, 256)
+    nelem = plan.nbytes // 2
+    g = torch.Generator(device="cuda")
+    g.manual_seed(44)
+    tens = [torch.empty(c, dtype=torch.bfloat16, device="cuda").normal_(0, 0.02, generator=g) for c in counts]
+    outs = [torch.zeros_like(t) for t in tens]
+    fb = torch.zeros(nelem, dtype=torch.bfloat16, device="cuda")
+    peers = [torch.empty(nelem, dtype=torch.bfloat16, device="cuda").normal_(0, 0.02, generator=g) for _ in range(7)]
+    offs, _ = O.fusion_offsets(counts, 2, 256)
+    host_peers = [bits(p_, 0, nelem) for p_ in peers]
+    want = [O.reduce_n([bits(t, 0, c)] + [hp[int(o) // 2:int(o) // 2 + c] for hp in host_peers], O.BFLOAT16, O.SUM, keep=1, threads=16)
+            for t, c, o in zip(tens, counts, offs)]
+
+    def check_c4(what):
+        torch.cuda.synchronize()
+        for i, c in enumerate(counts):
+            if not (bits(outs[i], 0, c) == want[i]).all():
+                sys.exit(f"{what}: tensor {i} of {c} elements differs from the oracle")
+            outs[i].zero_()
+
+    def fused(i):
+        plan.reduce(comp.SUM, tens, peers, outs, lp_mode=comp.LP_KEEP_PRECISION, stream=stream)
+
+    def three(i):
+        plan.pack(tens, fb, stream=stream)
+        comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, [fb] + peers, fb, nelem, lp_mode=comp.LP_KEEP_PRECISION, stream=stream)
+        plan.unpack(fb, outs, stream=stream)
+    fused(0)
+    k_fused = comp.last_kernel()
+    check_c4("c4_fused")
+    k = max(steps, 50)
+    ms = timed(fused, k, max(warmup, 5))
+    res["c4_fused"] = other_entry("c4_fused", ms, 9 * payload, k_fused, k, "bit-exact vs oracle: every tensor")
+    three(0)
+    check_c4("c4_three_step")
+    kernels = []
+    plan.pack(tens, fb, stream=stream)
+    kernels.append(comp.last_kernel())
+    comp.comp_reduce_n(comp.BFLOAT16, comp.SUM, [fb] + peers, fb, nelem, lp_mode=comp.LP_KEEP_PRECISION, stream=stream)
+    kernels.append(comp.last_kernel())
+    ms = timed(three, k, max(warmup, 5))
+    res["c4_three_step"] = other_entry("c4_three_step", ms, 13 * payload, " + ".join(kernels + [kernels[0]]), k,
+                                       "bit-exact vs oracle: every tensor")
+    plan.close()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -249,6 +375,8 @@ def main():
     ap.add_argument("--workload", default="c5_bf16", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-sample", type=int, default=1 << 28, help="elements per buffer for the CPU baseline")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the other benchmark configurations that a default run times after the headline")
     ap.add_argument("--set", action="append", default=[], metavar="NAME=VALUE", help="launch knob (mi_ccl_set_param)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -374,6 +502,10 @@ def main():
                      "single_launch_ms_median": round(launch_ms_median, 4), "single_launch_ms_min": round(singles[0], 4)},
         "cpu_baseline": base,
     }
+    if args.workload == "c5_bf16" and not args.no_other_workloads and not args.set:
+        del sets, outs, extra_outs      # the headline's 18 GB go back before the other configurations allocate theirs
+        torch.cuda.empty_cache()
+        out["other_workloads"] = other_workloads(torch, comp, stream, args.steps, args.warmup)
     print(json.dumps(out))
 
 

@@ -17,6 +17,12 @@
 
 #include "launch_geometry.hpp"
 
+// The inline assembly below (sub-dword byte lanes, MODE-register writes, "sc1 nt" stores with hand-placed wait states)
+// is written against the gfx950 instruction set and its hazard rules; no other target is built or tested.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "these kernels are written for gfx950 (MI355X) only"
+#endif
+
 namespace mi {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -509,9 +515,14 @@ __device__ __forceinline__ u32x4 ld_loose(const u32x4_u* p) { return __builtin_n
 __device__ __forceinline__ void st_loose(u32x4_u* p, u32x4 v) { __builtin_nontemporal_store(v, p); }
 // The same store with device scope on top (sc1 nt).  A 1 : 1 copy gains 2-6 % from it (6.65 against 6.50 TB/s at
 // 512 MiB, 6.19 against 5.85 at 64 MiB); the reduce kernels, the converters, pack / unpack and the broadcast measure
-// 0-8 % slower with it, so only the copy uses it.  The compiler does not know that this is a store: the two wait states
-// behind it are the ones it would insert itself between a vector-memory store of more than 64 bits and the next write
-// of the registers that hold the store's data (without them a lane's data is overwritten before the store has read it).
+// 0-8 % slower with it, so only the copy uses it.  The compiler does not know that this is a store, so what it would
+// do for one is done by hand: (1) gfx9 reads the data registers of a vector-memory store of more than 64 bits up to two
+// cycles after issue, and a VALU or VMEM write to them in that window is a hazard the compiler's hazard pass covers with
+// wait states -- hence the "s_nop 1" (two wait states) inside the same asm statement, which nothing can be scheduled
+// into (without it 3 % of a 2-input reduce's elements came back as the NEXT iteration's data); (2) "memory" keeps
+// loads and stores from moving across it; (3) the asm is counted by no s_waitcnt the compiler emits, which is harmless
+// for a store whose completion nobody waits for (the kernel's end drains it).  Bit-exact copy tests with odd heads and
+// tails, across several launches, cover it (tests/test_gpu_parity.py, tests/test_gpu_large_launches.py).
 __device__ __forceinline__ void st_loose_device_scope(u32x4_u* p, u32x4 v) {
     asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
 }

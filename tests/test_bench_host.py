@@ -26,3 +26,18 @@ def test_measured_traffic_is_tied_to_the_kernel():
         assert os.path.exists(os.path.join(ROOT, e["summary"]))
     assert bench.measured_traffic("c1_fp32", "reduce_vec_kernel") is None or "c1_fp32" in table["workloads"]
     assert bench.measured_traffic("no_such_workload", "copy_kernel") is None
+
+
+def test_other_workloads_schema():
+    """The five entries a default run adds under "other_workloads", and the keys of an entry."""
+    import bench
+    assert bench.OTHER_WORKLOADS == ("c1_fp32", "c2_bf16", "c5_fp32", "c4_fused", "c4_three_step")
+    e = bench.other_entry("c1_fp32", 0.0323, 201_326_592, "reduce_vec_kernel", 64, "bit-exact vs oracle: every element")
+    assert tuple(e) == bench.OTHER_KEYS
+    assert e["GBps"] == round(201_326_592 / 0.0323e-3 / 1e9, 1) and abs(e["frac"] - e["GBps"] / 8000.0) < 1e-4
+    assert e["traffic"] == bench.measured_traffic("c1_fp32", "reduce_vec_kernel")
+    assert bench.other_entry("c1_fp32", 1.0, 1, "another_kernel", 1, "")["traffic"] is None
+    assert bench.other_entry("c4_three_step", 1.0, 1, "fusion_copy_kernel + reduce_multi_kernel + fusion_copy_kernel", 1, "")["traffic"] is None
+    src = open(bench.__file__).read()
+    for name in bench.OTHER_WORKLOADS:
+        assert f'"{name}"' in src

@@ -3,7 +3,8 @@
 (reduce with zeros is the identity on finite values, x + (-x) = +0, in-place equals out-of-place); the 2-input in-place
 fp32 sum at 16,777,216 elements, the 8-input bf16 sum at 33,554,432, and the fusion configuration at its full counts
 (256 bf16 tensors, log-uniform over [2,048, 2,097,152], 256-byte aligned offsets, seven peer fusion buffers) through
-pack + reduce + unpack and through the fused single pass."""
+pack + reduce + unpack and through the fused single pass; and the datatype x op sweep's six (type, operation) pairs with
+four inputs at 16 MiB, 64 MiB and 1 GiB per buffer, by the automatic kernel choice, every element."""
 import numpy as np
 import pytest
 
@@ -208,3 +209,44 @@ def test_c4_fusion_256_tensors_full_counts(comp):
         assert (outs[i].cpu().numpy().view(np.uint16) == want[i]).all(), f"fused, static table: tensor {i}"
     plan.close()
 
+
+
+C3_CASES = [("int8", "SUM"), ("int32", "SUM"), ("int64", "MAX"), ("float16", "SUM"), ("float32", "MIN"), ("float64", "PROD")]
+
+
+@pytest.mark.parametrize("tname,opname", C3_CASES)
+def test_c3_four_inputs_16MiB_64MiB_1GiB_automatic_kernel_every_element(comp, tname, opname):
+    """The sweep's (type, operation) pairs at its three largest sizes, kernel form chosen by the library (variant 0):
+    the streaming kernel at 16 MiB per buffer, the phased kernel at 64 MiB and 1 GiB.  Integers uniform over the full
+    range of the type, floats uniform[-2, 2] (product: uniform[0.9, 1.1]), float16 by a round-to-nearest-even cast;
+    every element against the 16-thread oracle."""
+    import torch
+    tdt = getattr(torch, tname)
+    dt = {"int8": O.INT8, "int32": O.INT32, "int64": O.INT64, "float16": O.FLOAT16, "float32": O.FLOAT32, "float64": O.FLOAT64}[tname]
+    op = getattr(O, opname)
+    esz = O.DTYPE_SIZE[dt]
+    np_t = O.NP_STORAGE[dt]
+    view = {1: torch.int8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[esz]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(3000 + dt)
+    assert comp.get_param("variant") == 0
+    for size, kernel in ((16 << 20, "reduce_vec_kernel"), (64 << 20, "reduce_multi_phased_kernel"), (1 << 30, "reduce_multi_phased_kernel")):
+        count = size // esz
+        if tdt.is_floating_point:
+            lo, hi = (0.9, 1.1) if op == O.PROD else (-2.0, 2.0)
+            srcs = [torch.empty(count, dtype=torch.float32 if esz <= 4 else torch.float64, device="cuda").uniform_(lo, hi, generator=g).to(tdt)
+                    for _ in range(4)]
+        else:
+            info = torch.iinfo(tdt)
+            srcs = [torch.randint(info.min, info.max, (count,), dtype=tdt, device="cuda", generator=g) for _ in range(4)]
+        out = torch.zeros(count, dtype=tdt, device="cuda")
+        comp.comp_reduce_n(dt, op, srcs, out, count)
+        torch.cuda.synchronize()
+        assert comp.last_kernel() == kernel, (size, comp.last_kernel())
+        host = [s_.view(view).cpu().numpy().view(np_t) for s_ in srcs]
+        want = O.reduce_n(host, dt, op, threads=16)
+        got = out.view(view).cpu().numpy()
+        u = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[esz]
+        bad = got.view(u) != want.view(u)
+        assert not bad.any(), f"{tname} {opname} at {size >> 20} MiB: {np.count_nonzero(bad)} elements differ, first at {np.flatnonzero(bad)[:5]}"
+        del host, want, got, srcs, out

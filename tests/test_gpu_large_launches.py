@@ -95,7 +95,9 @@ def test_copy_of_more_than_64_GiB(comp):
         assert torch.equal(dst[lo:hi], src[lo:hi]), f"copy differs in bytes [{lo}, {hi})"
     assert int(dst[:3].count_nonzero()) == 0 and int(dst[3 + n:].count_nonzero()) == 0
     del dst
-    # the converter at a count that needs two launches: 2^32 + 4,099 bf16 values widened (8 values per ... 4 per lane)
+    # the widening converter beyond 2^32 values (64-bit indexing): at four values per lane that is 2^22 tiles, still ONE
+    # launch -- a converter needs more than 2^34 values to reach HIP's limit of 2^24 - 1 blocks, so the cutting of
+    # converter launches is exercised with the artificial launch_block_limit above and by the CPU geometry test only
     cnt = (1 << 32) + 4099
     h = src.view(torch.int16)[:cnt]
     f = torch.empty(cnt, dtype=torch.int32, device="cuda")

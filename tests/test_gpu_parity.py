@@ -370,28 +370,30 @@ def test_all_pairs_of_16bit_values_sum_and_prod(comp, dtype, impl):
 @pytest.mark.parametrize("dtype", [O.INT16, O.UINT16])
 def test_all_pairs_of_16bit_integers_sum_and_prod(comp, dtype):
     """Every (in, inout) pair of 16-bit integer patterns -- 2^32 pairs -- through the GPU kernel: the wrapped sum and
-    product (65535 x 65535 overflows a signed int, so both sides multiply in unsigned).  Checked against the oracle
-    and against the closed form on 32-bit unsigned integers, which shares no code with either."""
+    product (65535 x 65535 overflows a signed int, so both sides multiply in unsigned).  Every pair is checked on the
+    GPU against the closed form in torch's wrapping 32-bit integer arithmetic, which shares no code with the kernels
+    or the oracle; a sample of rows (the extremes among them) also against the oracle."""
     import torch
     np_t = O.NP_STORAGE[dtype]
-    allv = np.arange(65536, dtype=np.uint16)
-    rows = 512
-    a = np.tile(allv, rows)
-    da = to_dev(a.view(np_t))
-    a32 = a.astype(np.uint32)
+    rows = 2048
+    allv = torch.arange(65536, dtype=torch.int32, device="cuda")
+    a32 = allv.repeat(rows)                                     # in: every value, `rows` times over
+    da = a32.to(torch.int16)                                    # keeps the low 16 bits
     for op in (O.SUM, O.PROD):
         for r0 in range(0, 65536, rows):
-            b = np.repeat(allv[r0:r0 + rows], 65536)
-            db = to_dev(b.view(np_t))
-            comp.comp_reduce(dtype, op, da, a.size, db)
+            b32 = allv[r0:r0 + rows].repeat_interleave(65536)   # inout: one value per row
+            db = b32.to(torch.int16)
+            comp.comp_reduce(dtype, op, da, da.numel(), db)
             torch.cuda.synchronize()
-            got = to_host(db, np_t).view(np.uint16)
-            b32 = b.astype(np.uint32)
-            closed = ((b32 + a32) if op == O.SUM else (b32 * a32)).astype(np.uint16)     # modulo 2^32, then modulo 2^16
-            assert (got == closed).all(), (dtype, op, r0, "closed form")
-            if r0 % (16 * rows) == 0 or r0 + rows == 65536:
-                want = O.reduce_n([b.view(np_t), a.view(np_t)], dtype, op, threads=16)
-                assert (got == want.view(np.uint16)).all(), (dtype, op, r0, "oracle")
+            closed = ((b32 + a32) if op == O.SUM else (b32 * a32)).to(torch.int16)      # modulo 2^32, then modulo 2^16
+            assert torch.equal(db, closed), (dtype, op, r0, "closed form")
+            if r0 in (0, 32768 - rows, 32768, 65536 - rows):
+                for r in (0, rows - 1):
+                    b = np.full(65536, r0 + r, np.uint16).view(np_t)
+                    a = np.arange(65536, dtype=np.uint16).view(np_t)
+                    want = O.reduce_n([b, a], dtype, op)
+                    got = db[r * 65536:(r + 1) * 65536].cpu().numpy().view(np.uint16)
+                    assert (got == want.view(np.uint16)).all(), (dtype, op, r0 + r, "oracle")
 
 
 def test_arguments_and_errors(comp):
