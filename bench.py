@@ -51,6 +51,13 @@ WORKLOADS = {
                            desc="one 2,007,564,288-byte buffer written, one 16-byte store per lane (the copy kernels' shape)"),
     "write_only_four": dict(dtype="bfloat16", n=0, m=1, count=1_003_782_144, keep=False, sets=1, probe="write_four",
                             desc="one 2,007,564,288-byte buffer written, four 16-byte stores per lane (the reduce kernels' shape)"),
+    # the same two probes at the footprint of C1 (2 x 64 MiB read, 64 MiB written, rotating over 8 buffer sets)
+    "read_only_c1": dict(dtype="float32", n=2, m=0, count=16_777_216, keep=False, sets=8, probe="read",
+                         desc="two 64 MiB buffers read, nothing written, rotating over 8 buffer sets (C1's reads alone)"),
+    "write_only_one_c1": dict(dtype="float32", n=0, m=1, count=16_777_216, keep=False, sets=8, probe="write_one",
+                              desc="one 64 MiB buffer written, one 16-byte store per lane, rotating over 8 buffer sets (C1's writes alone)"),
+    "write_only_four_c1": dict(dtype="float32", n=0, m=1, count=16_777_216, keep=False, sets=8, probe="write_four",
+                               desc="one 64 MiB buffer written, four 16-byte stores per lane, rotating over 8 buffer sets"),
     "memcpy_dtod": dict(dtype="bfloat16", n=1, count=1_003_782_144, keep=False, sets=1, probe="memcpy",
                         desc="hipMemcpyDtoDAsync of 2,007,564,288 bytes (the runtime's own device-to-device copy)"),
 }

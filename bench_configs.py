@@ -18,6 +18,7 @@
   copy   ccl_comp_copy at 64 MiB, 512 MiB and 3 GiB, and the bf16 <-> fp32 array converters at 2^28 elements
 
     python bench_configs.py [--out results/configs.json] [--skip c3,batch,types,align,write,copy] [--only c1,c4] [--c3-k 7]
+                            [--set realign=0]
 
 --only runs just the named sections (c1, c2, c3, batch, types, align, write, copy, c4, latency), --c3-k just the named sizes of
 the sweep (size = 1 KiB x 4^k): what a profiler run of one kernel wants.
@@ -60,6 +61,7 @@ def main():
     ap.add_argument("--skip", default="")
     ap.add_argument("--only", default="")
     ap.add_argument("--c3-k", default="", help="comma-separated exponents k of the C3 sizes 1 KiB x 4^k (default: all 11)")
+    ap.add_argument("--set", action="append", default=[], metavar="NAME=VALUE", help="launch knob (mi_ccl_set_param)")
     args = ap.parse_args()
     only = [x for x in args.only.split(",") if x]
     skip = [x for x in args.skip.split(",") if x]
@@ -73,6 +75,9 @@ def main():
     import oracle_lib as O          # the checker
     comp.lib()
     torch.cuda.set_device(0)
+    for kv in args.set:
+        k_, v_ = kv.split("=")
+        comp.set_param(k_, int(v_))
     res = {}
     rows = []
     checked = [0]

@@ -252,7 +252,11 @@ const char* mi_ccl_last_kernel(void);
  * costs speed only and is what the tests of that path use), "num_cus" (read
  * only), "fp16_impl" (what MI_CCL_FP16_DEFAULT stands for: 2, 3 or 4 of enum mi_ccl_fp16_impl above), and
  * "launch_block_limit" (blocks per launch of the copy, broadcast and converter kernels, which cut larger work into
- * several launches; 0 = what HIP allows, 2^24 - 1; smaller values let tests exercise the cutting).
+ * several launches; 0 = what HIP allows, 2^24 - 1; smaller values let tests exercise the cutting), "realign" (0/1,
+ * default 1: an input of a 16- or 8-bit type whose vectors start off a 4-byte boundary -- a peer's block behind an odd
+ * number of elements, a tensor behind an odd-sized one in a tight fusion buffer -- is read on that boundary and shifted
+ * into place in registers instead of with misaligned vector loads; same results, about a fifth faster for such
+ * layouts) and "realigned_launches" (read only: how many launches of the calling thread took that path).
  * Returns invalid_arguments for an unknown name or out-of-range value. */
 int mi_ccl_set_param(const char* name, long value);
 long mi_ccl_get_param(const char* name);

@@ -23,7 +23,8 @@ struct BatchTable {                     // by-value kernel argument (3.8 KB of t
     const void* p[kBatchMaxPtrs];       // job j: inputs p[j * (n + 1) + 0 .. n - 1], output p[j * (n + 1) + n]
     uint64_t count[kBatchMaxJobs];      // elements
     uint32_t tile_end[kBatchMaxJobs];   // tiles of jobs 0..j together
-    uint8_t head[kBatchMaxJobs];        // elements before job j's first vector
+    uint8_t head[kBatchMaxJobs];        // elements before job j's first vector (bits 0-6); bit 7: the job's last whole
+                                        // vector is left to the edge lanes, so that vector nvec may be read (load_vectors)
 };
 static_assert(sizeof(BatchTable) + 64 <= 4096, "the job table and the other arguments must fit the kernel-argument segment");
 
@@ -34,6 +35,7 @@ struct BatchLaunchArgs {
     int n, n_jobs, op;
     hipStream_t stream;
     Tuning tune;
+    size_t skip_from_count = 0;         // > 0: jobs of this many elements or more are left out (the caller has launched them)
 };
 
 template <class TR, int OP>
@@ -51,9 +53,10 @@ reduce_batch_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tiles) {
         }
         const int j = lo;
         const uint32_t t = it - (j ? tb.tile_end[j - 1] : 0u);
-        const uint32_t head = tb.head[j];
+        const uint32_t head = tb.head[j] & 0x7fu, beyond = tb.head[j] >> 7;
         const uint64_t count = tb.count[j];
-        const uint64_t nvec = (count - head) / TR::VEC;
+        const uint64_t nvec = (count - head) / TR::VEC - beyond;
+        const uint64_t nload = nvec + beyond;
         const uint32_t tail = (uint32_t)(count - head - nvec * TR::VEC);
         const int b = j * (n + 1);                      // the job's pointers: tb.p[b .. b + n]
         unsigned char* dst = (unsigned char*)tb.p[b + n];
@@ -61,17 +64,14 @@ reduce_batch_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tiles) {
         uint64_t idx[kBatchUnroll];
 #pragma unroll
         for (int u = 0; u < kBatchUnroll; u++) idx[u] = (uint64_t)t * kTile + threadIdx.x + (uint64_t)u * kBlock;
-        if (idx[0] < nvec) {
+        if (idx[0] < nload) {
             Accs<TR> a[kBatchUnroll];
-            const u32x4_u* s0 = (const u32x4_u*)((const unsigned char*)tb.p[b] + head * sizeof(E));
+            u32x4 x[kBatchUnroll];
+            load_vectors<sizeof(E), kBatchUnroll, false>((const unsigned char*)tb.p[b] + head * sizeof(E), idx, nvec, nload, x);
 #pragma unroll
-            for (int u = 0; u < kBatchUnroll; u++)
-                a[u] = vec_init<TR>((idx[u] < nvec) ? ld_loose(s0 + idx[u]) : u32x4{ 0, 0, 0, 0 });
+            for (int u = 0; u < kBatchUnroll; u++) a[u] = vec_init<TR>(x[u]);
             for (int k = 1; k < n; k++) {
-                const u32x4_u* sk = (const u32x4_u*)((const unsigned char*)tb.p[b + k] + head * sizeof(E));
-                u32x4 x[kBatchUnroll];
-#pragma unroll
-                for (int u = 0; u < kBatchUnroll; u++) x[u] = (idx[u] < nvec) ? ld_loose(sk + idx[u]) : u32x4{ 0, 0, 0, 0 };
+                load_vectors<sizeof(E), kBatchUnroll, false>((const unsigned char*)tb.p[b + k] + head * sizeof(E), idx, nvec, nload, x);
 #pragma unroll
                 for (int u = 0; u < kBatchUnroll; u++) vec_step<TR, OP>(x[u], a[u]);
             }
@@ -91,46 +91,254 @@ reduce_batch_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tiles) {
     }
 }
 
-// Host side: fills tables of at most kBatchMaxJobs jobs / kBatchMaxPtrs pointers and launches one kernel per table.
+// ---------------------------------------------------------------------------------------------------
+// The phased form of the same, for batches that move enough to fill whole phases (the chunks a large reduce-scatter
+// stages: N pair- or N-input reduces of a few MiB to tens of MiB each).  The jobs' vectors are laid end to end in tiles
+// of kBatchPhaseTile vectors (32 KiB of every buffer of ONE job: four vectors per lane of a block, the group that
+// reduce_multi_phased_kernel keeps in flight per input; a job's last tile is padded), and the tiles are dealt out as
+// that kernel deals out its groups: group q of block b in a phase is tile (phase x 11 + q) x grid + b, so that at every
+// step the chip reads `grid` consecutive tiles.  A block's tiles of one phase ascend, so the job of a tile is found
+// by moving a cursor along the running tile counts (scalar work on kernel arguments) from a binary search for the
+// phase's first tile.  Staging (registers and LDS), barrier, early arrival and arithmetic are those of
+// reduce_multi_phased_kernel; a job's edge elements are written directly by the block that takes its first tile.
+constexpr int kBatchPhaseG = 4;
+constexpr uint64_t kBatchPhaseTile = (uint64_t)kBatchPhaseG * kPhaseBlock;
+
+struct BatchSlot {                  // where one tile lives; the same for every lane of the block
+    bool valid;                     // false: the phase has no such tile (nvec = nload = 0: nothing is read or stored)
+    uint32_t job;                   // index into the table
+    uint32_t p0;                    // index of the job's first pointer in BatchTable::p
+    uint32_t head;                  // elements before the job's first vector
+    uint64_t first;                 // the tile's first vector, counted within the job
+    uint64_t nvec, nload;           // the job's vectors that are computed / that may be read
+};
+
+template <class TR>
+__device__ __forceinline__ BatchSlot batch_locate(const BatchTable& tb, int n, uint64_t tile, uint32_t total_tiles, int& j) {
+    if (tile >= total_tiles) return BatchSlot{ false, 0, 0, 0, 0, 0, 0 };
+    while (tb.tile_end[j] <= tile) j++;         // tile < total_tiles = tile_end[n_jobs - 1]: j stays below n_jobs
+    const uint32_t beg = j ? tb.tile_end[j - 1] : 0u;
+    const uint32_t beyond = tb.head[j] >> 7;
+    BatchSlot s;
+    s.valid = true;
+    s.job = (uint32_t)j;
+    s.p0 = (uint32_t)(j * (n + 1));
+    s.head = tb.head[j] & 0x7fu;
+    s.first = (tile - beg) * kBatchPhaseTile;
+    s.nvec = (tb.count[j] - s.head) / TR::VEC - beyond;
+    s.nload = s.nvec + beyond;
+    return s;
+}
+
+// One tile: four vectors per lane, the inputs one after the other (reduce_rt_tile for a job of the table); the block
+// that takes a job's first tile also computes the job's elements before its first and after its last vector and
+// stores them at once (a few bytes).
+template <class TR, int OP>
+__device__ __forceinline__ void reduce_batch_tile(const BatchTable& tb, int n, const BatchSlot& s, u32x4 (&out)[kBatchPhaseG],
+                                                  PhaseSync* arrive_ps = nullptr, int arrive_k = 0) {
+    typedef typename TR::elem_t E;
+    constexpr int G = kBatchPhaseG;
+    Accs<TR> a[G];
+    u32x4 x[G];
+    uint64_t idx[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) idx[g] = s.first + (uint64_t)g * kPhaseBlock + threadIdx.x;
+    load_vectors<sizeof(E), G, false>((const unsigned char*)tb.p[s.p0] + s.head * sizeof(E), idx, s.nvec, s.nload, x);
+#pragma unroll
+    for (int g = 0; g < G; g++) a[g] = vec_init<TR>(x[g]);
+    for (int k = 1; k < n; k++) {
+        if (k == arrive_k && threadIdx.x == 0) phase_arrive(arrive_ps);     // arrive_k == 0: never
+        load_vectors<sizeof(E), G, false>((const unsigned char*)tb.p[s.p0 + k] + s.head * sizeof(E), idx, s.nvec, s.nload, x);
+#pragma unroll
+        for (int g = 0; g < G; g++) vec_step<TR, OP>(x[g], a[g]);
+    }
+#pragma unroll
+    for (int g = 0; g < G; g++) out[g] = vec_finish<TR>(a[g]);
+    if (s.valid && s.first == 0) {
+        const uint32_t tail = (uint32_t)(tb.count[s.job] - s.head - s.nvec * TR::VEC);
+        if (threadIdx.x < s.head + tail) {
+            const uint32_t e = threadIdx.x;
+            const uint64_t i = (e < s.head) ? e : (uint64_t)s.head + s.nvec * TR::VEC + (e - s.head);
+            typename TR::acc_t r = TR::init(ld_elem<E>(tb.p[s.p0], i));
+            for (int k = 1; k < n; k++) r = TR::template step<OP>(ld_elem<E>(tb.p[s.p0 + k], i), r);
+            st_elem<E>((void*)tb.p[s.p0 + n], i, TR::finish(r));
+        }
+    }
+}
+
+template <class TR, int OP>
+__global__ void __launch_bounds__(kPhaseBlock)
+reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tiles, PhaseSync* ps, int early_loads,
+                           int early_stores, long spin_ticks) {
+    typedef typename TR::elem_t E;
+    kernel_prologue<TR, OP>();
+    constexpr int G = kBatchPhaseG;
+    constexpr int RG = MultiPhaseRegs<TR>::groups;
+    constexpr int LG = kPhaseU / G;
+    static_assert(kPhaseU % G == 0, "LDS steps must be a multiple of the group size");
+    __shared__ u32x4 stage[kPhaseU * kPhaseBlock];
+    const uint64_t grid = gridDim.x;
+    const uint64_t per_phase = grid * (uint64_t)(RG + LG);  // tiles
+    bool give_up = false;
+    unsigned gen = 0;
+    if (threadIdx.x == 0) gen = phase_generation(ps);
+    for (uint64_t t0 = 0; t0 < total_tiles; t0 += per_phase) {
+        const uint64_t tile0 = t0 + blockIdx.x;             // this block's tile of group q: tile0 + q * grid
+        int j0 = 0;                                         // the job of this block's first tile of the phase
+        if (tile0 < total_tiles) {
+            int lo = 0, hi = n_jobs - 1;
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if (tb.tile_end[mid] > tile0) hi = mid;
+                else lo = mid + 1;
+            }
+            j0 = lo;
+        }
+        int jr = j0;
+        u32x4 rs[G * (RG > 0 ? RG : 1)];
+#pragma unroll
+        for (int q = 0; q < RG; q++) {
+            const BatchSlot s = batch_locate<TR>(tb, n, tile0 + (uint64_t)q * grid, total_tiles, jr);
+            if (s.valid) {
+                u32x4 v[G];
+                reduce_batch_tile<TR, OP>(tb, n, s, v);
+#pragma unroll
+                for (int g = 0; g < G; g++) rs[q * G + g] = v[g];
+            }
+        }
+        bool arrived = false;
+        for (int q = 0; q < LG; q++) {
+            const BatchSlot s = batch_locate<TR>(tb, n, tile0 + (uint64_t)(RG + q) * grid, total_tiles, jr);
+            if (!s.valid) break;                            // tiles ascend with q: nothing further in this phase
+            const int rem = (LG - q) * n * G;               // loads per lane still to issue in this phase
+            int arrive_k = 0;
+            if (!arrived) {
+                const int k = rem > early_loads ? (rem - early_loads + G - 1) / G : 0;
+                if (k == 0 && threadIdx.x == 0) phase_arrive(ps);
+                arrive_k = k < n ? k : 0;
+                arrived = k < n;
+            }
+            u32x4 v[G];
+            reduce_batch_tile<TR, OP>(tb, n, s, v, ps, arrive_k);
+#pragma unroll
+            for (int g = 0; g < G; g++) stage[(q * G + g) * kPhaseBlock + threadIdx.x] = v[g];
+        }
+        if (early_loads == 0) __syncthreads();              // "when done" means the whole block, and its loads have landed
+        if (!arrived && threadIdx.x == 0) phase_arrive(ps);
+        phase_wait(ps, ++gen, give_up, spin_ticks);
+        const bool more = t0 + per_phase < total_tiles;
+        const int arrive_u = more ? kPhaseU - early_stores : -1;    // kPhaseU: after the last store
+        int jw = j0;
+#pragma unroll
+        for (int q = 0; q < RG; q++) {
+            const BatchSlot s = batch_locate<TR>(tb, n, tile0 + (uint64_t)q * grid, total_tiles, jw);
+            u32x4_u* d = (u32x4_u*)((unsigned char*)tb.p[s.p0 + n] + s.head * sizeof(E));
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const uint64_t i = s.first + (uint64_t)g * kPhaseBlock + threadIdx.x;
+                if (i < s.nvec) st_loose(d + i, rs[q * G + g]);
+            }
+        }
+        for (int q = 0; q < LG; q++) {
+            const BatchSlot s = batch_locate<TR>(tb, n, tile0 + (uint64_t)(RG + q) * grid, total_tiles, jw);
+            u32x4_u* d = (u32x4_u*)((unsigned char*)tb.p[s.p0 + n] + s.head * sizeof(E));
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const uint64_t i = s.first + (uint64_t)g * kPhaseBlock + threadIdx.x;
+                if (q * G + g == arrive_u && threadIdx.x == 0) phase_arrive(ps);
+                if (i < s.nvec) st_loose(d + i, stage[(q * G + g) * kPhaseBlock + threadIdx.x]);
+            }
+        }
+        if (more) {
+            if (arrive_u == kPhaseU) {
+                __syncthreads();                            // "when done": every wave's stores have been acknowledged
+                if (threadIdx.x == 0) phase_arrive(ps);
+            }
+            phase_wait(ps, ++gen, give_up, spin_ticks);
+        }
+    }
+}
+
+// Host side: fills tables of at most kBatchMaxJobs jobs / kBatchMaxPtrs pointers and launches one kernel per table,
+// in the phased form when the table's jobs together fill whole phases (the rule of the single reduce, wants_phased,
+// on their total), else in the streaming form.
+inline bool skipped(const BatchLaunchArgs& a, int j) {
+    return a.skip_from_count > 0 && a.counts[j] >= a.skip_from_count;
+}
+
 template <class TR, int OP>
 inline hipError_t launch_batch_op(const BatchLaunchArgs& a) {
     typedef typename TR::elem_t E;
-    constexpr uint64_t kTile = (uint64_t)kBlock * kBatchUnroll;
     const int per_launch = (kBatchMaxPtrs / (a.n + 1)) < kBatchMaxJobs ? (kBatchMaxPtrs / (a.n + 1)) : kBatchMaxJobs;
+    const uint64_t phase_grid = (uint64_t)(a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
     int j0 = 0;
     while (j0 < a.n_jobs) {
-        BatchTable tb;
+        // the jobs of this table: where each one's vectors start (the 16-byte boundary of the buffer that makes the
+        // loose accesses cheapest) and whether it leaves its last whole vector to the edge lanes (vector_split)
+        VecSplit split[kBatchMaxJobs];
         int nj = 0;
-        uint64_t tiles = 0;
+        uint64_t small_tiles = 0, phase_tiles = 0, vectors = 0;     // tiles of the streaming form (16 KiB), of the phased form (32 KiB)
+        uint32_t realigned = 0;
         for (; j0 + nj < a.n_jobs && nj < per_launch; nj++) {
             const int j = j0 + nj;
-            const uint64_t count = a.counts[j];
-            // the vectors of a job start on the 16-byte boundary of the buffer that makes the loose accesses cheapest (vector_head)
-            LaunchArgs one;
-            one.srcs = a.srcs + (size_t)j * a.n;
-            one.n = a.n;
-            one.dst = a.dsts[j];
-            one.count = count;
-            uint64_t head = count ? vector_head<E>(one) : 0;
-            if (head > count) head = count;
-            const uint64_t nvec = (count - head) / TR::VEC;
-            const uint64_t jt = count ? (nvec ? (nvec + kTile - 1) / kTile : 1) : 0;    // a job of edge elements only still gets a tile
-            if (tiles + jt > 0x7fffffffull) {
+            VecSplit v = { 0, 0, 0, 0 };
+            if (a.counts[j] && !skipped(a, j)) {
+                LaunchArgs one;
+                one.srcs = a.srcs + (size_t)j * a.n;
+                one.n = a.n;
+                one.dst = a.dsts[j];
+                one.count = a.counts[j];
+                one.tune = a.tune;
+                v = vector_split<E, TR::VEC>(one);
+            }
+            constexpr uint64_t kSmall = (uint64_t)kBlock * kBatchUnroll;
+            const bool work = a.counts[j] && !skipped(a, j);
+            const uint64_t jt = work ? (v.nvec ? (v.nvec + kSmall - 1) / kSmall : 1) : 0;   // edge elements only: still a tile
+            if (small_tiles + jt > 0x7fffffffull) {
                 if (nj == 0) return hipErrorInvalidValue;       // one job of more than 2^31 tiles (32 TiB)
                 break;                                          // the next launch takes it
             }
-            tiles += jt;
-            for (int k = 0; k < a.n; k++) tb.p[nj * (a.n + 1) + k] = a.srcs[(size_t)j * a.n + k];
-            tb.p[nj * (a.n + 1) + a.n] = a.dsts[j];
-            tb.count[nj] = count;
-            tb.tile_end[nj] = (uint32_t)tiles;
-            tb.head[nj] = (uint8_t)head;
+            small_tiles += jt;
+            phase_tiles += work ? (v.nvec ? (v.nvec + kBatchPhaseTile - 1) / kBatchPhaseTile : 1) : 0;
+            vectors += v.nvec;
+            realigned |= v.beyond;
+            split[nj] = v;
+        }
+        bool phased = false;
+        if (a.tune.sync != nullptr && a.tune.num_cus >= kPhaseGroups) {
+            if (a.tune.variant != 0) phased = a.tune.variant == 8;
+            else
+                phased = a.tune.max_blocks == 0 && a.n >= 2 &&
+                         (uint64_t)(a.n + 1) * vectors * 16u >= (uint64_t)a.tune.phased_min_bytes &&
+                         batch_phases_full_enough(vectors, phase_tiles, phase_grid * (uint64_t)(MultiPhaseRegs<TR>::groups + kPhaseU / kBatchPhaseG),
+                                                  kBatchPhaseTile, a.n);
+        }
+        const uint64_t tile = phased ? kBatchPhaseTile : (uint64_t)kBlock * kBatchUnroll;
+        BatchTable tb;
+        uint64_t tiles = 0;
+        for (int q = 0; q < nj; q++) {
+            const int j = j0 + q;
+            const bool work = a.counts[j] && !skipped(a, j);
+            tiles += work ? (split[q].nvec ? (split[q].nvec + tile - 1) / tile : 1) : 0;
+            for (int k = 0; k < a.n; k++) tb.p[q * (a.n + 1) + k] = a.srcs[(size_t)j * a.n + k];
+            tb.p[q * (a.n + 1) + a.n] = a.dsts[j];
+            tb.count[q] = work ? a.counts[j] : 0;
+            tb.tile_end[q] = (uint32_t)tiles;
+            tb.head[q] = (uint8_t)(split[q].head | (split[q].beyond << 7));
         }
         j0 += nj;
         if (tiles == 0) continue;
-        const int grid = grid_for(tiles, a.tune);
-        g_last_kernel = "reduce_batch_kernel";
-        hipLaunchKernelGGL((reduce_batch_kernel<TR, OP>), dim3(grid), dim3(kBlock), 0, a.stream, tb, a.n, nj, (uint32_t)tiles);
+        g_realigned_launches += realigned;
+        if (phased) {
+            g_last_kernel = "reduce_batch_phased_kernel";
+            hipLaunchKernelGGL((reduce_batch_phased_kernel<TR, OP>), dim3((unsigned)phase_grid), dim3(kPhaseBlock), 0, a.stream, tb, a.n,
+                               nj, (uint32_t)tiles, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks);
+        }
+        else {
+            g_last_kernel = "reduce_batch_kernel";
+            hipLaunchKernelGGL((reduce_batch_kernel<TR, OP>), dim3(grid_for(tiles, a.tune)), dim3(kBlock), 0, a.stream, tb, a.n, nj,
+                               (uint32_t)tiles);
+        }
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }

@@ -125,12 +125,12 @@ void require_gpu_memory(const void* p, size_t bytes, const char* fn, const char*
             return;
         auto it = std::upper_bound(t_known.begin(), t_known.end(), a,
                                    [](uintptr_t v, const known_range& r) { return v < r.lo; });
-        if (it != t_known.begin() && a < (it - 1)->hi) {
-            if (a + bytes > (it - 1)->hi)
-                fail(std::string(fn) + ": " + arg + " runs past the end of its allocation");
+        if (it != t_known.begin() && a + bytes <= (it - 1)->hi) {
             t_last = *(it - 1);
             return;
         }
+        // not inside anything remembered -- or past the end of a remembered allocation, which may have been freed and
+        // replaced by a larger one at the same address: ask the runtime
     }
     uintptr_t lo = 0, hi = 0;
     if (!gpu_can_reach(p, &lo, &hi))

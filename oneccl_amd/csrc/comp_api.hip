@@ -6,7 +6,6 @@
 #include <string.h>
 
 #include <atomic>
-#include <vector>
 #include <cctype>
 
 #include "../../include/mi_ccl_comp.h"
@@ -44,6 +43,7 @@ MI_DECLARE(Bf16KeepTraits<true>);
 // tuning state and device facts
 
 thread_local const char* g_last_kernel = "";
+thread_local unsigned long g_realigned_launches = 0;
 
 static std::atomic<int> g_waves_per_cu{ 256 };
 static std::atomic<int> g_max_blocks{ 0 };
@@ -54,6 +54,7 @@ static std::atomic<int> g_phase_early_loads{ 12 };
 static std::atomic<int> g_phase_early_stores{ -1 };
 static std::atomic<long> g_phase_spin_ticks{ kPhaseSpinTicks };
 static std::atomic<int> g_fp16_impl{ MI_CCL_FP16_AVX512F };
+static std::atomic<int> g_realign{ 1 };
 static std::atomic<long> g_launch_block_limit{ 0 };     // 0: what HIP allows; smaller values are for tests of the splitting
 static_assert(kGeomBlock == kBlock, "the geometry header and the kernels agree on the block size");
 
@@ -70,6 +71,7 @@ static std::atomic<int> g_num_cus[64];
 // overlapping launches lose their phase alignment and run at the unaligned speed, about a quarter slower.  (A set
 // comes round again after kPhaseSlots calls; launches that far apart and still overlapping share it, which costs
 // speed only, never correctness.)
+constexpr size_t kBatchCopyAlone = 32u << 20;      // mi_ccl_comp_reduce_batch: one-input jobs from this many bytes get copy_kernel launches of their own
 constexpr int kPhaseSlots = 16;
 static __device__ PhaseSync g_phase_sync[kPhaseSlots];
 static std::atomic<PhaseSync*> g_phase_sync_ptr[64];
@@ -116,6 +118,7 @@ Tuning current_tuning() {
     t.early_stores = g_phase_early_stores.load(std::memory_order_relaxed);
     t.spin_ticks = g_phase_spin_ticks.load(std::memory_order_relaxed);
     t.fp16_impl = g_fp16_impl.load(std::memory_order_relaxed);
+    t.realign = g_realign.load(std::memory_order_relaxed);
     return t;
 }
 
@@ -649,37 +652,21 @@ int mi_ccl_comp_reduce_batch(int dtype, int op, const void* const* srcs, int n, 
     a.tune = current_tuning();
     if (fp16_impl != MI_CCL_FP16_DEFAULT)
         a.tune.fp16_impl = fp16_impl;
-    // A job that moves as much as a launch of its own would be phased for (the chunks of a large reduce-scatter:
-    // hundreds of MB each) goes through the single-reduce path, which picks the kernel form for its size; one more
-    // launch is nothing against it.  The others share the batch launch.
-    const uint64_t big = (uint64_t)a.tune.phased_min_bytes;
-    int n_big = 0;
-    if (a.tune.variant == 0)
-        for (int j = 0; j < n_jobs; j++) n_big += (uint64_t)(n + 1) * counts[j] * esz >= big;
-    if (n_big == 0)
-        return status_of(dispatch_batch(dtype, keep, bf16_impl, a));
-    std::vector<const void*> s_small;
-    std::vector<void*> d_small;
-    std::vector<size_t> c_small;
-    for (int j = 0; j < n_jobs; j++) {
-        if ((uint64_t)(n + 1) * counts[j] * esz >= big) {
-            const int rc = reduce_n_impl(dtype, op, srcs + (size_t)j * n, n, dsts + j, 1, counts[j], lp_mode, bf16_impl,
-                                         fp16_impl, stream);
-            if (rc != MI_CCL_SUCCESS)
-                return rc;
-        }
-        else if (counts[j]) {
-            s_small.insert(s_small.end(), srcs + (size_t)j * n, srcs + (size_t)(j + 1) * n);
-            d_small.push_back(dsts[j]);
-            c_small.push_back(counts[j]);
-        }
+    // Everything a job can be refused for has been looked at above, for every job, before the first launch.  Nothing is
+    // allocated, on the host or on the device: the tables are built on the stack and travel in the kernel arguments.
+    // One input per job, rounded after every pair, is a byte copy per job (copy_data): a job of kBatchCopyAlone bytes or
+    // more goes to the copy kernel, whose one-store-per-wave shape is about a tenth faster and whose launch is
+    // nothing against such a copy; the others share the batch launch.
+    if (n == 1 && !keep && a.tune.variant == 0) {
+        const size_t from = (kBatchCopyAlone + esz - 1) / esz;
+        for (int j = 0; j < n_jobs; j++)
+            if (counts[j] >= from && dsts[j] != srcs[j]) {
+                const int rc = launch_copy(srcs[j], dsts[j], counts[j] * esz, true, (hipStream_t)stream);
+                if (rc != MI_CCL_SUCCESS)
+                    return rc;
+            }
+        a.skip_from_count = from;
     }
-    if (c_small.empty())
-        return MI_CCL_SUCCESS;
-    a.srcs = s_small.data();
-    a.dsts = d_small.data();
-    a.counts = c_small.data();
-    a.n_jobs = (int)c_small.size();
     return status_of(dispatch_batch(dtype, keep, bf16_impl, a));
 }
 
@@ -875,6 +862,10 @@ int mi_ccl_set_param(const char* name, long value) {
         g_launch_block_limit.store(value);
         return MI_CCL_SUCCESS;
     }
+    if (!strcmp(name, "realign") && (value == 0 || value == 1)) {
+        g_realign.store((int)value);
+        return MI_CCL_SUCCESS;
+    }
     return MI_CCL_INVALID_ARGUMENTS;
 }
 
@@ -903,6 +894,10 @@ long mi_ccl_get_param(const char* name) {
         return g_launch_block_limit.load();
     if (!strcmp(name, "num_cus"))
         return num_cus();
+    if (!strcmp(name, "realign"))
+        return g_realign.load();
+    if (!strcmp(name, "realigned_launches"))
+        return (long)g_realigned_launches;
     return -1;
 }
 

@@ -53,15 +53,31 @@ __device__ __forceinline__ uint32_t fusion_head(const void* out) {
     return (mis % ES) == 0 ? ((16u - mis) & 15u) / ES : 0;
 }
 
+// What the realignment in registers (load_vectors) needs of an item when any of its inputs' vectors start off a 4-byte
+// boundary: the vector behind the last computed one must be readable.  Inside a tensor it is (the next item's data:
+// `spare` bytes of the tensor follow the item); in a tensor's last item the last whole vector is left to the edge
+// lanes instead.  Returns bit 0: vector nvec may be read; bit 1: nvec was the count before one vector was taken off.
+// own / peer_off: where the item's vectors start in the own tensor and, as an offset, in every peer's buffer.
+template <uint32_t ES>
+__device__ __forceinline__ uint32_t fusion_beyond(const void* own, const PeerPtrs& peers, int n_peers, uint64_t peer_off,
+                                                  uint32_t nvec, uint64_t spare, uint32_t realign) {
+    if (ES >= 4 || !realign || nvec == 0) return 0;
+    uint32_t odd = (uint32_t)(uintptr_t)own;
+    for (int j = 0; j < n_peers; j++) odd |= (uint32_t)((uintptr_t)peers.p[j] + peer_off);
+    if ((odd & 3u) == 0) return 0;
+    return spare >= 16 ? 1u : 3u;
+}
+
 // out_t[i] = own_t[i] OP peer_0[off_t + i] OP ... : one pass, same arithmetic as reduce_multi_kernel
 template <class TR, int OP>
 __global__ void __launch_bounds__(kBlock)
 fusion_reduce_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers, const uint64_t* off,
-                     const uint64_t* bytes, const FusionItem* items, uint32_t nitems, uint32_t t0) {
+                     const uint64_t* bytes, const FusionItem* items, uint32_t nitems, uint32_t t0, uint32_t realign) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr uint32_t ES = sizeof(E);
     const uint32_t tid = threadIdx.x;
+    const uint64_t idx[4] = { tid, tid + (uint32_t)kBlock, tid + 2u * kBlock, tid + 3u * kBlock };
     for (uint32_t it = blockIdx.x; it < nitems; it += gridDim.x) {
         const FusionItem w = items[it];
         const uint64_t lo = (uint64_t)w.c * kFusionChunk;
@@ -74,31 +90,25 @@ fusion_reduce_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers
         {
             uint32_t head = fusion_head<ES>(o);
             if (head > nelem) head = nelem;
-            const uint32_t nvec = (nelem - head) / TR::VEC, tail = nelem - head - nvec * TR::VEC;
+            uint32_t nvec = (nelem - head) / TR::VEC;
+            const uint32_t beyond = fusion_beyond<ES>(a + head * ES, peers, n_peers, poff + head * ES, nvec, left - nb, realign);
+            nvec -= beyond >> 1;
+            const uint32_t tail = nelem - head - nvec * TR::VEC;
+            const uint64_t nload = nvec + (beyond & 1u);
             Accs<TR> acc[4];
-            const u32x4_u* s0 = (const u32x4_u*)(a + head * ES);
+            u32x4 x[4];
+            load_vectors<ES, 4, false>(a + head * ES, idx, nvec, nload, x);
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const uint32_t i = tid + u * kBlock;
-                acc[u] = vec_init<TR>((i < nvec) ? ld_loose(s0 + i) : u32x4{ 0, 0, 0, 0 });
-            }
+            for (int u = 0; u < 4; u++) acc[u] = vec_init<TR>(x[u]);
             for (int j = 0; j < n_peers; j++) {
-                const u32x4_u* sj = (const u32x4_u*)((const unsigned char*)peers.p[j] + poff + head * ES);
-                u32x4 x[4];
-#pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    const uint32_t i = tid + u * kBlock;
-                    x[u] = (i < nvec) ? ld_loose(sj + i) : u32x4{ 0, 0, 0, 0 };
-                }
+                load_vectors<ES, 4, false>((const unsigned char*)peers.p[j] + poff + head * ES, idx, nvec, nload, x);
 #pragma unroll
                 for (int u = 0; u < 4; u++) vec_step<TR, OP>(x[u], acc[u]);
             }
             u32x4_u* d = (u32x4_u*)(o + head * ES);
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const uint32_t i = tid + u * kBlock;
-                if (i < nvec) st_loose(d + i, vec_finish<TR>(acc[u]));
-            }
+            for (int u = 0; u < 4; u++)
+                if (idx[u] < nvec) st_loose(d + idx[u], vec_finish<TR>(acc[u]));
             if (tid < head + tail) {
                 const uint32_t i = (tid < head) ? tid : head + nvec * TR::VEC + (tid - head);
                 typename TR::acc_t r = TR::init(ld_elem<E>(a, i));
@@ -127,7 +137,7 @@ template <class TR, int OP, int NT>
 __global__ void __launch_bounds__(kPhaseBlock)
 fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, const uint64_t* off, const uint64_t* bytes,
                             const FusionItem* items, uint32_t nitems, uint32_t t0, PhaseSync* ps, int early_loads,
-                            int early_stores, long spin_ticks) {
+                            int early_stores, long spin_ticks, uint32_t realign) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr uint32_t ES = sizeof(E);
@@ -151,7 +161,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
         // item -> tensor tables -> pointers is walked once, for all items at once, instead of once per item.
         uint64_t d_a = 0, d_o = 0, d_poff = 0;
         uint32_t d_nb = 0;      // 0: no item in this slot
-        uint32_t d_head = 0;    // elements before the item's first vector
+        uint32_t d_head = 0;    // elements before the item's first vector (bits 0-7); bits 8-9: fusion_beyond's answer
         if (lane < (uint32_t)SLOTS) {
             const uint64_t it = p0 + (uint64_t)lane * gridDim.x + blockIdx.x;
             if (it < nitems) {
@@ -163,6 +173,10 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                 d_o = (uint64_t)(uintptr_t)out.p[w.t - t0] + lo;
                 d_poff = off[w.t] + lo;
                 d_head = fusion_head<ES>((const void*)(uintptr_t)d_o);
+                const uint32_t ne = d_nb / ES;
+                if (d_head > ne) d_head = ne;
+                d_head |= fusion_beyond<ES>((const void*)(uintptr_t)(d_a + d_head * ES), peers, NP, d_poff + d_head * ES,
+                                            (ne - d_head) / TR::VEC, left - d_nb, realign) << 8;
             }
         }
         // The block reports its arrival at the barriers a little before it is done (see phase_arrive): in front of the
@@ -184,16 +198,19 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
             const uint64_t poff = __shfl(d_poff, k, 64);
             const uint32_t nelem = nb / ES;
             {
-                uint32_t head = __shfl(d_head, k, 64);
-                if (head > nelem) head = nelem;
-                const uint32_t nvec = (nelem - head) / TR::VEC, tail = nelem - head - nvec * TR::VEC;
-                const u32x4_u* s[NT];
-                s[0] = (const u32x4_u*)(a + head * ES);
+                const uint32_t hb = __shfl(d_head, k, 64);
+                const uint32_t head = hb & 0xffu, beyond = (hb >> 8) & 1u;
+                const uint32_t nvec = (nelem - head) / TR::VEC - (hb >> 9), tail = nelem - head - nvec * TR::VEC;
+                const unsigned char* s[NT];
+                s[0] = a + head * ES;
 #pragma unroll
-                for (int j = 0; j < NP; j++) s[j + 1] = (const u32x4_u*)((const unsigned char*)peers.p[j] + poff + head * ES);
+                for (int j = 0; j < NP; j++) s[j + 1] = (const unsigned char*)peers.p[j] + poff + head * ES;
                 const uint64_t idx[2] = { tid, tid + (uint32_t)kPhaseBlock };
                 u32x4 res[2];
-                reduce_group_guarded<TR, OP, NT, 2>(s, idx, nvec, res);
+                if (nvec >= 2u * kPhaseBlock)       // a whole item: no lane is out of range (the same answer for the whole block)
+                    reduce_group<TR, OP, NT, 2, true>(s, idx, nvec, nvec + beyond, res);
+                else
+                    reduce_group<TR, OP, NT, 2, false>(s, idx, nvec, nvec + beyond, res);
                 if (k < S) {
                     stage[(2 * k) * kPhaseBlock + tid] = res[0];
                     stage[(2 * k + 1) * kPhaseBlock + tid] = res[1];
@@ -235,9 +252,9 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
             unsigned char* o = (unsigned char*)(uintptr_t)__shfl(d_o, k, 64);
             {
                 const uint32_t nelem = nb / ES;
-                uint32_t head = __shfl(d_head, k, 64);
-                if (head > nelem) head = nelem;
-                const uint32_t nvec = (nelem - head) / TR::VEC;
+                const uint32_t hb = __shfl(d_head, k, 64);
+                const uint32_t head = hb & 0xffu;
+                const uint32_t nvec = (nelem - head) / TR::VEC - (hb >> 9);
                 u32x4_u* d = (u32x4_u*)(o + head * ES);
                 u32x4 v0 = { 0, 0, 0, 0 }, v1 = v0;
                 if (k < S) {
@@ -272,7 +289,7 @@ inline hipError_t launch_fusion_phased(const FusionLaunchArgs& a, const FusionPt
     g_last_kernel = "fusion_reduce_phased_kernel";
     hipLaunchKernelGGL((fusion_reduce_phased_kernel<TR, OP, NT>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, own, out, pp,
                        a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0, a.tune.sync,
-                       a.tune.early_loads, phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks);
+                       a.tune.early_loads, phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks, (uint32_t)a.tune.realign);
     return hipGetLastError();
 }
 
@@ -314,7 +331,8 @@ inline hipError_t launch_fusion_op(const FusionLaunchArgs& a) {
             int grid = grid_for(i1 - i0, a.tune);
             g_last_kernel = "fusion_reduce_kernel";
             hipLaunchKernelGGL((fusion_reduce_kernel<TR, OP>), dim3(grid), dim3(kBlock), 0, a.stream, own, out, pp,
-                               a.n_peers, a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0);
+                               a.n_peers, a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0,
+                               (uint32_t)a.tune.realign);
             e = hipGetLastError();
         }
         if (e != hipSuccess)

@@ -139,25 +139,32 @@ MI_GEOM_HD inline BcastLane bcast_lane(uint32_t blk, uint32_t tid, uint32_t sect
 // priced -- 1 per input that is off it by a multiple of 4 bytes, 8 per input off it otherwise, 16 per output off it --
 // and the cheapest wins, the first destination's among equals.  (A plain majority, the rule before, put the grid on
 // seven peers 4 bytes off and paid for a loose output: 6.67 against 7.00.)
-inline unsigned loose_read_price(unsigned off) {
-    return (off & 15u) == 0 ? 0u : (off & 3u) == 0 ? 1u : 8u;
+// With the kernels' realignment in registers (reduce_kernels.hpp, load_vectors) an input off the 4-byte boundary is
+// read on that boundary like one that is a multiple of 4 bytes off, plus one more load per wave and a few ALU
+// instructions per vector.  Measured on the same 8 x 1 GiB bf16 (7.13 TB/s aligned): seven peers realigned 6.68 (-0.9 %
+// per input), eight inputs realigned 6.24 (-1.6 % per input), against -2.6 % per input for loose reads off the 4-byte
+// boundary (four of eight inputs: 6.39 loose, 6.90 realigned) and -6.4 % for a loose output: about half the price.
+constexpr unsigned kRealignedReadPrice = 4;
+inline unsigned loose_read_price(unsigned off, bool realign) {
+    return (off & 15u) == 0 ? 0u : (off & 3u) == 0 ? 1u : realign ? kRealignedReadPrice : 8u;
 }
 constexpr unsigned kLooseWritePrice = 16;
-inline unsigned grid_price(unsigned c, const unsigned* in_mis, int n, const unsigned* out_mis, int m) {
+inline unsigned grid_price(unsigned c, const unsigned* in_mis, int n, const unsigned* out_mis, int m, bool realign = false) {
     unsigned p = 0;
-    for (int j = 0; j < n; j++) p += loose_read_price(in_mis[j] - c);
+    for (int j = 0; j < n; j++) p += loose_read_price(in_mis[j] - c, realign);
     for (int k = 0; k < m; k++) p += ((out_mis[k] - c) & 15u) == 0 ? 0u : kLooseWritePrice;
     return p;
 }
-// in_mis / out_mis: the buffers' addresses modulo 16; returns the address modulo 16 at which the vectors start
-inline unsigned vector_grid(const unsigned* in_mis, int n, const unsigned* out_mis, int m) {
-    unsigned mis = out_mis[0] & 15u, best = grid_price(mis, in_mis, n, out_mis, m);
+// in_mis / out_mis: the buffers' addresses modulo 16; realign: inputs off a 4-byte boundary are realigned in registers
+// by the kernel; returns the address modulo 16 at which the vectors start
+inline unsigned vector_grid(const unsigned* in_mis, int n, const unsigned* out_mis, int m, bool realign = false) {
+    unsigned mis = out_mis[0] & 15u, best = grid_price(mis, in_mis, n, out_mis, m, realign);
     for (int k = 1; k < m; k++) {
-        const unsigned p = grid_price(out_mis[k], in_mis, n, out_mis, m);
+        const unsigned p = grid_price(out_mis[k], in_mis, n, out_mis, m, realign);
         if (p < best) { best = p; mis = out_mis[k] & 15u; }
     }
     for (int j = 0; j < n; j++) {
-        const unsigned p = grid_price(in_mis[j], in_mis, n, out_mis, m);
+        const unsigned p = grid_price(in_mis[j], in_mis, n, out_mis, m, realign);
         if (p < best) { best = p; mis = in_mis[j] & 15u; }
     }
     return mis;
@@ -173,6 +180,17 @@ inline bool phases_full_enough(uint64_t nvec, uint64_t vectors_per_phase, int n_
     if (nvec == 0 || vectors_per_phase == 0 || n_inputs < 1) return false;
     const uint64_t phases = (nvec + vectors_per_phase - 1) / vectors_per_phase;
     const double fill = (double)nvec / (double)(phases * vectors_per_phase);
+    const double need = 2.0 / n_inputs < 0.9 ? 2.0 / n_inputs : 0.9;
+    return fill >= need;
+}
+
+// The same question for a batch of jobs whose vectors are laid end to end in tiles of tile_vectors vectors, every job
+// padded to whole tiles: `vectors` result vectors in `tiles` tiles, tiles_per_phase tiles to a phase.  The padding
+// counts as empty space like the unused end of the last phase.
+inline bool batch_phases_full_enough(uint64_t vectors, uint64_t tiles, uint64_t tiles_per_phase, uint64_t tile_vectors, int n_inputs) {
+    if (vectors == 0 || tiles == 0 || tiles_per_phase == 0 || n_inputs < 1) return false;
+    const uint64_t phases = (tiles + tiles_per_phase - 1) / tiles_per_phase;
+    const double fill = (double)vectors / (double)(phases * tiles_per_phase * tile_vectors);
     const double need = 2.0 / n_inputs < 0.9 ? 2.0 / n_inputs : 0.9;
     return fill >= need;
 }

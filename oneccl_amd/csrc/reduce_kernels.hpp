@@ -57,11 +57,14 @@ struct Tuning {
     int early_stores;        // ... and stores per lane still to issue when it reports the end of its writes (< 0: per type)
     long spin_ticks;         // phased kernels: longest wait at one barrier, in 100 MHz ticks, before a block goes on alone
     int fp16_impl;           // which CPU implementation's float16 results to reproduce: 2, 3 (through fp32) or 4 (native)
+    int realign;             // 1: inputs off a 4-byte boundary are read on that boundary and realigned in registers
 };
 
 // Name of the kernel template the calling thread's most recent entry-point call launched (diagnostics and
 // measurement: lets a benchmark say which kernel its figures belong to).
 extern thread_local const char* g_last_kernel;
+// Launches by the calling thread whose inputs off a 4-byte boundary were realigned in registers (tests ask for it).
+extern thread_local unsigned long g_realigned_launches;
 
 struct LaunchArgs {
     const void* const* srcs;    // host array of n device pointers
@@ -73,6 +76,13 @@ struct LaunchArgs {
     Tuning tune;
     void* const* dsts = nullptr;    // m > 1: host array of m device pointers, the result goes to each (dst is unused)
     int m = 1;
+};
+
+// How the elements of a call are divided: `head` elements, `nvec` vectors, `tail` elements; beyond = 1: vector nvec
+// lies inside every buffer and may be read (see vector_split and load_vectors).
+struct VecSplit {
+    uint32_t head, tail, beyond;
+    uint64_t nvec;
 };
 
 // ---------------------------------------------------------------------------------------------------
@@ -539,6 +549,100 @@ __device__ __forceinline__ void st_elem(void* p, uint64_t i, E x) {
     ((LooseElem<E>*)p)[i].v = x;
 }
 
+// ---- inputs that sit 1-3 bytes off a 4-byte boundary ------------------------------------------------------------------
+// A loose vector load is nearly free while its address is a multiple of 4 and dear when it is not (every dword of the
+// lane then straddles two: 8 x 1 GiB bf16 with the peers 2 bytes off the vectors' boundary ran at 5.66 against 7.14
+// TB/s).  Such an input -- a peer's block behind an odd number of 16-bit elements, the tensors behind an odd-sized one
+// in a tightly packed fusion buffer, int8 at any odd offset -- is therefore read from the 4-byte boundary s = 1..3
+// bytes below the lane's vector, and the vector is put together in registers: its last s bytes are the first bytes of
+// the NEXT lane's load (fetched with a DPP wave shift, no memory or LDS instruction), and every dword is one
+// v_alignbyte_b32 of two neighbours.  Lane 63 has no next lane: it alone loads one more dword.  The lane behind the
+// last vector that is computed must load too (only its first dword is used), which is why the host, when any input of
+// a launch needs this, hands the last whole vector to the element-wise edge lanes: vector `nvec` is then still inside
+// every buffer and may be read (nload = nvec + 1).  All of this runs in wave-uniform control flow around the DPP.
+__device__ __forceinline__ uint32_t from_next_lane(uint32_t mine, uint32_t for_last_lane) {
+    // wave_shl:1 -- lane i reads `mine` of lane i + 1; lane 63, whose source is out of range, keeps `for_last_lane`
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)for_last_lane, (int)mine, 0x130, 0xf, 0xf, false);
+}
+template <int K>
+__device__ __forceinline__ uint32_t from_lane_of_quad(uint32_t v) {     // every lane reads lane K of its group of four
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, K * 0x55, 0xf, 0xf, false);
+}
+__device__ __forceinline__ u32x4 shift_into_place(u32x4 x, uint32_t next0, uint32_t s) {
+    u32x4 r;
+    r[0] = __builtin_amdgcn_alignbyte(x[1], x[0], s);
+    r[1] = __builtin_amdgcn_alignbyte(x[2], x[1], s);
+    r[2] = __builtin_amdgcn_alignbyte(x[3], x[2], s);
+    r[3] = __builtin_amdgcn_alignbyte(next0, x[3], s);
+    return r;
+}
+
+// The dwords behind lane 63's G vectors (sa: the input's 4-byte boundary below its first vector), fetched by ONE load
+// instruction: lane 64 - G + g fetches the one of vector g.  Zero in the other lanes and where lane 63's vector is not
+// computed.  G is 1, 2 or 4, so the fetching lanes are lanes of the wave's last group of four.
+template <int G, bool FULL>
+__device__ __forceinline__ uint32_t load_behind_last_lane(const u32x4_u* sa, const uint64_t (&idx)[G], uint64_t nvec) {
+    static_assert(G == 1 || G == 2 || G == 4, "the fetching lanes must be lanes of one group of four");
+    const uint32_t lane = threadIdx.x & 63u;
+    uint32_t e = 0;
+    if (lane >= 64u - G) {
+        // idx[lane - (64 - G)], picked by compare-and-select; the empty asm keeps the compiler from turning the chain
+        // into an indexed read of idx[], which it would put in scratch memory
+        uint32_t lo = (uint32_t)idx[0], hi = (uint32_t)(idx[0] >> 32);
+#pragma unroll
+        for (int g = 1; g < G; g++) {
+            const bool mine = lane == 64u - G + g;
+            lo = mine ? (uint32_t)idx[g] : lo;
+            hi = mine ? (uint32_t)(idx[g] >> 32) : hi;
+            asm("" : "+v"(lo), "+v"(hi));
+        }
+        const uint64_t i = (((uint64_t)hi << 32) | lo) + (63u - lane);      // lane 63's vector g
+        if (FULL || i < nvec) e = __builtin_nontemporal_load((const uint32_t*)(sa + i + 1));
+    }
+    return e;
+}
+// x[g] as loaded from sa -> the vectors that start s bytes further on; e: load_behind_last_lane's result
+template <int G>
+__device__ __forceinline__ void shift_vectors(u32x4 (&x)[G], uint32_t e, uint32_t s) {
+    if constexpr (G == 4) {
+        x[0] = shift_into_place(x[0], from_next_lane(x[0][0], from_lane_of_quad<0>(e)), s);
+        x[1] = shift_into_place(x[1], from_next_lane(x[1][0], from_lane_of_quad<1>(e)), s);
+        x[2] = shift_into_place(x[2], from_next_lane(x[2][0], from_lane_of_quad<2>(e)), s);
+        x[3] = shift_into_place(x[3], from_next_lane(x[3][0], from_lane_of_quad<3>(e)), s);
+    }
+    else if constexpr (G == 2) {
+        x[0] = shift_into_place(x[0], from_next_lane(x[0][0], from_lane_of_quad<2>(e)), s);
+        x[1] = shift_into_place(x[1], from_next_lane(x[1][0], from_lane_of_quad<3>(e)), s);
+    }
+    else {
+        x[0] = shift_into_place(x[0], from_next_lane(x[0][0], e), s);
+    }
+}
+
+// Vectors idx[0..G) of one input whose first vector starts at `base` (any alignment): x[g] is the vector for every
+// idx[g] < nvec; what the other lanes get is unspecified (they must not store).  ES: element size; FULL: the caller
+// knows that every idx[g] of every lane of the wave is below nvec.  nload > nvec switches the in-register
+// realignment on for an input that is off a 4-byte boundary (vector nvec must then be readable).  Must be called by
+// all lanes of a wave together, with idx[g] of lane i + 1 = idx[g] of lane i + 1.
+template <int ES, int G, bool FULL>
+__device__ __forceinline__ void load_vectors(const unsigned char* base, const uint64_t (&idx)[G], uint64_t nvec,
+                                             uint64_t nload, u32x4 (&x)[G]) {
+    if constexpr (ES < 4) {
+        const uint32_t s = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)base & 3u);
+        if (s != 0 && nload > nvec) {
+            const u32x4_u* sa = (const u32x4_u*)(base - s);
+#pragma unroll
+            for (int g = 0; g < G; g++) x[g] = (FULL || idx[g] < nload) ? ld_loose(sa + idx[g]) : u32x4{ 0, 0, 0, 0 };
+            const uint32_t e = load_behind_last_lane<G, FULL>(sa, idx, nvec);
+            shift_vectors<G>(x, e, s);
+            return;
+        }
+    }
+    const u32x4_u* sp = (const u32x4_u*)base;
+#pragma unroll
+    for (int g = 0; g < G; g++) x[g] = (FULL || idx[g] < nvec) ? ld_loose(sp + idx[g]) : u32x4{ 0, 0, 0, 0 };
+}
+
 // The count % VEC elements after the last full vector and the elements before the first aligned one:
 // at most 2*(VEC-1) <= 30 elements, one per lane of the first wave of block 0.
 template <class TR, int OP, class SRC>
@@ -574,48 +678,46 @@ struct TileIter {
     }
 };
 
-// Fixed N (1..8): all N*UNROLL loads of a tile are issued before the first use.
+// Fixed N (1..8): all N*UNROLL loads of a tile are issued before the first use.  `beyond` (0 or 1): vector nvec may be
+// read, which lets inputs off a 4-byte boundary be realigned in registers (load_vectors).
 template <class TR, int OP, int N, int UNROLL>
 __global__ void __launch_bounds__(kBlock)
-reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint32_t tail, int xcd_chunked) {
+reduce_vec_kernel(SrcFixed<N> src, void* dst, uint32_t head, uint64_t nvec, uint32_t tail, int xcd_chunked, uint32_t beyond) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr uint64_t kTile = (uint64_t)kBlock * UNROLL;
-    const u32x4_u* s[N];
+    const unsigned char* s[N];
 #pragma unroll
-    for (int j = 0; j < N; j++) s[j] = (const u32x4_u*)((const unsigned char*)src.p[j] + head * sizeof(E));
+    for (int j = 0; j < N; j++) s[j] = (const unsigned char*)src.p[j] + head * sizeof(E);
     u32x4_u* d = (u32x4_u*)((unsigned char*)dst + head * sizeof(E));
     const uint64_t ntiles = (nvec + kTile - 1) / kTile;
+    const uint64_t nload = nvec + beyond;
 
     for (TileIter it(ntiles, xcd_chunked); it.tile < it.end; it.tile += it.stride) {
-        const uint64_t base = it.tile * kTile + threadIdx.x;
-        if (base + (uint64_t)(UNROLL - 1) * kBlock < nvec) {
-            u32x4 x[N][UNROLL];
+        uint64_t idx[UNROLL];
 #pragma unroll
-            for (int j = 0; j < N; j++)
+        for (int u = 0; u < UNROLL; u++) idx[u] = it.tile * kTile + threadIdx.x + (uint64_t)u * kBlock;
+        u32x4 x[N][UNROLL];
+        if ((it.tile + 1) * kTile <= nvec) {        // a whole tile (the same answer for every lane of the block)
 #pragma unroll
-                for (int u = 0; u < UNROLL; u++) x[j][u] = ld_loose(s[j] + base + (uint64_t)u * kBlock);
+            for (int j = 0; j < N; j++) load_vectors<sizeof(E), UNROLL, true>(s[j], idx, nvec, nload, x[j]);
 #pragma unroll
             for (int u = 0; u < UNROLL; u++) {
                 Accs<TR> a = vec_init<TR>(x[0][u]);
 #pragma unroll
                 for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j][u], a);
-                st_loose(d + base + (uint64_t)u * kBlock, vec_finish<TR>(a));
+                st_loose(d + idx[u], vec_finish<TR>(a));
             }
         }
         else {
 #pragma unroll
+            for (int j = 0; j < N; j++) load_vectors<sizeof(E), UNROLL, false>(s[j], idx, nvec, nload, x[j]);
+#pragma unroll
             for (int u = 0; u < UNROLL; u++) {
-                const uint64_t i = base + (uint64_t)u * kBlock;
-                if (i < nvec) {
-                    u32x4 x[N];
+                Accs<TR> a = vec_init<TR>(x[0][u]);
 #pragma unroll
-                    for (int j = 0; j < N; j++) x[j] = ld_loose(s[j] + i);
-                    Accs<TR> a = vec_init<TR>(x[0]);
-#pragma unroll
-                    for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j], a);
-                    st_loose(d + i, vec_finish<TR>(a));
-                }
+                for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j][u], a);
+                if (idx[u] < nvec) st_loose(d + idx[u], vec_finish<TR>(a));
             }
         }
     }
@@ -696,42 +798,51 @@ __device__ __forceinline__ void phase_wait(PhaseSync* ps, unsigned gen, bool& gi
     __builtin_amdgcn_s_barrier();
 }
 
-// G vectors per lane at once: all G x N loads are issued before the first is used, so that a lane keeps about
-// eight 128-bit loads in flight whatever N is.  Callers branch around this (a real branch keeps the compiler
-// from hoisting the loads of later steps, which would spill).
-template <class TR, int OP, int N, int G>
-__device__ __forceinline__ void reduce_group(const u32x4_u* const (&s)[N], const uint64_t (&idx)[G], u32x4 (&out)[G]) {
-    u32x4 x[G][N];
+// G vectors per lane of N inputs (a compile-time count) at once: all N x G loads are issued before the first is
+// used, vector 0 of every input, then vector 1 of every input, ...; the inputs that are realigned in registers get
+// their one extra load each behind those, and are shifted into place when everything is under way.  base[j]: where
+// input j's first vector starts; idx, nvec, nload, FULL as for load_vectors.
+template <class TR, int OP, int N, int G, bool FULL>
+__device__ __forceinline__ void reduce_group(const unsigned char* const (&base)[N], const uint64_t (&idx)[G], uint64_t nvec,
+                                             uint64_t nload, u32x4 (&out)[G]) {
+    typedef typename TR::elem_t E;
+    u32x4 x[N][G];
+    if constexpr (sizeof(E) < 4) {
+        uint32_t s[N], e[N];
+        const u32x4_u* sa[N];
+        uint32_t any = 0;
 #pragma unroll
-    for (int g = 0; g < G; g++)
+        for (int j = 0; j < N; j++) {
+            s[j] = nload > nvec ? __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)base[j] & 3u) : 0u;
+            sa[j] = (const u32x4_u*)(base[j] - s[j]);
+            any |= s[j];
+        }
 #pragma unroll
-        for (int j = 0; j < N; j++) x[g][j] = ld_loose(s[j] + idx[g]);
+        for (int g = 0; g < G; g++)
 #pragma unroll
-    for (int g = 0; g < G; g++) {
-        Accs<TR> a = vec_init<TR>(x[g][0]);
+            for (int j = 0; j < N; j++)
+                x[j][g] = (FULL || idx[g] < (s[j] ? nload : nvec)) ? ld_loose(sa[j] + idx[g]) : u32x4{ 0, 0, 0, 0 };
+        if (any) {
 #pragma unroll
-        for (int j = 1; j < N; j++) vec_step<TR, OP>(x[g][j], a);
-        out[g] = vec_finish<TR>(a);
-    }
-}
-
-// the same for a group that may reach past the end of the buffer: slots at or beyond nvec are left alone
-template <class TR, int OP, int N, int G>
-__device__ __forceinline__ void reduce_group_guarded(const u32x4_u* const (&s)[N], const uint64_t (&idx)[G],
-                                                     uint64_t nvec, u32x4 (&out)[G]) {
-    if (idx[G - 1] < nvec) {
-        reduce_group<TR, OP, N, G>(s, idx, out);
+            for (int j = 0; j < N; j++) e[j] = s[j] ? load_behind_last_lane<G, FULL>(sa[j], idx, nvec) : 0u;
+#pragma unroll
+            for (int j = 0; j < N; j++)
+                if (s[j]) shift_vectors<G>(x[j], e[j], s[j]);
+        }
     }
     else {
 #pragma unroll
-        for (int g = 0; g < G; g++) {
-            if (idx[g] < nvec) {
-                const uint64_t one[1] = { idx[g] };
-                u32x4 o[1];
-                reduce_group<TR, OP, N, 1>(s, one, o);
-                out[g] = o[0];
-            }
-        }
+        for (int g = 0; g < G; g++)
+#pragma unroll
+            for (int j = 0; j < N; j++)
+                x[j][g] = (FULL || idx[g] < nvec) ? ld_loose((const u32x4_u*)base[j] + idx[g]) : u32x4{ 0, 0, 0, 0 };
+    }
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        Accs<TR> a = vec_init<TR>(x[0][g]);
+#pragma unroll
+        for (int j = 1; j < N; j++) vec_step<TR, OP>(x[j][g], a);
+        out[g] = vec_finish<TR>(a);
     }
 }
 
@@ -743,19 +854,17 @@ __device__ __forceinline__ void reduce_group_guarded(const u32x4_u* const (&s)[N
 
 template <class TR, int OP, int UNROLL>
 __device__ __forceinline__ void reduce_rt_tile(const SrcTable& src, int n, uint32_t head, const uint64_t (&idx)[UNROLL],
-                                               uint64_t nvec, u32x4 (&out)[UNROLL], PhaseSync* arrive_ps = nullptr,
-                                               int arrive_j = 0) {
+                                               uint64_t nvec, uint64_t nload, u32x4 (&out)[UNROLL],
+                                               PhaseSync* arrive_ps = nullptr, int arrive_j = 0) {
     typedef typename TR::elem_t E;
     Accs<TR> a[UNROLL];
-    const u32x4_u* s0 = (const u32x4_u*)((const unsigned char*)src.p[0] + head * sizeof(E));
+    u32x4 x[UNROLL];
+    load_vectors<sizeof(E), UNROLL, false>((const unsigned char*)src.p[0] + head * sizeof(E), idx, nvec, nload, x);
 #pragma unroll
-    for (int u = 0; u < UNROLL; u++) a[u] = vec_init<TR>((idx[u] < nvec) ? ld_loose(s0 + idx[u]) : u32x4{ 0, 0, 0, 0 });
+    for (int u = 0; u < UNROLL; u++) a[u] = vec_init<TR>(x[u]);
     for (int j = 1; j < n; j++) {
-        const u32x4_u* sj = (const u32x4_u*)((const unsigned char*)src.p[j] + head * sizeof(E));
-        u32x4 x[UNROLL];
         if (j == arrive_j && threadIdx.x == 0) phase_arrive(arrive_ps);     // arrive_j == 0: never
-#pragma unroll
-        for (int u = 0; u < UNROLL; u++) x[u] = (idx[u] < nvec) ? ld_loose(sj + idx[u]) : u32x4{ 0, 0, 0, 0 };
+        load_vectors<sizeof(E), UNROLL, false>((const unsigned char*)src.p[j] + head * sizeof(E), idx, nvec, nload, x);
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) vec_step<TR, OP>(x[u], a[u]);
     }
@@ -780,17 +889,18 @@ __device__ __forceinline__ void reduce_multi_edges(const SrcTable& src, int n, c
 template <class TR, int OP, int UNROLL>
 __global__ void __launch_bounds__(kBlock)
 reduce_multi_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uint64_t nvec, uint32_t tail,
-                    int xcd_chunked) {
+                    int xcd_chunked, uint32_t beyond) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr uint64_t kTile = (uint64_t)kBlock * UNROLL;
     const uint64_t ntiles = (nvec + kTile - 1) / kTile;
+    const uint64_t nload = nvec + beyond;
     for (TileIter it(ntiles, xcd_chunked); it.tile < it.end; it.tile += it.stride) {
         uint64_t idx[UNROLL];
         u32x4 v[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) idx[u] = it.tile * kTile + threadIdx.x + (uint64_t)u * kBlock;
-        reduce_rt_tile<TR, OP, UNROLL>(src, n, head, idx, nvec, v);
+        reduce_rt_tile<TR, OP, UNROLL>(src, n, head, idx, nvec, nload, v);
         for (int k = 0; k < m; k++) {
             u32x4_u* d = (u32x4_u*)((unsigned char*)dst.p[k] + head * sizeof(E));
 #pragma unroll
@@ -840,9 +950,10 @@ inline int phase_early_stores(const Tuning& t, int n_dsts) {
 template <class TR, int OP>
 __global__ void __launch_bounds__(kPhaseBlock)
 reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uint64_t nvec, uint32_t tail,
-                           PhaseSync* ps, int early_loads, int early_stores, long spin_ticks) {
+                           PhaseSync* ps, int early_loads, int early_stores, long spin_ticks, uint32_t beyond) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
+    const uint64_t nload = nvec + beyond;               // vector nvec may be read when beyond = 1 (load_vectors)
     constexpr int G = 4;                                // vectors per lane and input in flight
     constexpr int RG = MultiPhaseRegs<TR>::groups;
     constexpr int LG = kPhaseU / G;                     // groups staged in LDS
@@ -863,8 +974,8 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
             u32x4 v[G];
 #pragma unroll
             for (int g = 0; g < G; g++) idx[g] = pos(p0, q * G + g);
-            if (idx[0] < nvec) {
-                reduce_rt_tile<TR, OP, G>(src, n, head, idx, nvec, v);
+            if (idx[0] < nload) {
+                reduce_rt_tile<TR, OP, G>(src, n, head, idx, nvec, nload, v);
 #pragma unroll
                 for (int g = 0; g < G; g++) rs[q * G + g] = v[g];
             }
@@ -875,7 +986,7 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
             u32x4 v[G];
 #pragma unroll
             for (int g = 0; g < G; g++) idx[g] = pos(p0, (RG + q) * G + g);
-            if (idx[0] >= nvec) break;      // slabs grow with q: nothing further for this lane in this phase
+            if (idx[0] >= nload) break;     // slabs grow with q: nothing further for this lane in this phase
             // the arrival goes in front of the first load that leaves early_loads or fewer still to issue
             const int rem = (LG - q) * n * G;
             int arrive_j = 0;
@@ -885,7 +996,7 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
                 arrive_j = j < n ? j : 0;
                 arrived = j < n;
             }
-            reduce_rt_tile<TR, OP, G>(src, n, head, idx, nvec, v, ps, arrive_j);
+            reduce_rt_tile<TR, OP, G>(src, n, head, idx, nvec, nload, v, ps, arrive_j);
 #pragma unroll
             for (int g = 0; g < G; g++) stage[(q * G + g) * kPhaseBlock + threadIdx.x] = v[g];
         }
@@ -931,14 +1042,15 @@ inline int grid_for(uint64_t ntiles, const Tuning& t) {
 }
 
 template <class TR, int OP, int N, int UNROLL>
-inline hipError_t launch_fixed(const LaunchArgs& a, uint32_t head, uint64_t nvec, uint32_t tail) {
+inline hipError_t launch_fixed(const LaunchArgs& a, const VecSplit& v) {
     SrcFixed<N> s;
     for (int j = 0; j < N; j++) s.p[j] = a.srcs[j];
     const uint64_t tile = (uint64_t)kBlock * UNROLL;
-    int grid = grid_for((nvec + tile - 1) / tile, a.tune);
+    int grid = grid_for((v.nvec + tile - 1) / tile, a.tune);
     g_last_kernel = "reduce_vec_kernel";
+    g_realigned_launches += v.beyond;
     hipLaunchKernelGGL((reduce_vec_kernel<TR, OP, N, UNROLL>), dim3(grid), dim3(kBlock), 0, a.stream, s, a.dst,
-                       head, nvec, tail, a.tune.xcd_chunked);
+                       v.head, v.nvec, v.tail, a.tune.xcd_chunked, v.beyond);
     return hipGetLastError();
 }
 
@@ -958,17 +1070,17 @@ struct StreamUnroll {
 };
 
 template <class TR, int OP, int N>
-inline hipError_t launch_fixed_unroll(const LaunchArgs& a, uint32_t head, uint64_t nvec, uint32_t tail) {
+inline hipError_t launch_fixed_unroll(const LaunchArgs& a, const VecSplit& v) {
     constexpr int kDefault = StreamUnroll<TR>::get(N);
     if constexpr (HasUnrollVariants<TR>::value) {
         switch (a.tune.variant) {
-            case 1: return launch_fixed<TR, OP, N, 1>(a, head, nvec, tail);
-            case 2: return launch_fixed<TR, OP, N, 2>(a, head, nvec, tail);
-            case 4: return launch_fixed<TR, OP, N, 4>(a, head, nvec, tail);
+            case 1: return launch_fixed<TR, OP, N, 1>(a, v);
+            case 2: return launch_fixed<TR, OP, N, 2>(a, v);
+            case 4: return launch_fixed<TR, OP, N, 4>(a, v);
             default: break;
         }
     }
-    return launch_fixed<TR, OP, N, kDefault>(a, head, nvec, tail);
+    return launch_fixed<TR, OP, N, kDefault>(a, v);
 }
 
 // When the phased form pays: from Tuning::phased_min_bytes of traffic per launch (default 160 MB), with two or more
@@ -994,61 +1106,78 @@ inline uint64_t vector_head(const LaunchArgs& a) {
     unsigned in_mis[kMaxSrcs], out_mis[kMaxDsts];
     for (int j = 0; j < a.n; j++) in_mis[j] = (unsigned)((uintptr_t)a.srcs[j] & 15u);
     for (int k = 0; k < a.m; k++) out_mis[k] = (unsigned)((uintptr_t)(a.dsts ? a.dsts[k] : a.dst) & 15u);
-    const unsigned mis = vector_grid(in_mis, a.n, out_mis, a.m);
+    const unsigned mis = vector_grid(in_mis, a.n, out_mis, a.m, sizeof(E) < 4 && a.tune.realign);
     return (mis % sizeof(E)) == 0 ? ((16u - mis) & 15u) / sizeof(E) : 0;
+}
+
+// How the elements of a call are divided: `head` elements, `nvec` vectors, `tail` elements.  When an input's vectors
+// start off a 4-byte boundary (16- and 8-bit types only) and Tuning::realign is on, the last whole vector goes to the
+// tail (beyond = 1): the kernels may then read vector nvec, which the realignment in registers needs (load_vectors).
+template <class E, uint32_t VEC>
+inline VecSplit vector_split(const LaunchArgs& a) {
+    VecSplit v;
+    uint64_t head = vector_head<E>(a);
+    if (head > a.count) head = a.count;
+    v.head = (uint32_t)head;
+    v.nvec = (a.count - head) / VEC;
+    v.tail = (uint32_t)(a.count - head - v.nvec * VEC);
+    v.beyond = 0;
+    if (sizeof(E) < 4 && a.tune.realign && v.nvec > 0) {
+        for (int j = 0; j < a.n; j++)
+            if (((uintptr_t)a.srcs[j] + head * sizeof(E)) & 3u) v.beyond = 1;
+        if (v.beyond) {
+            v.nvec -= 1;
+            v.tail += VEC;
+        }
+    }
+    return v;
 }
 
 template <class TR, int OP>
 inline hipError_t launch_multi_op(const LaunchArgs& a) {
     typedef typename TR::elem_t E;
-    constexpr uint32_t VEC = TR::VEC;
     SrcTable s;
     DstTable d;
     for (int j = 0; j < a.n; j++) s.p[j] = a.srcs[j];
     for (int k = 0; k < a.m; k++) d.p[k] = a.dsts ? a.dsts[k] : a.dst;
-    uint64_t head = vector_head<E>(a);
-    if (head > a.count) head = a.count;
-    const uint64_t nvec = (a.count - head) / VEC;
-    const uint32_t tail = (uint32_t)(a.count - head - nvec * VEC);
-    if (wants_phased(a, nvec, MultiPhaseRegs<TR>::groups)) {
+    const VecSplit v = vector_split<E, TR::VEC>(a);
+    g_realigned_launches += v.beyond;
+    if (wants_phased(a, v.nvec, MultiPhaseRegs<TR>::groups)) {
         int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
         g_last_kernel = "reduce_multi_phased_kernel";
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
-                           a.m, (uint32_t)head, nvec, tail, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune, a.m), a.tune.spin_ticks);
+                           a.m, v.head, v.nvec, v.tail, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune, a.m),
+                           a.tune.spin_ticks, v.beyond);
         return hipGetLastError();
     }
     constexpr int UNROLL = 4;
     const uint64_t tile = (uint64_t)kBlock * UNROLL;
-    int grid = grid_for((nvec + tile - 1) / tile, a.tune);
+    int grid = grid_for((v.nvec + tile - 1) / tile, a.tune);
     g_last_kernel = "reduce_multi_kernel";
     hipLaunchKernelGGL((reduce_multi_kernel<TR, OP, UNROLL>), dim3(grid), dim3(kBlock), 0, a.stream, s, a.n, d, a.m,
-                       (uint32_t)head, nvec, tail, a.tune.xcd_chunked);
+                       v.head, v.nvec, v.tail, a.tune.xcd_chunked, v.beyond);
     return hipGetLastError();
 }
 
 template <class TR, int OP>
 inline hipError_t launch_op(const LaunchArgs& a) {
     typedef typename TR::elem_t E;
-    constexpr uint32_t VEC = TR::VEC;
     if (a.m > 1 || a.n > kMaxFixedN) return launch_multi_op<TR, OP>(a);     // run-time counts of inputs and outputs
-    uint64_t head = vector_head<E>(a);
-    if (head > a.count) head = a.count;
-    const uint64_t nvec = (a.count - head) / VEC;
-    const uint32_t tail = (uint32_t)(a.count - head - nvec * VEC);
-    if (wants_phased(a, nvec, MultiPhaseRegs<TR>::groups)) return launch_multi_op<TR, OP>(a);     // the phased kernel takes any number of inputs
+    const VecSplit v = vector_split<E, TR::VEC>(a);
+    if (wants_phased(a, v.nvec, MultiPhaseRegs<TR>::groups)) return launch_multi_op<TR, OP>(a);     // the phased kernel takes any number of inputs
     // five or more inputs in the range between latency-bound and phased (64 to 240 MB of traffic): taking the inputs
     // one after the other, as the run-time-count streaming kernel does, measures 5-12 % above loading them together
-    if (a.n >= 5 && a.tune.variant == 0 && (uint64_t)(a.n + 1) * nvec * 16u >= (uint64_t)a.tune.phased_min_bytes / 5 * 2)
+    if (a.n >= 5 && a.tune.variant == 0 && (uint64_t)(a.n + 1) * v.nvec * 16u >= (uint64_t)a.tune.phased_min_bytes / 5 * 2)
         return launch_multi_op<TR, OP>(a);
     switch (a.n) {
-        case 1: return launch_fixed_unroll<TR, OP, 1>(a, (uint32_t)head, nvec, tail);
-        case 2: return launch_fixed_unroll<TR, OP, 2>(a, (uint32_t)head, nvec, tail);
-        case 3: return launch_fixed_unroll<TR, OP, 3>(a, (uint32_t)head, nvec, tail);
-        case 4: return launch_fixed_unroll<TR, OP, 4>(a, (uint32_t)head, nvec, tail);
-        case 5: return launch_fixed_unroll<TR, OP, 5>(a, (uint32_t)head, nvec, tail);
-        case 6: return launch_fixed_unroll<TR, OP, 6>(a, (uint32_t)head, nvec, tail);
-        case 7: return launch_fixed_unroll<TR, OP, 7>(a, (uint32_t)head, nvec, tail);
-        case 8: return launch_fixed_unroll<TR, OP, 8>(a, (uint32_t)head, nvec, tail);
+        case 1: return launch_fixed_unroll<TR, OP, 1>(a, v);
+        case 2: return launch_fixed_unroll<TR, OP, 2>(a, v);
+        case 3: return launch_fixed_unroll<TR, OP, 3>(a, v);
+        case 4: return launch_fixed_unroll<TR, OP, 4>(a, v);
+        case 5: return launch_fixed_unroll<TR, OP, 5>(a, v);
+        case 6: return launch_fixed_unroll<TR, OP, 6>(a, v);
+        case 7: return launch_fixed_unroll<TR, OP, 7>(a, v);
+        case 8: return launch_fixed_unroll<TR, OP, 8>(a, v);
         default: return hipErrorInvalidValue;
     }
 }

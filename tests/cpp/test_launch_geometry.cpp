@@ -156,6 +156,10 @@ int main() {
         EXPECT(vector_grid(spread, 8, o0, 1) == 0);
         EXPECT(vector_grid(in2, 1, o0, 1) == 0);        // one input 2 bytes off costs less than a loose output
         EXPECT(vector_grid(in2, 2, o0, 1) == 0 && vector_grid(in2, 3, o0, 1) == 2);
+        // with the kernels' realignment in registers a read off the 4-byte boundary costs half: four such inputs are
+        // worth a loose output, eight are not
+        EXPECT(vector_grid(in2, 8, o0, 1, true) == 2 && vector_grid(in2, 4, o0, 1, true) == 0 && vector_grid(in2, 3, o0, 1, true) == 0);
+        EXPECT(vector_grid(spread, 8, o0, 1, true) == 0 && vector_grid(peers4, 8, o6, 1, true) == 4);
         uint64_t x = 88172645463325252ull;
         for (int it = 0; it < 20000; it++) {
             unsigned in[8], out[3];
@@ -164,13 +168,14 @@ int main() {
             const unsigned gran = 1u << ((x >> 16) % 4);        // 1-, 2-, 4- and 8-byte elements
             for (int j = 0; j < n; j++) in[j] = (unsigned)((x >> (20 + 4 * j)) & 15u) / gran * gran;
             for (int k = 0; k < m; k++) out[k] = (unsigned)((x >> (52 + 4 * k)) & 15u) / gran * gran;
-            const unsigned g = vector_grid(in, n, out, m);
+            const bool ra = (x >> 19) & 1;
+            const unsigned g = vector_grid(in, n, out, m, ra);
             bool is_one = false;
             unsigned best = ~0u;
-            for (int j = 0; j < n; j++) { is_one |= in[j] == g; const unsigned p = grid_price(in[j], in, n, out, m); if (p < best) best = p; }
-            for (int k = 0; k < m; k++) { is_one |= out[k] == g; const unsigned p = grid_price(out[k], in, n, out, m); if (p < best) best = p; }
-            EXPECT(is_one && grid_price(g, in, n, out, m) == best);
-            EXPECT(grid_price(out[0], in, n, out, m) > best || g == out[0]);    // the first destination's among equals
+            for (int j = 0; j < n; j++) { is_one |= in[j] == g; const unsigned p = grid_price(in[j], in, n, out, m, ra); if (p < best) best = p; }
+            for (int k = 0; k < m; k++) { is_one |= out[k] == g; const unsigned p = grid_price(out[k], in, n, out, m, ra); if (p < best) best = p; }
+            EXPECT(is_one && grid_price(g, in, n, out, m, ra) == best);
+            EXPECT(grid_price(out[0], in, n, out, m, ra) > best || g == out[0]);    // the first destination's among equals
         }
     }
     // whether the phased form pays: the measured crossovers (one phase holds 88 MiB of results on 256 CUs)

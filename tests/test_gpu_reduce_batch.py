@@ -20,7 +20,7 @@ def comp():
     return c
 
 
-def _run(comp, rng, dtype, op, n, counts, lp=0, impl=2, f16=0, keep=0, kind="config", in_place_every=3, mixed_align=True):
+def _run(comp, rng, dtype, op, n, counts, lp=0, impl=2, f16=0, keep=0, kind="config", in_place_every=3, mixed_align=True, variant=0):
     """Builds the jobs (every buffer inside a zero-padded holder at its own element shift), runs them in one call and
     checks every job against the oracle and every holder for writes outside the payload."""
     import torch
@@ -46,8 +46,12 @@ def _run(comp, rng, dtype, op, n, counts, lp=0, impl=2, f16=0, keep=0, kind="con
         ptrs = [h.data_ptr() + (pad + sh) * esz for h, sh in zip(holders, shifts)]
         jobs.append((ptrs, out_h.data_ptr() + (pad + out_sh) * esz, count))
         checks.append((srcs, out_h, pad + out_sh, count, holders))
-    comp.comp_reduce_batch(dtype, op, jobs, lp_mode=lp, bf16_impl=impl, fp16_impl=f16)
-    torch.cuda.synchronize()
+    comp.set_param("variant", variant)      # 8: the phased form whatever the sizes
+    try:
+        comp.comp_reduce_batch(dtype, op, jobs, lp_mode=lp, bf16_impl=impl, fp16_impl=f16)
+        torch.cuda.synchronize()
+    finally:
+        comp.set_param("variant", 0)
     kw = dict(keep=keep, bf16_impl=impl, fp16_impl=f16 or O.FP16_AVX512F)
     for j, (srcs, out_h, lo, count, holders) in enumerate(checks):
         g = to_host(out_h, np_t)
@@ -64,6 +68,9 @@ def test_every_dtype_and_op_seven_jobs(comp, dtype, op):
     rng = np.random.default_rng(7000 + dtype * 4 + op)
     for n in (1, 2, 3, 8):
         _run(comp, rng, dtype, op, n, [1, 17, 0, 4099, 15, 70_001, 1000])
+    for n in (2, 5):
+        _run(comp, rng, dtype, op, n, [1, 17, 0, 4099, 15, 70_001, 1000, 9_000], variant=8)
+        assert comp.last_kernel() == "reduce_batch_phased_kernel"
 
 
 @pytest.mark.parametrize("n_jobs", [1, 7, 64, 200])
@@ -75,10 +82,11 @@ def test_job_counts_and_mixed_sizes(comp, n_jobs):
     if n_jobs > 3:
         counts[2] = 0
         counts[3] = 1
-    _run(comp, rng, O.FLOAT32, O.SUM, 2, counts)
-    _run(comp, rng, O.INT8, O.MAX, 2, counts)
-    if n_jobs <= 64:
-        _run(comp, rng, O.BFLOAT16, O.SUM, 8, counts, lp=comp.LP_KEEP_PRECISION, keep=1)
+    for variant in (0, 8):
+        _run(comp, rng, O.FLOAT32, O.SUM, 2, counts, variant=variant)
+        _run(comp, rng, O.INT8, O.MAX, 2, counts, variant=variant)
+        if n_jobs <= 64:
+            _run(comp, rng, O.BFLOAT16, O.SUM, 8, counts, lp=comp.LP_KEEP_PRECISION, keep=1, variant=variant)
 
 
 def test_more_jobs_than_one_table_holds_with_eight_inputs(comp):
@@ -90,17 +98,32 @@ def test_more_jobs_than_one_table_holds_with_eight_inputs(comp):
 
 
 def test_large_jobs_mixed_with_small_ones(comp):
-    """Jobs that move 160 MB or more get launches of their own (the phased kernel for the two largest here), the rest
-    share one: the chunks of a large reduce-scatter beside a few stragglers, in one call, every job against the oracle.
-    All jobs large, and only the middle one large, as well."""
+    """The chunks of a large reduce-scatter beside a few stragglers in one call: when the jobs of a launch together fill
+    whole phases they run in the phased form (several phases here, job boundaries inside a phase, jobs smaller than
+    one block's share), else in the streaming form; every job against the oracle.  One input per job is a copy per
+    job: the large ones go to the copy kernel."""
     rng = np.random.default_rng(7170)
-    big2 = (340 << 20) // 4           # two fp32 inputs: 3 x 340 MiB of traffic, four nearly full phases
+    big2 = (340 << 20) // 4           # two fp32 inputs: 3 x 340 MiB of traffic each
     _run(comp, rng, O.FLOAT32, O.SUM, 2, [1000, big2, 0, 77, big2 + 5, 1 << 20, 14 << 20], in_place_every=2)
+    assert comp.last_kernel() == "reduce_batch_phased_kernel"
+    _run(comp, rng, O.FLOAT32, O.SUM, 2, [14 << 20, 14 << 20 | 1], mixed_align=False)      # 112 MiB of results: 1.3 phases
     assert comp.last_kernel() == "reduce_batch_kernel"
-    _run(comp, rng, O.FLOAT32, O.SUM, 2, [14 << 20, 14 << 20 | 1], mixed_align=False)
-    assert comp.last_kernel() == "reduce_vec_kernel"
     _run(comp, rng, O.BFLOAT16, O.SUM, 4, [5, 40 << 20, 9], lp=comp.LP_KEEP_PRECISION, keep=1)
+    assert comp.last_kernel() == "reduce_batch_phased_kernel"
     _run(comp, rng, O.INT8, O.MAX, 1, [3, 200 << 20, 4099])
+    assert comp.last_kernel() == "reduce_batch_kernel"          # the two small jobs; the large one was a copy_kernel launch
+
+
+def test_chunk_sized_jobs_take_the_phased_form(comp):
+    """64 jobs of four inputs of 1 MiB and of 4 MiB each, and seven pair-reduces of 48 MiB (the read_reduce_write shape
+    at a tmp-buffer's chunk size): by the automatic choice, all jobs in one launch."""
+    rng = np.random.default_rng(7180)
+    _run(comp, rng, O.INT32, O.SUM, 4, [(1 << 20) // 4] * 64, in_place_every=0, mixed_align=False)
+    assert comp.last_kernel() == "reduce_batch_phased_kernel"
+    _run(comp, rng, O.FLOAT16, O.SUM, 4, [(4 << 20) // 2 + (j % 3) for j in range(64)])
+    assert comp.last_kernel() == "reduce_batch_phased_kernel"
+    _run(comp, rng, O.BFLOAT16, O.SUM, 2, [(48 << 20) // 2] * 7, in_place_every=0)
+    assert comp.last_kernel() == "reduce_batch_phased_kernel"
 
 
 def test_sixteen_bit_modes_and_nan_patterns(comp):
