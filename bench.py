@@ -58,6 +58,13 @@ WORKLOADS = {
                               desc="one 64 MiB buffer written, one 16-byte store per lane, rotating over 8 buffer sets (C1's writes alone)"),
     "write_only_four_c1": dict(dtype="float32", n=0, m=1, count=16_777_216, keep=False, sets=8, probe="write_four",
                                desc="one 64 MiB buffer written, four 16-byte stores per lane, rotating over 8 buffer sets"),
+    # ... and at the footprint of the sweep's 16 MiB point (4 x 16 MiB read, 16 MiB written, 8 buffer sets)
+    "read_only_c3_16m": dict(dtype="float32", n=4, m=0, count=4_194_304, keep=False, sets=8, probe="read",
+                             desc="four 16 MiB buffers read, nothing written, rotating over 8 buffer sets"),
+    "write_only_one_c3_16m": dict(dtype="float32", n=0, m=1, count=4_194_304, keep=False, sets=8, probe="write_one",
+                                  desc="one 16 MiB buffer written, one 16-byte store per lane, rotating over 8 buffer sets"),
+    "c3_fp32_16m": dict(dtype="float32", n=4, count=4_194_304, keep=False, sets=8,
+                        desc="4-input fp32 sum, 4,194,304 elements per buffer (16 MiB), rotating over 8 buffer sets"),
     "memcpy_dtod": dict(dtype="bfloat16", n=1, count=1_003_782_144, keep=False, sets=1, probe="memcpy",
                         desc="hipMemcpyDtoDAsync of 2,007,564,288 bytes (the runtime's own device-to-device copy)"),
 }

@@ -42,15 +42,27 @@ for p_ in (ROOT, os.path.join(ROOT, "tests")):
         sys.path.insert(0, p_)
 
 
+MARK = {"on": False, "buf": None, "segments": 0, "comp": None}
+
+
 def timed(torch, fn, steps, warm):
+    """Microseconds per call over `steps` back-to-back calls after `warm` untimed ones.  With --markers the timed calls
+    sit between two marker launches of the library's probe kernels (a four-store write probe before, a one-store
+    write probe after, on a 4 KiB buffer), so that a profiler's list of dispatches can be cut into the rows of the
+    table: the n-th pair of markers encloses the n-th timed loop."""
     for i in range(warm):
         fn(i)
+    if MARK["on"]:
+        MARK["comp"].probe_bandwidth(MARK["comp"].PROBE_WRITE_FOUR, [MARK["buf"]], 4096)
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     e0.record()
     for i in range(steps):
         fn(i)
     e1.record()
+    if MARK["on"]:
+        MARK["comp"].probe_bandwidth(MARK["comp"].PROBE_WRITE_ONE, [MARK["buf"]], 4096)
+    MARK["segments"] += 1
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) / steps * 1e3      # us
 
@@ -62,6 +74,7 @@ def main():
     ap.add_argument("--only", default="")
     ap.add_argument("--c3-k", default="", help="comma-separated exponents k of the C3 sizes 1 KiB x 4^k (default: all 11)")
     ap.add_argument("--set", action="append", default=[], metavar="NAME=VALUE", help="launch knob (mi_ccl_set_param)")
+    ap.add_argument("--markers", action="store_true", help="enclose every timed loop in two marker launches (for profiler runs)")
     args = ap.parse_args()
     only = [x for x in args.only.split(",") if x]
     skip = [x for x in args.skip.split(",") if x]
@@ -81,10 +94,15 @@ def main():
     res = {}
     rows = []
     checked = [0]
+    if args.markers:
+        MARK.update(on=True, buf=torch.zeros(4096, dtype=torch.uint8, device="cuda"), comp=comp)
+    seen_segments = [0]
 
     def add(name, us, byts, extra=""):
         gbs = byts / us / 1e3
-        res[name] = dict(us=round(us, 2), GBps=round(gbs, 1), bytes=byts, pct_hbm_peak=round(gbs / 80.0, 2), checked=True)
+        res[name] = dict(us=round(us, 2), GBps=round(gbs, 1), bytes=byts, pct_hbm_peak=round(gbs / 80.0, 2), checked=True,
+                         timed_loops=list(range(seen_segments[0], MARK["segments"])))     # which timed loops belong to the row
+        seen_segments[0] = MARK["segments"]
         rows.append(f"| {name} | {byts:,} | {us:,.1f} | {gbs:,.0f} | {gbs / 80.0:.1f} % | {extra} |")
 
     INT_VIEW = {1: torch.int8, 2: torch.int16, 4: torch.int32, 8: torch.int64}

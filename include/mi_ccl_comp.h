@@ -125,13 +125,16 @@ int mi_ccl_comp_reduce_write_n(int dtype, int op, const void* const* srcs, int n
  * dsts[j][i] = srcs[j * n + 0][i] OP srcs[j * n + 1][i] OP ... OP srcs[j * n + n - 1][i] (1 <= n <= 8, the same for every
  * job).  srcs (n_jobs x n pointers, job after job), dsts and counts are HOST arrays; a job's output may be one of its
  * own inputs, the jobs must not overlap one another; a job with count 0 is skipped without looking at its pointers.
- * The job table travels in the kernel arguments (96 jobs or 320 pointers (inputs and outputs) per launch, more jobs take more launches):
- * nothing is allocated.  Replaces read_reduce_write (n = 2: even[i] = pair[i] + local[i] for every peer i in one kernel,
- * src/coll/algorithms/reduce_scatter/sycl/reduce_scatter_large_sycl_impl.hpp:22-66), reduce_read_write_kernel_{1..7}
- * (src/kernels/kernels.cl:156-177) and, with n = 1, copy_data (N copies in one kernel, used at :216-224 of the same
- * file); it is also the small-message path: 64 reduces of a few KiB cost one launch, not 64.  A job that moves
- * "phased_min_bytes" (160 MB) or more, (n + 1) x its bytes, gets a launch of its own in the kernel form its size calls
- * for (still nothing allocated on the device).  lp_mode: MI_CCL_LP_PAIRWISE or MI_CCL_LP_KEEP_PRECISION (bfloat16). */
+ * The job table travels in the kernel arguments (96 jobs or 320 pointers (inputs and outputs) per launch, more jobs take
+ * more launches): nothing is allocated, on the host or on the device.  Every job's arguments are checked before the
+ * first launch, so an argument error leaves every output as it was.  Replaces read_reduce_write (n = 2: even[i] = pair[i]
+ * + local[i] for every peer i in one kernel, src/coll/algorithms/reduce_scatter/sycl/reduce_scatter_large_sycl_impl.hpp:22-66),
+ * reduce_read_write_kernel_{1..7} (src/kernels/kernels.cl:156-177) and, with n = 1, copy_data (N copies in one kernel,
+ * used at :216-224 of the same file); it is also the small-message path: 64 reduces of a few KiB cost one launch, not
+ * 64.  The jobs of a launch that together fill whole phases (from "phased_min_bytes" = 160 MB of traffic, two or more
+ * inputs: the chunks a large reduce-scatter stages) run in the phased kernel form, all jobs in one launch; with one
+ * input per job, a job of 32 MiB or more is a launch of the copy kernel.  lp_mode: MI_CCL_LP_PAIRWISE or
+ * MI_CCL_LP_KEEP_PRECISION (bfloat16). */
 int mi_ccl_comp_reduce_batch(int dtype, int op, const void* const* srcs, int n, void* const* dsts,
                              const size_t* counts, int n_jobs, int lp_mode, int bf16_impl, int fp16_impl,
                              void* stream);
@@ -245,7 +248,7 @@ const char* mi_ccl_last_kernel(void);
  * "phased_min_bytes" (scales the sizes from which the phased kernels are used; default 160 MB),
  * "phase_early_loads" / "phase_early_stores" (phased kernels: how many 16-byte loads / stores per lane a block still
  * has to issue when it reports the end of its read / write phase to the chip-wide barrier, which hides the barrier's
- * latency; defaults 12 and -1 = chosen per element type, 4 or 16, and 0 with three or more destinations; 0 = report
+ * latency; defaults 12 and -1 = chosen per element type, 4 or 16, and 16 with several destinations; 0 = report
  * when the whole block is done and its stores are acknowledged; timing only, results do not
  * depend on them), "phase_spin_ticks" (phased kernels: the longest a block waits at one barrier, in 100 MHz ticks,
  * before it goes on alone and stops waiting for the rest of the launch; default 20000 = 200 us; 0 = never wait, which

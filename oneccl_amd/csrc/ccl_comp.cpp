@@ -8,6 +8,7 @@
 #include <algorithm>
 
 #include "../../include/mi_ccl_comp.h"
+#include "ccl_trace.hpp"
 
 namespace {
 
@@ -280,6 +281,7 @@ void ccl_comp_forget_pointers() {
 }
 
 ccl::status ccl_comp_copy(const void* in_buf, void* out_buf, size_t bytes, bool use_nontemporal, ccl_sched* sched) {
+    ccl_trace_range tr("ccl_comp_copy");
     require_gpu_memory(in_buf, bytes, "ccl_comp_copy", "in_buf");
     require_gpu_memory(out_buf, bytes, "ccl_comp_copy", "out_buf");
     return to_status(mi_ccl_comp_copy(in_buf, out_buf, bytes, use_nontemporal ? 1 : 0, stream_of(sched)),
@@ -289,6 +291,7 @@ ccl::status ccl_comp_copy(const void* in_buf, void* out_buf, size_t bytes, bool 
 ccl::status ccl_comp_reduce(ccl_sched* sched, const void* in_buf, size_t in_count, void* inout_buf,
                             size_t* out_count, const ccl_datatype& dtype, ccl::reduction reduction,
                             ccl::reduction_fn reduction_fn, const ccl::fn_context* context) {
+    ccl_trace_range tr("ccl_comp_reduce");
     if (!in_count)
         return ccl::status::success;                                   // comp.cpp:132-134
     if (reduction == ccl::reduction::custom) {
@@ -314,6 +317,7 @@ ccl::status ccl_comp_batch_reduce(const void* in_buf, const std::vector<size_t>&
                                   ccl::reduction reduction, ccl::reduction_fn reduction_fn,
                                   const ccl::fn_context* context, int bf16_keep_precision_mode, float* tmp,
                                   float* acc, ccl_sched* sched) {
+    ccl_trace_range tr("ccl_comp_batch_reduce");
     (void)tmp;
     (void)acc;
     if (reduction == ccl::reduction::custom) {                         // chain of pairwise calls, comp.cpp:236-245
@@ -420,6 +424,7 @@ void ccl_convert_fp16_to_fp32_arrays(const void* fp16_buf, float* fp32_buf, size
 ccl::status ccl_comp_reduce_n(ccl_sched* sched, const void* own_buf, const std::vector<const void*>& peer_bufs,
                               size_t count, void* out_buf, const ccl_datatype& dtype, ccl::reduction reduction,
                               int bf16_keep_precision_mode) {
+    ccl_trace_range tr("ccl_comp_reduce_n");
     if (!count)
         return ccl::status::success;
     if (reduction == ccl::reduction::custom)
@@ -439,6 +444,7 @@ ccl::status ccl_comp_reduce_n(ccl_sched* sched, const void* own_buf, const std::
 ccl::status ccl_comp_reduce_write_n(ccl_sched* sched, const void* own_buf, const std::vector<const void*>& peer_bufs,
                                     size_t count, const std::vector<void*>& out_bufs, const ccl_datatype& dtype,
                                     ccl::reduction reduction, int bf16_keep_precision_mode) {
+    ccl_trace_range tr("ccl_comp_reduce_write_n");
     if (!count)
         return ccl::status::success;
     if (reduction == ccl::reduction::custom)
@@ -459,6 +465,7 @@ ccl::status ccl_comp_reduce_write_n(ccl_sched* sched, const void* own_buf, const
 ccl::status ccl_comp_reduce_batch(ccl_sched* sched, const std::vector<const void*>& srcs, int n_inputs,
                                   const std::vector<void*>& dsts, const std::vector<size_t>& counts,
                                   const ccl_datatype& dtype, ccl::reduction reduction, int bf16_keep_precision_mode) {
+    ccl_trace_range tr("ccl_comp_reduce_batch");
     if (dsts.empty())
         return ccl::status::success;
     if (reduction == ccl::reduction::custom)

@@ -3,6 +3,7 @@
 
 #include "../../include/mi_ccl_comp.h"
 #include "ccl_fusion.hpp"
+#include "ccl_trace.hpp"
 
 struct ccl_fusion_hip_backend::impl {
     // fusion plans cached by (dtype, counts), the way the reference caches the fused schedule by its key
@@ -50,6 +51,7 @@ void ccl_fusion_hip_backend::release(void* buf) {
 
 void ccl_fusion_hip_backend::pack(const std::vector<const void*>& tensors, const std::vector<size_t>& counts,
                                   const ccl_datatype& dtype, void* fusion_buf, void* stream) {
+    ccl_trace_range tr("ccl_fusion pack");
     int rc = mi_ccl_fusion_pack(p->plan_for(counts, dtype), tensors.data(), fusion_buf, stream);
     if (rc != MI_CCL_SUCCESS)
         throw ccl::exception(std::string("mi_ccl_fusion_pack: ") + mi_ccl_status_str(rc));
@@ -57,6 +59,7 @@ void ccl_fusion_hip_backend::pack(const std::vector<const void*>& tensors, const
 
 void ccl_fusion_hip_backend::unpack(const void* fusion_buf, const std::vector<void*>& tensors,
                                     const std::vector<size_t>& counts, const ccl_datatype& dtype, void* stream) {
+    ccl_trace_range tr("ccl_fusion unpack");
     int rc = mi_ccl_fusion_unpack(p->plan_for(counts, dtype), fusion_buf, tensors.data(), stream);
     if (rc != MI_CCL_SUCCESS)
         throw ccl::exception(std::string("mi_ccl_fusion_unpack: ") + mi_ccl_status_str(rc));

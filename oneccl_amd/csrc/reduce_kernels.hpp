@@ -934,13 +934,13 @@ template <bool RNE>
 struct PhaseEarlyStores<Bf16KeepTraits<RNE>> {
     static constexpr int value = 4;
 };
-// With three or more destinations a block stores several hundred vectors per lane and phase, its waves drift apart,
-// and an early report from one of them lets the next reads start under far too many outstanding writes: there the
-// block reports when every wave's stores have been acknowledged (8 -> 8 at 1 GiB: 6.27 against 5.79 TB/s, 4 -> 4: 6.20
-// against 5.87; 8 -> 2 and 2 -> 2 still gain 0.5-2 % from the early report).
+// With several destinations the block's waves meet before each of them (see the write phase below), so the report
+// that goes out 16 stores before the end of the last destination speaks for the whole block; without that meeting an
+// early report with three or more destinations let the next reads start under far too many outstanding writes (8 -> 8
+// at 1 GiB: 5.78 TB/s with 4 stores early against 6.25 with a strict report, 6.45 with the meeting and 16 early).
 template <class TR>
 inline int phase_early_stores(const Tuning& t, int n_dsts) {
-    const int v = t.early_stores >= 0 ? t.early_stores : n_dsts >= 3 ? 0 : PhaseEarlyStores<TR>::value;
+    const int v = t.early_stores >= 0 ? t.early_stores : n_dsts >= 2 ? 16 : PhaseEarlyStores<TR>::value;
     return v < kPhaseU ? v : kPhaseU;
 }
 
@@ -1006,6 +1006,12 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
         const bool more = p0 + per_phase < nvec;
         const int arrive_u = more ? kPhaseU - early_stores : -1;    // kPhaseU: after the last store
         for (int k = 0; k < m; k++) {
+            // The block's waves start every destination together: left alone they drift apart over the several hundred
+            // stores per lane of a phase with many destinations, the chip then writes to several destinations at once,
+            // and an early report from the first wave says little about the others (8 -> 8 at 1 GiB: 6.45 against 6.25
+            // TB/s, 4 -> 4: 6.37 against 6.17, 8 -> 16: 6.2 against 5.95; a further meeting half-way through a destination
+            // costs 1 % again).
+            if (k > 0) __syncthreads();
             u32x4_u* d = (u32x4_u*)((unsigned char*)dst.p[k] + head * sizeof(E));
 #pragma unroll
             for (int u = 0; u < G * RG; u++) {

@@ -17,6 +17,7 @@
 #include "../../oneccl_amd/csrc/ccl_comp.hpp"
 #include "../../oneccl_amd/csrc/ccl_fusion.hpp"
 #include "../../oneccl_amd/csrc/ccl_pipeline.hpp"
+#include "../../oneccl_amd/csrc/ccl_trace.hpp"
 #include "../../include/mi_ccl_comp.h"
 #include "../../oracle/ccl_comp_oracle.h"
 
@@ -607,6 +608,22 @@ int main() {
         ccl_comp_reduce(&sched, d_a.p, count, d_b.p, nullptr, f32, ccl::reduction::sum, nullptr);
         EXPECT(d_b.host()[17] == 7.0f, "check_pointers = 0");
         ccl::global_data::env().check_pointers = 1;
+    }
+    // profiler ranges around the operator-level calls: none unless switched on (MI_CCL_TRACE=1 or ccl_trace_enable)
+    {
+        DevBuf<float> a(std::vector<float>(64, 1.0f)), b(std::vector<float>(64, 2.0f));
+        const unsigned long before = ccl_trace_ranges_opened();
+        if (!getenv("MI_CCL_TRACE")) {
+            ccl_comp_reduce(&sched, a.p, 64, b.p, nullptr, DT(ccl::datatype::float32), ccl::reduction::sum, nullptr);
+            EXPECT(ccl_trace_ranges_opened() == before, "a range was opened with the knob off");
+        }
+        ccl_trace_enable(true);
+        const unsigned long on0 = ccl_trace_ranges_opened();
+        ccl_comp_reduce(&sched, a.p, 64, b.p, nullptr, DT(ccl::datatype::float32), ccl::reduction::sum, nullptr);
+        ccl_comp_copy(a.p, b.p, 64 * 4, false, &sched);
+        EXPECT(ccl_trace_ranges_opened() == on0 + 2, "two calls, two ranges");
+        ccl_trace_enable(false);
+        EXPECT(b.host()[5] == 1.0f, "results with ranges on");
     }
     CK(hipStreamDestroy(stream));
     printf("%d checks, %d failed\n", g_checks, g_fail);
