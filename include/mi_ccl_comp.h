@@ -259,7 +259,13 @@ const char* mi_ccl_last_kernel(void);
  * default 1: an input of a 16- or 8-bit type whose vectors start off a 4-byte boundary -- a peer's block behind an odd
  * number of elements, a tensor behind an odd-sized one in a tight fusion buffer -- is read on that boundary and shifted
  * into place in registers instead of with misaligned vector loads; same results, about a fifth faster for such
- * layouts) and "realigned_launches" (read only: how many launches of the calling thread took that path).
+ * layouts), "realigned_launches" (read only: how many launches of the calling thread took that path), "line_start"
+ * (0/1, default 1: a reduce, copy or broadcast of 1 MiB or more per buffer starts its 16-byte vectors on a 128-byte
+ * line of the buffers that matter most -- the outputs before the inputs -- so up to 127 bytes at the front are
+ * handled element by element; buffers that share an offset from the lines then run like aligned ones, +6 %) and
+ * "wave_runs" (phased kernels: a wave's vectors of one step lie next to each other instead of a block apart, which
+ * halves to quarters the lines two waves share; 0 never, 1 = default, when a buffer is off the 128-byte lines, 2
+ * always).  Neither changes a result.
  * Returns invalid_arguments for an unknown name or out-of-range value. */
 int mi_ccl_set_param(const char* name, long value);
 long mi_ccl_get_param(const char* name);

@@ -100,7 +100,7 @@ reduce_batch_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tiles) {
 // step the chip reads `grid` consecutive tiles.  A block's tiles of one phase ascend, so the job of a tile is found
 // by moving a cursor along the running tile counts (scalar work on kernel arguments) from a binary search for the
 // phase's first tile.  Staging (registers and LDS), barrier, early arrival and arithmetic are those of
-// reduce_multi_phased_kernel; a job's edge elements are written directly by the block that takes its first tile.
+// reduce_multi_phased_kernel; the jobs' edge elements are computed after the last phase, job j by block j mod grid.
 constexpr int kBatchPhaseG = 4;
 constexpr uint64_t kBatchPhaseTile = (uint64_t)kBatchPhaseG * kPhaseBlock;
 
@@ -130,19 +130,24 @@ __device__ __forceinline__ BatchSlot batch_locate(const BatchTable& tb, int n, u
     return s;
 }
 
-// One tile: four vectors per lane, the inputs one after the other (reduce_rt_tile for a job of the table); the block
-// that takes a job's first tile also computes the job's elements before its first and after its last vector and
-// stores them at once (a few bytes).
+// One tile: four vectors per lane, the inputs one after the other (reduce_rt_tile for a job of the table).
+// Vector g of this lane within a tile: the four lie a quarter of the tile apart, or -- wave_runs, for buffers off the
+// 128-byte lines -- 64 vectors apart, so that a wave covers 4 KiB in one run (see reduce_multi_phased_kernel).
+__device__ __forceinline__ uint32_t batch_tile_vector(int g, uint32_t wave_runs) {
+    return wave_runs ? (threadIdx.x & ~63u) * kBatchPhaseG + (uint32_t)g * 64u + (threadIdx.x & 63u)
+                     : (uint32_t)g * kPhaseBlock + threadIdx.x;
+}
+
 template <class TR, int OP>
-__device__ __forceinline__ void reduce_batch_tile(const BatchTable& tb, int n, const BatchSlot& s, u32x4 (&out)[kBatchPhaseG],
-                                                  PhaseSync* arrive_ps = nullptr, int arrive_k = 0) {
+__device__ __forceinline__ void reduce_batch_tile(const BatchTable& tb, int n, const BatchSlot& s, uint32_t wave_runs,
+                                                  u32x4 (&out)[kBatchPhaseG], PhaseSync* arrive_ps = nullptr, int arrive_k = 0) {
     typedef typename TR::elem_t E;
     constexpr int G = kBatchPhaseG;
     Accs<TR> a[G];
     u32x4 x[G];
     uint64_t idx[G];
 #pragma unroll
-    for (int g = 0; g < G; g++) idx[g] = s.first + (uint64_t)g * kPhaseBlock + threadIdx.x;
+    for (int g = 0; g < G; g++) idx[g] = s.first + batch_tile_vector(g, wave_runs);
     load_vectors<sizeof(E), G, false>((const unsigned char*)tb.p[s.p0] + s.head * sizeof(E), idx, s.nvec, s.nload, x);
 #pragma unroll
     for (int g = 0; g < G; g++) a[g] = vec_init<TR>(x[g]);
@@ -154,22 +159,31 @@ __device__ __forceinline__ void reduce_batch_tile(const BatchTable& tb, int n, c
     }
 #pragma unroll
     for (int g = 0; g < G; g++) out[g] = vec_finish<TR>(a[g]);
-    if (s.valid && s.first == 0) {
-        const uint32_t tail = (uint32_t)(tb.count[s.job] - s.head - s.nvec * TR::VEC);
-        if (threadIdx.x < s.head + tail) {
-            const uint32_t e = threadIdx.x;
-            const uint64_t i = (e < s.head) ? e : (uint64_t)s.head + s.nvec * TR::VEC + (e - s.head);
-            typename TR::acc_t r = TR::init(ld_elem<E>(tb.p[s.p0], i));
-            for (int k = 1; k < n; k++) r = TR::template step<OP>(ld_elem<E>(tb.p[s.p0 + k], i), r);
-            st_elem<E>((void*)tb.p[s.p0 + n], i, TR::finish(r));
-        }
+}
+
+// A job's elements before its first and after its last vector, one per lane (at most 127 + 2 * VEC - 1 of them).
+template <class TR, int OP>
+__device__ __forceinline__ void reduce_batch_edges(const BatchTable& tb, int n, int j) {
+    typedef typename TR::elem_t E;
+    const uint64_t count = tb.count[j];
+    if (count == 0) return;
+    const uint32_t head = tb.head[j] & 0x7fu, beyond = tb.head[j] >> 7;
+    const uint64_t nvec = (count - head) / TR::VEC - beyond;
+    const uint32_t tail = (uint32_t)(count - head - nvec * TR::VEC);
+    if (threadIdx.x < head + tail) {
+        const uint32_t p0 = (uint32_t)(j * (n + 1));
+        const uint32_t e = threadIdx.x;
+        const uint64_t i = (e < head) ? e : (uint64_t)head + nvec * TR::VEC + (e - head);
+        typename TR::acc_t r = TR::init(ld_elem<E>(tb.p[p0], i));
+        for (int k = 1; k < n; k++) r = TR::template step<OP>(ld_elem<E>(tb.p[p0 + k], i), r);
+        st_elem<E>((void*)tb.p[p0 + n], i, TR::finish(r));
     }
 }
 
 template <class TR, int OP>
 __global__ void __launch_bounds__(kPhaseBlock)
 reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tiles, PhaseSync* ps, int early_loads,
-                           int early_stores, long spin_ticks) {
+                           int early_stores, long spin_ticks, uint32_t wave_runs) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr int G = kBatchPhaseG;
@@ -201,7 +215,7 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
             const BatchSlot s = batch_locate<TR>(tb, n, tile0 + (uint64_t)q * grid, total_tiles, jr);
             if (s.valid) {
                 u32x4 v[G];
-                reduce_batch_tile<TR, OP>(tb, n, s, v);
+                reduce_batch_tile<TR, OP>(tb, n, s, wave_runs, v);
 #pragma unroll
                 for (int g = 0; g < G; g++) rs[q * G + g] = v[g];
             }
@@ -219,7 +233,7 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
                 arrived = k < n;
             }
             u32x4 v[G];
-            reduce_batch_tile<TR, OP>(tb, n, s, v, ps, arrive_k);
+            reduce_batch_tile<TR, OP>(tb, n, s, wave_runs, v, ps, arrive_k);
 #pragma unroll
             for (int g = 0; g < G; g++) stage[(q * G + g) * kPhaseBlock + threadIdx.x] = v[g];
         }
@@ -235,7 +249,7 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
             u32x4_u* d = (u32x4_u*)((unsigned char*)tb.p[s.p0 + n] + s.head * sizeof(E));
 #pragma unroll
             for (int g = 0; g < G; g++) {
-                const uint64_t i = s.first + (uint64_t)g * kPhaseBlock + threadIdx.x;
+                const uint64_t i = s.first + batch_tile_vector(g, wave_runs);
                 if (i < s.nvec) st_loose(d + i, rs[q * G + g]);
             }
         }
@@ -244,7 +258,7 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
             u32x4_u* d = (u32x4_u*)((unsigned char*)tb.p[s.p0 + n] + s.head * sizeof(E));
 #pragma unroll
             for (int g = 0; g < G; g++) {
-                const uint64_t i = s.first + (uint64_t)g * kPhaseBlock + threadIdx.x;
+                const uint64_t i = s.first + batch_tile_vector(g, wave_runs);
                 if (q * G + g == arrive_u && threadIdx.x == 0) phase_arrive(ps);
                 if (i < s.nvec) st_loose(d + i, stage[(q * G + g) * kPhaseBlock + threadIdx.x]);
             }
@@ -257,6 +271,10 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
             phase_wait(ps, ++gen, give_up, spin_ticks);
         }
     }
+    // The jobs' edge elements, after the last phase and spread over the blocks: their loads depend on one another (the
+    // inputs are taken in order), and inside a read phase that chain of round trips held up the one block of a job's
+    // first tile, and with it the barrier (64 jobs of 4 x 4 MiB with 112-byte heads: 241 us against 222 us).
+    for (int j = blockIdx.x; j < n_jobs; j += gridDim.x) reduce_batch_edges<TR, OP>(tb, n, j);
 }
 
 // Host side: fills tables of at most kBatchMaxJobs jobs / kBatchMaxPtrs pointers and launches one kernel per table,
@@ -316,6 +334,7 @@ inline hipError_t launch_batch_op(const BatchLaunchArgs& a) {
         const uint64_t tile = phased ? kBatchPhaseTile : (uint64_t)kBlock * kBatchUnroll;
         BatchTable tb;
         uint64_t tiles = 0;
+        uint32_t off_lines = 0;         // does any buffer's first vector start off a 128-byte line?
         for (int q = 0; q < nj; q++) {
             const int j = j0 + q;
             const bool work = a.counts[j] && !skipped(a, j);
@@ -325,14 +344,19 @@ inline hipError_t launch_batch_op(const BatchLaunchArgs& a) {
             tb.count[q] = work ? a.counts[j] : 0;
             tb.tile_end[q] = (uint32_t)tiles;
             tb.head[q] = (uint8_t)(split[q].head | (split[q].beyond << 7));
+            if (work)
+                for (int k = 0; k <= a.n; k++)
+                    off_lines |= (uint32_t)((uintptr_t)tb.p[q * (a.n + 1) + k] + split[q].head * sizeof(E)) & (kLineBytes - 1);
         }
+        const uint32_t wave_runs = a.tune.wave_runs == 2 || (a.tune.wave_runs == 1 && off_lines);
         j0 += nj;
         if (tiles == 0) continue;
         g_realigned_launches += realigned;
         if (phased) {
             g_last_kernel = "reduce_batch_phased_kernel";
             hipLaunchKernelGGL((reduce_batch_phased_kernel<TR, OP>), dim3((unsigned)phase_grid), dim3(kPhaseBlock), 0, a.stream, tb, a.n,
-                               nj, (uint32_t)tiles, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks);
+                               nj, (uint32_t)tiles, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks,
+                               wave_runs);
         }
         else {
             g_last_kernel = "reduce_batch_kernel";

@@ -55,6 +55,8 @@ static std::atomic<int> g_phase_early_stores{ -1 };
 static std::atomic<long> g_phase_spin_ticks{ kPhaseSpinTicks };
 static std::atomic<int> g_fp16_impl{ MI_CCL_FP16_AVX512F };
 static std::atomic<int> g_realign{ 1 };
+static std::atomic<int> g_line_start{ 1 };
+static std::atomic<int> g_wave_runs{ 1 };
 static std::atomic<long> g_launch_block_limit{ 0 };     // 0: what HIP allows; smaller values are for tests of the splitting
 static_assert(kGeomBlock == kBlock, "the geometry header and the kernels agree on the block size");
 
@@ -119,6 +121,8 @@ Tuning current_tuning() {
     t.spin_ticks = g_phase_spin_ticks.load(std::memory_order_relaxed);
     t.fp16_impl = g_fp16_impl.load(std::memory_order_relaxed);
     t.realign = g_realign.load(std::memory_order_relaxed);
+    t.line_start = g_line_start.load(std::memory_order_relaxed);
+    t.wave_runs = g_wave_runs.load(std::memory_order_relaxed);
     return t;
 }
 
@@ -692,7 +696,10 @@ int mi_ccl_comp_batch_reduce(const void* in_buf, const size_t* offsets, size_t n
 
 namespace mi {
 static int launch_copy(const void* in, void* out, size_t bytes, bool nontemporal, hipStream_t stream) {
-    const LaneWork w = lane_work((uintptr_t)out, 1, bytes, 16);
+    // large copies start their vectors on a 128-byte line of the output (a line written in two parts costs more than
+    // one read in two parts)
+    const uint32_t boundary = bytes >= kLineStartBytes && g_line_start.load(std::memory_order_relaxed) ? kLineBytes : 16u;
+    const LaneWork w = lane_work((uintptr_t)out, 1, bytes, 16, boundary);
     const uint64_t limit = block_limit(), n = num_launches(w, kBlock, limit);
     for (uint64_t i = 0; i < n; i++) {
         const LaunchPiece p = launch_piece(w, kBlock, limit, i);
@@ -712,9 +719,11 @@ static int launch_copy(const void* in, void* out, size_t bytes, bool nontemporal
     return MI_CCL_SUCCESS;
 }
 
-// m >= 2 destinations; the vectors start where the first destination reaches a 16-byte boundary
+// m >= 2 destinations; the vectors start where the first destination reaches a 16-byte boundary (a 128-byte line when
+// the buffer is large)
 static int launch_broadcast(const void* in, void* const* dsts, int m, size_t bytes, hipStream_t stream) {
-    const BcastShape b = bcast_shape((uintptr_t)dsts[0], bytes, kBcastSect);
+    const uint32_t boundary = bytes >= kLineStartBytes && g_line_start.load(std::memory_order_relaxed) ? kLineBytes : 16u;
+    const BcastShape b = bcast_shape((uintptr_t)dsts[0], bytes, kBcastSect, boundary);
     const uint64_t limit = block_limit(), n = bcast_num_launches(b, m, limit);
     for (uint64_t i = 0; i < n; i++) {
         const BcastPiece p = bcast_piece(b, m, limit, i);
@@ -866,6 +875,14 @@ int mi_ccl_set_param(const char* name, long value) {
         g_realign.store((int)value);
         return MI_CCL_SUCCESS;
     }
+    if (!strcmp(name, "line_start") && (value == 0 || value == 1)) {
+        g_line_start.store((int)value);
+        return MI_CCL_SUCCESS;
+    }
+    if (!strcmp(name, "wave_runs") && value >= 0 && value <= 2) {
+        g_wave_runs.store((int)value);
+        return MI_CCL_SUCCESS;
+    }
     return MI_CCL_INVALID_ARGUMENTS;
 }
 
@@ -898,6 +915,10 @@ long mi_ccl_get_param(const char* name) {
         return g_realign.load();
     if (!strcmp(name, "realigned_launches"))
         return (long)g_realigned_launches;
+    if (!strcmp(name, "line_start"))
+        return g_line_start.load();
+    if (!strcmp(name, "wave_runs"))
+        return g_wave_runs.load();
     return -1;
 }
 

@@ -13,7 +13,7 @@
 
 namespace mi {
 
-constexpr int kFusionGroup = 192;                 // tensors per launch (pointer tables must fit the kernarg segment)
+constexpr int kFusionGroup = 256;                 // tensors per launch (two pointer tables must fit the 4 KiB of kernel arguments)
 constexpr int kFusionMaxPeers = 16;
 constexpr uint32_t kFusionChunk = 16384;          // bytes of one tensor per work item = kBlock lanes x 16 B x 4
 
@@ -21,8 +21,17 @@ struct FusionItem {
     uint32_t t;     // tensor index
     uint32_t c;     // chunk index inside the tensor
 };
+// Device addresses fit 48 bits; a table keeps them as 32 low and 16 high bits, 1.5 KiB for kFusionGroup of them.
 struct FusionPtrs {
-    const void* p[kFusionGroup];
+    uint32_t lo[kFusionGroup];
+    uint16_t hi[kFusionGroup];
+    bool set(size_t i, const void* p) {
+        const uint64_t v = (uint64_t)(uintptr_t)p;
+        lo[i] = (uint32_t)v;
+        hi[i] = (uint16_t)(v >> 32);
+        return (v >> 48) == 0;
+    }
+    __device__ __forceinline__ uint64_t get(uint32_t i) const { return ((uint64_t)hi[i] << 32) | lo[i]; }
 };
 struct PeerPtrs {
     const void* p[kFusionMaxPeers];
@@ -83,8 +92,8 @@ fusion_reduce_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers
         const uint64_t lo = (uint64_t)w.c * kFusionChunk;
         const uint64_t left = bytes[w.t] - lo;
         const uint32_t nb = left < kFusionChunk ? (uint32_t)left : kFusionChunk;
-        const unsigned char* a = (const unsigned char*)own.p[w.t - t0] + lo;
-        unsigned char* o = (unsigned char*)out.p[w.t - t0] + lo;
+        const unsigned char* a = (const unsigned char*)(uintptr_t)own.get(w.t - t0) + lo;
+        unsigned char* o = (unsigned char*)(uintptr_t)out.get(w.t - t0) + lo;
         const uint64_t poff = off[w.t] + lo;
         const uint32_t nelem = nb / ES;
         {
@@ -137,7 +146,7 @@ template <class TR, int OP, int NT>
 __global__ void __launch_bounds__(kPhaseBlock)
 fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, const uint64_t* off, const uint64_t* bytes,
                             const FusionItem* items, uint32_t nitems, uint32_t t0, PhaseSync* ps, int early_loads,
-                            int early_stores, long spin_ticks, uint32_t realign) {
+                            int early_stores, long spin_ticks, uint32_t realign, uint32_t wave_runs) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr uint32_t ES = sizeof(E);
@@ -161,7 +170,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
         // item -> tensor tables -> pointers is walked once, for all items at once, instead of once per item.
         uint64_t d_a = 0, d_o = 0, d_poff = 0;
         uint32_t d_nb = 0;      // 0: no item in this slot
-        uint32_t d_head = 0;    // elements before the item's first vector (bits 0-7); bits 8-9: fusion_beyond's answer
+        uint32_t d_head = 0;    // elements before the item's first vector (bits 0-7); bits 8-9: fusion_beyond's answer; bit 10: a buffer is off the 128-byte lines
         if (lane < (uint32_t)SLOTS) {
             const uint64_t it = p0 + (uint64_t)lane * gridDim.x + blockIdx.x;
             if (it < nitems) {
@@ -169,14 +178,18 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                 const uint64_t lo = (uint64_t)w.c * kFusionChunk;
                 const uint64_t left = bytes[w.t] - lo;
                 d_nb = left < kFusionChunk ? (uint32_t)left : kFusionChunk;
-                d_a = (uint64_t)(uintptr_t)own.p[w.t - t0] + lo;
-                d_o = (uint64_t)(uintptr_t)out.p[w.t - t0] + lo;
+                d_a = own.get(w.t - t0) + lo;
+                d_o = out.get(w.t - t0) + lo;
                 d_poff = off[w.t] + lo;
                 d_head = fusion_head<ES>((const void*)(uintptr_t)d_o);
                 const uint32_t ne = d_nb / ES;
                 if (d_head > ne) d_head = ne;
                 d_head |= fusion_beyond<ES>((const void*)(uintptr_t)(d_a + d_head * ES), peers, NP, d_poff + d_head * ES,
                                             (ne - d_head) / TR::VEC, left - d_nb, realign) << 8;
+                const uint32_t hbytes = (d_head & 0xffu) * ES;
+                uint32_t off_lines = (uint32_t)(d_a + hbytes) | (uint32_t)(d_o + hbytes);
+                for (int j = 0; j < NP; j++) off_lines |= (uint32_t)((uintptr_t)peers.p[j] + d_poff + hbytes);
+                if (off_lines & (kLineBytes - 1)) d_head |= 1u << 10;
             }
         }
         // The block reports its arrival at the barriers a little before it is done (see phase_arrive): in front of the
@@ -200,12 +213,26 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
             {
                 const uint32_t hb = __shfl(d_head, k, 64);
                 const uint32_t head = hb & 0xffu, beyond = (hb >> 8) & 1u;
-                const uint32_t nvec = (nelem - head) / TR::VEC - (hb >> 9), tail = nelem - head - nvec * TR::VEC;
+                const uint32_t nvec = (nelem - head) / TR::VEC - ((hb >> 9) & 1u), tail = nelem - head - nvec * TR::VEC;
                 const unsigned char* s[NT];
                 s[0] = a + head * ES;
 #pragma unroll
                 for (int j = 0; j < NP; j++) s[j + 1] = (const unsigned char*)peers.p[j] + poff + head * ES;
-                const uint64_t idx[2] = { tid, tid + (uint32_t)kPhaseBlock };
+                // the item's two vectors of a lane: half an item apart, or -- when a buffer of the item is off the
+                // 128-byte lines -- 64 vectors apart, so that a wave covers 2 KiB in one run (fewer shared lines)
+                const bool runs = wave_runs == 2 || (wave_runs == 1 && (hb >> 10));
+                const uint32_t i0 = runs ? (tid & ~63u) * 2u + lane : tid;
+                const uint64_t idx[2] = { i0, i0 + (runs ? 64u : (uint32_t)kPhaseBlock) };
+                // The item's elements before its first and after its last vector (one per lane): their loads go out
+                // in front of the vectors', so that the lanes that have one wait once per item, not twice.
+                const bool edge = tid < head + tail;
+                const uint32_t ei = (tid < head) ? tid : head + nvec * TR::VEC + (tid - head);
+                E ev[NT];
+                if (edge) {
+                    ev[0] = ld_elem<E>(a, ei);
+#pragma unroll
+                    for (int j = 0; j < NP; j++) ev[j + 1] = ld_elem<E>((const unsigned char*)peers.p[j] + poff, ei);
+                }
                 u32x4 res[2];
                 if (nvec >= 2u * kPhaseBlock)       // a whole item: no lane is out of range (the same answer for the whole block)
                     reduce_group<TR, OP, NT, 2, true>(s, idx, nvec, nvec + beyond, res);
@@ -225,13 +252,11 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                     }
 #undef MI_RS_PUT
                 }
-                if (tid < head + tail) {
-                    const uint32_t i = (tid < head) ? tid : head + nvec * TR::VEC + (tid - head);
-                    typename TR::acc_t r = TR::init(ld_elem<E>(a, i));
+                if (edge) {
+                    typename TR::acc_t r = TR::init(ev[0]);
 #pragma unroll
-                    for (int j = 0; j < NP; j++)
-                        r = TR::template step<OP>(ld_elem<E>((const unsigned char*)peers.p[j] + poff, i), r);
-                    st_elem<E>(o, i, TR::finish(r));
+                    for (int j = 0; j < NP; j++) r = TR::template step<OP>(ev[j + 1], r);
+                    st_elem<E>(o, ei, TR::finish(r));
                 }
             }
         }
@@ -254,7 +279,7 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                 const uint32_t nelem = nb / ES;
                 const uint32_t hb = __shfl(d_head, k, 64);
                 const uint32_t head = hb & 0xffu;
-                const uint32_t nvec = (nelem - head) / TR::VEC - (hb >> 9);
+                const uint32_t nvec = (nelem - head) / TR::VEC - ((hb >> 9) & 1u);
                 u32x4_u* d = (u32x4_u*)(o + head * ES);
                 u32x4 v0 = { 0, 0, 0, 0 }, v1 = v0;
                 if (k < S) {
@@ -270,8 +295,11 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
                     }
 #undef MI_RS_GET
                 }
-                if (tid < nvec) st_loose(d + tid, v0);
-                if (tid + kPhaseBlock < nvec) st_loose(d + tid + kPhaseBlock, v1);
+                const bool runs = wave_runs == 2 || (wave_runs == 1 && (hb >> 10));
+                const uint32_t i0 = runs ? (tid & ~63u) * 2u + lane : tid;
+                const uint32_t i1 = i0 + (runs ? 64u : (uint32_t)kPhaseBlock);
+                if (i0 < nvec) st_loose(d + i0, v0);
+                if (i1 < nvec) st_loose(d + i1, v1);
             }
         }
         if (more) {
@@ -289,7 +317,8 @@ inline hipError_t launch_fusion_phased(const FusionLaunchArgs& a, const FusionPt
     g_last_kernel = "fusion_reduce_phased_kernel";
     hipLaunchKernelGGL((fusion_reduce_phased_kernel<TR, OP, NT>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, own, out, pp,
                        a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0, a.tune.sync,
-                       a.tune.early_loads, phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks, (uint32_t)a.tune.realign);
+                       a.tune.early_loads, phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks, (uint32_t)a.tune.realign,
+                       (uint32_t)a.tune.wave_runs);
     return hipGetLastError();
 }
 
@@ -302,11 +331,9 @@ inline hipError_t launch_fusion_op(const FusionLaunchArgs& a) {
         const uint64_t i0 = a.item_begin[t0], i1 = a.item_begin[t1];
         if (i1 == i0)
             continue;
-        FusionPtrs own, out;
-        for (size_t t = t0; t < t1; t++) {
-            own.p[t - t0] = a.own[t];
-            out.p[t - t0] = a.out[t];
-        }
+        FusionPtrs own = {}, out = {};
+        for (size_t t = t0; t < t1; t++)
+            if (!own.set(t - t0, a.own[t]) || !out.set(t - t0, a.out[t])) return hipErrorInvalidValue;   // not a device address
         hipError_t e = hipSuccess;
         // large groups with three or more peers (from 320 MB of traffic by default, 480 MB with three peers): separate
         // reads from writes in time (at most 16 KiB of padding per item is over-counted).  With one or two peers the

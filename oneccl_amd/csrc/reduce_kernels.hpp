@@ -58,6 +58,8 @@ struct Tuning {
     long spin_ticks;         // phased kernels: longest wait at one barrier, in 100 MHz ticks, before a block goes on alone
     int fp16_impl;           // which CPU implementation's float16 results to reproduce: 2, 3 (through fp32) or 4 (native)
     int realign;             // 1: inputs off a 4-byte boundary are read on that boundary and realigned in registers
+    int line_start;          // 1: large calls start their vectors on a 128-byte line of the buffers that matter most
+    int wave_runs;           // phased kernels: a wave's vectors of a group lie next to each other; 0 never, 1 when a buffer is off the lines, 2 always
 };
 
 // Name of the kernel template the calling thread's most recent entry-point call launched (diagnostics and
@@ -521,7 +523,11 @@ __device__ __forceinline__ u32x4 vec_finish(const Accs<TR>& a) {
 // peer's chunk at an odd offset -- still move as vectors.  The host starts the vectors on the 16-byte boundary of the
 // buffer that makes the loose accesses cheapest (vector_head).
 typedef u32x4 u32x4_u __attribute__((aligned(1)));
+#ifdef MI_EXP_LD_PLAIN
+__device__ __forceinline__ u32x4 ld_loose(const u32x4_u* p) { return *p; }
+#else
 __device__ __forceinline__ u32x4 ld_loose(const u32x4_u* p) { return __builtin_nontemporal_load(p); }
+#endif
 __device__ __forceinline__ void st_loose(u32x4_u* p, u32x4 v) { __builtin_nontemporal_store(v, p); }
 // The same store with device scope on top (sc1 nt).  A 1 : 1 copy gains 2-6 % from it (6.65 against 6.50 TB/s at
 // 512 MiB, 6.19 against 5.85 at 64 MiB); the reduce kernels, the converters, pack / unpack and the broadcast measure
@@ -644,7 +650,7 @@ __device__ __forceinline__ void load_vectors(const unsigned char* base, const ui
 }
 
 // The count % VEC elements after the last full vector and the elements before the first aligned one:
-// at most 2*(VEC-1) <= 30 elements, one per lane of the first wave of block 0.
+// at most 127 + 2 * VEC - 1 <= 158 elements (the head may reach to a 128-byte line), one per lane of block 0.
 template <class TR, int OP, class SRC>
 __device__ __forceinline__ void reduce_edges(const SRC& src, int n, void* dst, uint32_t head, uint64_t nvec,
                                              uint32_t tail) {
@@ -950,7 +956,8 @@ inline int phase_early_stores(const Tuning& t, int n_dsts) {
 template <class TR, int OP>
 __global__ void __launch_bounds__(kPhaseBlock)
 reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uint64_t nvec, uint32_t tail,
-                           PhaseSync* ps, int early_loads, int early_stores, long spin_ticks, uint32_t beyond) {
+                           PhaseSync* ps, int early_loads, int early_stores, long spin_ticks, uint32_t beyond,
+                           uint32_t wave_runs) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     const uint64_t nload = nvec + beyond;               // vector nvec may be read when beyond = 1 (load_vectors)
@@ -962,7 +969,14 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
     const uint64_t gthreads = (uint64_t)gridDim.x * kPhaseBlock;
     const uint64_t gtid = (uint64_t)blockIdx.x * kPhaseBlock + threadIdx.x;
     const uint64_t per_phase = gthreads * (uint64_t)(G * (RG + LG));
-    auto pos = [&](uint64_t p0, int u) -> uint64_t { return p0 + (uint64_t)u * gthreads + gtid; };   // slot u of this lane
+    // Slot u of this lane.  The G slots of a group lie one slab (gthreads vectors) apart: at every step the chip reads
+    // G compact windows.  With wave_runs they lie 64 vectors apart instead, so that a wave covers G KiB in one run and a
+    // block 32 KiB: buffers that are off the 128-byte lines then share a line between two waves a quarter as often.
+    const uint64_t lane_base = wave_runs ? (gtid & ~(uint64_t)63) * G + (threadIdx.x & 63u) : gtid;
+    const uint64_t slot_step = wave_runs ? 64u : gthreads;
+    auto pos = [&](uint64_t p0, int u) -> uint64_t {
+        return p0 + (uint64_t)(u / G) * (G * gthreads) + lane_base + (uint64_t)(u % G) * slot_step;
+    };
     bool give_up = false;
     unsigned gen = 0;
     if (threadIdx.x == 0) gen = phase_generation(ps);
@@ -1105,15 +1119,25 @@ inline bool wants_phased(const LaunchArgs& a, uint64_t nvec, int reg_groups) {
 }
 
 // Elements before the first vector: the vectors start on the 16-byte boundary that makes the loose accesses of the
-// buffers that disagree with it cheapest (vector_grid).  No head when that boundary is not a multiple of the element
-// size.
+// buffers that disagree with it cheapest (vector_grid) and, for large calls, on the 128-byte line that suits the
+// buffers on that boundary best (vector_start).  No head when that boundary is not a multiple of the element size.
+constexpr size_t kLineStartBytes = 1u << 20;
 template <class E>
 inline uint64_t vector_head(const LaunchArgs& a) {
-    unsigned in_mis[kMaxSrcs], out_mis[kMaxDsts];
-    for (int j = 0; j < a.n; j++) in_mis[j] = (unsigned)((uintptr_t)a.srcs[j] & 15u);
-    for (int k = 0; k < a.m; k++) out_mis[k] = (unsigned)((uintptr_t)(a.dsts ? a.dsts[k] : a.dst) & 15u);
+    unsigned in_mis[kMaxSrcs], out_mis[kMaxDsts], in_line[kMaxSrcs], out_line[kMaxDsts];
+    for (int j = 0; j < a.n; j++) {
+        in_line[j] = (unsigned)((uintptr_t)a.srcs[j] & (kLineBytes - 1));
+        in_mis[j] = in_line[j] & 15u;
+    }
+    for (int k = 0; k < a.m; k++) {
+        out_line[k] = (unsigned)((uintptr_t)(a.dsts ? a.dsts[k] : a.dst) & (kLineBytes - 1));
+        out_mis[k] = out_line[k] & 15u;
+    }
     const unsigned mis = vector_grid(in_mis, a.n, out_mis, a.m, sizeof(E) < 4 && a.tune.realign);
-    return (mis % sizeof(E)) == 0 ? ((16u - mis) & 15u) / sizeof(E) : 0;
+    if (mis % sizeof(E)) return 0;
+    // below kLineStartBytes per buffer a call is latency-bound and the head stays as short as it can be
+    const bool lines = a.tune.line_start && a.count * sizeof(E) >= kLineStartBytes;
+    return vector_start(in_line, a.n, out_line, a.m, mis, lines) / sizeof(E);
 }
 
 // How the elements of a call are divided: `head` elements, `nvec` vectors, `tail` elements.  When an input's vectors
@@ -1150,10 +1174,15 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
     g_realigned_launches += v.beyond;
     if (wants_phased(a, v.nvec, MultiPhaseRegs<TR>::groups)) {
         int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
+        // does any buffer's first vector start off a 128-byte line?
+        uint32_t off_lines = 0;
+        for (int j = 0; j < a.n; j++) off_lines |= (uint32_t)((uintptr_t)s.p[j] + v.head * sizeof(E)) & (kLineBytes - 1);
+        for (int k = 0; k < a.m; k++) off_lines |= (uint32_t)((uintptr_t)d.p[k] + v.head * sizeof(E)) & (kLineBytes - 1);
+        const uint32_t wave_runs = a.tune.wave_runs == 2 || (a.tune.wave_runs == 1 && off_lines);
         g_last_kernel = "reduce_multi_phased_kernel";
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
                            a.m, v.head, v.nvec, v.tail, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune, a.m),
-                           a.tune.spin_ticks, v.beyond);
+                           a.tune.spin_ticks, v.beyond, wave_runs);
         return hipGetLastError();
     }
     constexpr int UNROLL = 4;

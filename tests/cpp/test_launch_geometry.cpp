@@ -178,6 +178,40 @@ int main() {
             EXPECT(grid_price(out[0], in, n, out, m, ra) > best || g == out[0]);    // the first destination's among equals
         }
     }
+    // which 128-byte line the vectors start on: the measured cases, then every choice against a brute-force minimum
+    {
+        const unsigned al[8] = { 0 }, all16[8] = { 16, 16, 16, 16, 16, 16, 16, 16 }, peers16[8] = { 0, 16, 16, 16, 16, 16, 16, 16 };
+        const unsigned all2[8] = { 2, 2, 2, 2, 2, 2, 2, 2 }, own64[8] = { 64, 0, 0, 0, 0, 0, 0, 0 }, own16[8] = { 16, 0, 0, 0, 0, 0, 0, 0 };
+        const unsigned o0[1] = { 0 }, o16[1] = { 16 }, o2[1] = { 2 }, o64[1] = { 64 };
+        EXPECT(vector_start(al, 8, o0, 1, 0, true) == 0);
+        EXPECT(vector_start(all16, 8, o16, 1, 0, true) == 112);         // everything 16 bytes off: 112 bytes of head put all of it on lines
+        EXPECT(vector_start(all16, 8, o16, 1, 0, false) == 0);          // ... not asked for: the 16-byte boundary is enough
+        EXPECT(vector_start(all2, 8, o2, 1, 2, true) == 126 && vector_start(all2, 8, o2, 1, 2, false) == 14);
+        EXPECT(vector_start(peers16, 8, o0, 1, 0, true) == 0);          // the output's line is worth more than seven inputs'
+        EXPECT(vector_start(al, 8, o16, 1, 0, true) == 112);            // the output alone off: the head follows it
+        EXPECT(vector_start(own16, 8, o16, 1, 0, true) == 112);
+        EXPECT(vector_start(own64, 8, o64, 1, 0, true) == 0);           // whole 64 bytes off: seven inputs outweigh it
+        EXPECT(vector_start(own64, 2, o64, 1, 0, true) == 64);
+        uint64_t x = 1234567891234567ull;
+        for (int it = 0; it < 20000; it++) {
+            unsigned in[8], out[3], in16[8], out16[3];
+            x ^= x << 13; x ^= x >> 7; x ^= x << 17;
+            const int n = 1 + (int)(x % 8), m = 1 + (int)((x >> 8) % 3);
+            const unsigned gran = 1u << ((x >> 16) % 4);
+            uint64_t y = x * 0x9e3779b97f4a7c15ull;
+            for (int j = 0; j < n; j++) { in[j] = (unsigned)((y >> (7 * j)) & 127u) / gran * gran; in16[j] = in[j] & 15u; }
+            for (int k = 0; k < m; k++) { out[k] = (unsigned)((x >> (40 + 7 * k)) & 127u) / gran * gran; out16[k] = out[k] & 15u; }
+            const unsigned mis = vector_grid(in16, n, out16, m, false);
+            if (mis % gran) continue;
+            const unsigned h0 = (16u - mis) & 15u, s = vector_start(in, n, out, m, mis, true);
+            EXPECT(s >= h0 && s < 128 && (s - h0) % 16 == 0 && s % gran == 0);
+            EXPECT(vector_start(in, n, out, m, mis, false) == h0);
+            unsigned best = ~0u;
+            for (unsigned e = 0; e < 128; e += 16) { const unsigned p = line_price(h0 + e, in, n, out, m); if (p < best) best = p; }
+            EXPECT(line_price(s, in, n, out, m) == best);
+            EXPECT(line_price(h0, in, n, out, m) > best || s == h0);        // among equals the head stays as short as it can be
+        }
+    }
     // whether the phased form pays: the measured crossovers (one phase holds 88 MiB of results on 256 CUs)
     {
         const uint64_t per = 256ull * 512 * 44;

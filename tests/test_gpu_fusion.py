@@ -38,7 +38,7 @@ def test_fusion_offsets_match_oracle(comp):
 def test_pack_reduce_unpack_and_fused(comp, align, dtype):
     import torch
     rng = np.random.default_rng(42 + align + dtype)
-    k = 230                       # more than one launch group of tensors
+    k = 300                       # more than one launch group of tensors (256 per launch)
     counts = log_uniform_counts(rng, k, 1, 40000)
     counts[5] = 0 if align == 256 else 1
     np_t = O.NP_STORAGE[dtype]

@@ -66,11 +66,11 @@ def _case(comp, rng, counts, dtype, op, n_peers, align, lp, variant, check_memor
 
 @pytest.mark.parametrize("variant", [0, 8])
 def test_static_entry_point_equals_plan_entry_point_twice_in_a_row(comp, variant):
-    """First a larger group (more than one launch group of 192 tensors, odd sizes, an empty tensor), then a smaller
+    """First a larger group (more than one launch group of 256 tensors, odd sizes, an empty tensor), then a smaller
     one with another layout, dtype and peer count; variant 8 forces the phased kernels."""
     rng = np.random.default_rng(2026)
     _case(comp, rng, [3, 70_000], O.INT32, O.SUM, 1, 4, comp.LP_PAIRWISE, variant, check_memory=False)   # first use on this device
-    big = [int(c) for c in np.exp(rng.uniform(np.log(3), np.log(300_000), 230))]
+    big = [int(c) for c in np.exp(rng.uniform(np.log(3), np.log(300_000), 300))]
     big[7] = 0
     big[100] = 16384 * 3
     _case(comp, rng, big, O.BFLOAT16, O.SUM, 7, 256, comp.LP_KEEP_PRECISION, variant)
