@@ -11,8 +11,9 @@
          mi_ccl_comp_reduce_batch (one launch)
   types  every datatype x op at 512 MiB per buffer, 8 and 4 inputs
   align  buffers that disagree modulo 16 bytes: 8-input bf16 sum at 64 MiB per buffer with every input at its own
-         alignment, and with only the output off; the reference's tight fusion layout (alignment 1) of 400 odd-sized
-         tensors: pack, unpack and the fused reduce
+         alignment, and with only the output off; buffers on the 16-byte boundary but off the 128-byte lines (all of
+         them, the output alone, the peers); the reference's tight fusion layout (alignment 1) of 400 even- and
+         odd-sized tensors: pack, unpack and the fused reduce
   write  a reduce stored to several buffers, and one buffer written to several (the all-gather write side), at 64 MiB
          and 1 GiB per buffer
   copy   ccl_comp_copy at 64 MiB, 512 MiB and 3 GiB, and the bf16 <-> fp32 array converters at 2^28 elements
@@ -284,7 +285,9 @@ def main():
         na = 33_554_432
         sets = [[torch.empty(na + 64, dtype=torch.bfloat16, device="cuda").normal_(0, 1) for _ in range(9)] for _ in range(6)]
         for label, shifts in (("all aligned", [0] * 9), ("every input at its own alignment", [1, 2, 3, 4, 5, 6, 7, 0, 0]),
-                              ("only the output off by 6 bytes", [0] * 8 + [3])):
+                              ("only the output off by 6 bytes", [0] * 8 + [3]),
+                              ("every buffer 16 bytes past a 128-byte line", [8] * 9), ("every buffer 2 bytes past a line", [1] * 9),
+                              ("only the output 16 bytes past a line", [0] * 8 + [8]), ("the peers 16 bytes past a line", [0] + [8] * 7 + [0])):
             ptrs = [[t.data_ptr() + 2 * sh for t, sh in zip(s_, shifts)] for s_ in sets]
 
             def once():
