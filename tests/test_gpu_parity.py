@@ -591,7 +591,8 @@ def test_buffers_that_disagree_modulo_16_bytes(comp, variant, dtype, op, n, m):
 def test_randomised_calls_against_oracle(comp):
     """400 seeded random calls (MI_CCL_FUZZ_CASES / MI_CCL_FUZZ_SEED change that): dtype, op, input count (1..12),
     1..3 destinations, element count, 16-bit mode, per-buffer element shifts (shared or mixed misalignment), output
-    aliasing an input or not, kernel choice forced or automatic."""
+    aliasing an input or not, kernel choice forced or automatic, the 128-byte line rule and the wave-run layout on or
+    off."""
     import os
     import torch
     rng = np.random.default_rng(int(os.environ.get("MI_CCL_FUZZ_SEED", "20260101")))
@@ -599,16 +600,17 @@ def test_randomised_calls_against_oracle(comp):
         dtype = int(rng.integers(0, 12))
         op = int(rng.integers(0, 4))
         n = int(rng.integers(1, 13))
-        count = int(rng.choice([1, 2, 3, 15, 16, 17, 255, 1000, 4097, 65535, 200_003]))
+        count = int(rng.choice([1, 2, 3, 15, 16, 17, 255, 1000, 4097, 65535, 200_003, 1_100_003]))     # the last: heads up to a 128-byte line
         esz = O.DTYPE_SIZE[dtype]
         np_t = O.NP_STORAGE[dtype]
         lp, impl, keep, quirk = lp_variants(dtype)[int(rng.integers(0, len(lp_variants(dtype))))]
         kind = "bits" if dtype in (O.FLOAT16, O.BFLOAT16) and rng.random() < 0.5 else "config"
         srcs = make_inputs(rng, dtype, count, op, n, kind)
         same_shift = rng.random() < 0.6
-        base_shift = int(rng.integers(0, 16 // esz + 1))
-        shifts = [base_shift if same_shift else int(rng.integers(0, 16 // esz + 1)) for _ in range(n + 1)]
-        pad = 32
+        span = (128 if count > 1_000_000 else 16) // esz
+        base_shift = int(rng.integers(0, span + 1))
+        shifts = [base_shift if same_shift else int(rng.integers(0, span + 1)) for _ in range(n + 1)]
+        pad = 160
         holders, ptrs = [], []
         for s_, sh in zip(srcs, shifts):
             h = np.zeros(count + 2 * pad, np_t)
@@ -624,9 +626,12 @@ def test_randomised_calls_against_oracle(comp):
         m = int(rng.choice([1, 1, 2, 3]))
         extra = []       # further destinations: (holder, first element), with the output's shift or one of their own
         for _ in range(m - 1):
-            sh = shifts[alias if alias >= 0 else n] if same_shift else int(rng.integers(0, 16 // esz + 1))
+            sh = shifts[alias if alias >= 0 else n] if same_shift else int(rng.integers(0, span + 1))
             extra.append((to_dev(np.zeros(count + 2 * pad, np_t)), pad + sh))
+        line_start, wave_runs = int(rng.integers(0, 2)), int(rng.integers(0, 3))
         comp.set_param("variant", variant)
+        comp.set_param("line_start", line_start)
+        comp.set_param("wave_runs", wave_runs)
         try:
             out_ptr = out_holder.data_ptr() + out_lo * esz
             if m == 1:
@@ -637,10 +642,12 @@ def test_randomised_calls_against_oracle(comp):
             torch.cuda.synchronize()
         finally:
             comp.set_param("variant", 0)
+            comp.set_param("line_start", 1)
+            comp.set_param("wave_runs", 1)
         want = O.reduce_n(srcs, dtype, op, keep=keep, quirk_tail=quirk, bf16_impl=impl)
         got = to_host(out_holder, np_t)
         what = (f"case {case}: dtype={O.DTYPE_NAMES[dtype]} op={O.OP_NAMES[op]} n={n} m={m} count={count} lp={lp} impl={impl} "
-                f"shifts={shifts} alias={alias} variant={variant} kind={kind}")
+                f"shifts={shifts} alias={alias} variant={variant} line_start={line_start} wave_runs={wave_runs} kind={kind}")
         assert_same(got[out_lo:out_lo + count], want, dtype, what, srcs, op, keep=keep, bf16_impl=impl)
         for h, lo in extra:
             g2 = to_host(h, np_t)
