@@ -264,8 +264,8 @@ const char* mi_ccl_last_kernel(void);
  * line of the buffers that matter most -- the outputs before the inputs -- so up to 127 bytes at the front are
  * handled element by element; buffers that share an offset from the lines then run like aligned ones, +6 %) and
  * "wave_runs" (phased kernels: a wave's vectors of one step lie next to each other instead of a block apart, which
- * halves to quarters the lines two waves share; 0 never, 1 = default, when a buffer is off the 128-byte lines, 2
- * always).  Neither changes a result.
+ * halves to quarters the lines two waves share; 0 never, 1 = default, when a buffer is off the 128-byte lines and
+ * there is one destination, 2 always).  Neither changes a result.
  * Returns invalid_arguments for an unknown name or out-of-range value. */
 int mi_ccl_set_param(const char* name, long value);
 long mi_ccl_get_param(const char* name);

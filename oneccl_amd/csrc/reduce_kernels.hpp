@@ -1178,7 +1178,9 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
         uint32_t off_lines = 0;
         for (int j = 0; j < a.n; j++) off_lines |= (uint32_t)((uintptr_t)s.p[j] + v.head * sizeof(E)) & (kLineBytes - 1);
         for (int k = 0; k < a.m; k++) off_lines |= (uint32_t)((uintptr_t)d.p[k] + v.head * sizeof(E)) & (kLineBytes - 1);
-        const uint32_t wave_runs = a.tune.wave_runs == 2 || (a.tune.wave_runs == 1 && off_lines);
+        // (with several destinations the write phase, which wants the chip's stores in one compact window, loses more
+        // to the runs than the reads gain: 8 -> 8 at 1 GiB 6.28 against 6.46 TB/s)
+        const uint32_t wave_runs = a.tune.wave_runs == 2 || (a.tune.wave_runs == 1 && off_lines && a.m == 1);
         g_last_kernel = "reduce_multi_phased_kernel";
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
                            a.m, v.head, v.nvec, v.tail, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune, a.m),
