@@ -248,7 +248,7 @@ const char* mi_ccl_last_kernel(void);
  * "phased_min_bytes" (scales the sizes from which the phased kernels are used; default 160 MB),
  * "phase_early_loads" / "phase_early_stores" (phased kernels: how many 16-byte loads / stores per lane a block still
  * has to issue when it reports the end of its read / write phase to the chip-wide barrier, which hides the barrier's
- * latency; defaults 12 and -1 = chosen per element type, 4 or 16, and 16 with several destinations; 0 = report
+ * latency; defaults 12 and -1 = 16, or 20 with several destinations while the write phase is paced; 0 = report
  * when the whole block is done and its stores are acknowledged; timing only, results do not
  * depend on them), "phase_spin_ticks" (phased kernels: the longest a block waits at one barrier, in 100 MHz ticks,
  * before it goes on alone and stops waiting for the rest of the launch; default 20000 = 200 us; 0 = never wait, which
@@ -263,6 +263,11 @@ const char* mi_ccl_last_kernel(void);
  * (0/1, default 1: a reduce, copy or broadcast of 1 MiB or more per buffer starts its 16-byte vectors on a 128-byte
  * line of the buffers that matter most -- the outputs before the inputs -- so up to 127 bytes at the front are
  * handled element by element; buffers that share an offset from the lines then run like aligned ones, +6 %) and
+ * "phase_write_pace" (phased reduce with two or more destinations: the rate in GB/s at which the device clock lets
+ * the write phase's stores out, which keeps the blocks of the chip in step and the addresses written at any moment in
+ * one compact window; default 7400, 0 = unpaced, otherwise 100 to 100000; 8 inputs stored to 8 buffers of 1 GiB run at 6.95 TB/s paced and 6.4
+ * unpaced; a block that is behind the schedule is never held, so a rate above what HBM takes only switches the
+ * pacing off), "wall_clock_khz" (read only: the rate of that clock),
  * "wave_runs" (phased kernels: a wave's vectors of one step lie next to each other instead of a block apart, which
  * halves to quarters the lines two waves share; 0 never, 1 = default, when a buffer is off the 128-byte lines and
  * there is one destination, 2 always).  Neither changes a result.

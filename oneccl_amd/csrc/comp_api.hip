@@ -57,6 +57,7 @@ static std::atomic<int> g_fp16_impl{ MI_CCL_FP16_AVX512F };
 static std::atomic<int> g_realign{ 1 };
 static std::atomic<int> g_line_start{ 1 };
 static std::atomic<int> g_wave_runs{ 1 };
+static std::atomic<int> g_write_pace{ 7400 };
 static std::atomic<long> g_launch_block_limit{ 0 };     // 0: what HIP allows; smaller values are for tests of the splitting
 static_assert(kGeomBlock == kBlock, "the geometry header and the kernels agree on the block size");
 
@@ -107,6 +108,20 @@ static int num_cus() {
     return v;
 }
 
+static std::atomic<int> g_wall_khz[64];
+static int wall_khz() {         // the rate of wall_clock64(), which paces the write phase of the phased reduce
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        return 100000;
+    int v = g_wall_khz[dev].load(std::memory_order_relaxed);
+    if (v == 0) {
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeWallClockRate, dev) != hipSuccess || v <= 0)
+            v = 100000;
+        g_wall_khz[dev].store(v, std::memory_order_relaxed);
+    }
+    return v;
+}
+
 Tuning current_tuning() {
     Tuning t;
     t.waves_per_cu = g_waves_per_cu.load(std::memory_order_relaxed);
@@ -123,6 +138,8 @@ Tuning current_tuning() {
     t.realign = g_realign.load(std::memory_order_relaxed);
     t.line_start = g_line_start.load(std::memory_order_relaxed);
     t.wave_runs = g_wave_runs.load(std::memory_order_relaxed);
+    t.write_pace = g_write_pace.load(std::memory_order_relaxed);
+    t.wall_khz = wall_khz();
     return t;
 }
 
@@ -879,6 +896,10 @@ int mi_ccl_set_param(const char* name, long value) {
         g_line_start.store((int)value);
         return MI_CCL_SUCCESS;
     }
+    if (!strcmp(name, "phase_write_pace") && (value == 0 || (value >= 100 && value <= 100000))) {
+        g_write_pace.store((int)value);
+        return MI_CCL_SUCCESS;
+    }
     if (!strcmp(name, "wave_runs") && value >= 0 && value <= 2) {
         g_wave_runs.store((int)value);
         return MI_CCL_SUCCESS;
@@ -919,6 +940,10 @@ long mi_ccl_get_param(const char* name) {
         return g_line_start.load();
     if (!strcmp(name, "wave_runs"))
         return g_wave_runs.load();
+    if (!strcmp(name, "phase_write_pace"))
+        return g_write_pace.load();
+    if (!strcmp(name, "wall_clock_khz"))
+        return wall_khz();
     return -1;
 }
 

@@ -60,6 +60,8 @@ struct Tuning {
     int realign;             // 1: inputs off a 4-byte boundary are read on that boundary and realigned in registers
     int line_start;          // 1: large calls start their vectors on a 128-byte line of the buffers that matter most
     int wave_runs;           // phased kernels: a wave's vectors of a group lie next to each other; 0 never, 1 when a buffer is off the lines, 2 always
+    int write_pace;          // phased reduce with several destinations: the rate, in GB/s, at which the clock lets the write phase's stores out (0: unpaced)
+    int wall_khz;            // what wall_clock64() counts, in kHz
 };
 
 // Name of the kernel template the calling thread's most recent entry-point call launched (diagnostics and
@@ -926,27 +928,18 @@ struct MultiPhaseRegs {
 };
 
 // Stores per lane still to issue when a block reports the end of its write phase (Tuning::early_stores < 0 asks for
-// this).  Every plain type measures 0.7-1 % faster with 16 than with 4 (8 x 1 GiB and 4 x 1 GiB); the two bfloat16
-// families, whose lanes spend longer between their loads, are within 0.4 % from 4 to 20 and best at 4.
-template <class TR>
-struct PhaseEarlyStores {
-    static constexpr int value = 16;
-};
-template <bool RNE, bool VEC_SEM>
-struct PhaseEarlyStores<Bf16PairwiseTraits<RNE, VEC_SEM>> {
-    static constexpr int value = 4;
-};
-template <bool RNE>
-struct PhaseEarlyStores<Bf16KeepTraits<RNE>> {
-    static constexpr int value = 4;
-};
+// this).  Measured at 2 GB per buffer, 16 against 4: fp32 +1.2 % with 8 inputs, +1.6 % with 4, +2.7 % with 2; the two
+// bfloat16 families +0.1-0.3 %, +0.4-0.8 % and +1.5-1.9 %; 20 is within 0.3 % of 16 either way.
+constexpr int kPhaseEarlyStores = 16;
 // With several destinations the block's waves meet before each of them (see the write phase below), so the report
 // that goes out 16 stores before the end of the last destination speaks for the whole block; without that meeting an
 // early report with three or more destinations let the next reads start under far too many outstanding writes (8 -> 8
-// at 1 GiB: 5.78 TB/s with 4 stores early against 6.25 with a strict report, 6.45 with the meeting and 16 early).
+// at 1 GiB: 5.78 TB/s with 4 stores early against 6.25 with a strict report, 6.45 with the meeting and 16 early).  When
+// the clock paces the write phase (Tuning::write_pace) the last destination's 20 LDS-staged stores all come after the
+// report: 6.98 against 6.94 with 16.
 template <class TR>
 inline int phase_early_stores(const Tuning& t, int n_dsts) {
-    const int v = t.early_stores >= 0 ? t.early_stores : n_dsts >= 2 ? 16 : PhaseEarlyStores<TR>::value;
+    const int v = t.early_stores >= 0 ? t.early_stores : n_dsts >= 2 ? (t.write_pace > 0 ? kPhaseU : 16) : kPhaseEarlyStores;
     return v < kPhaseU ? v : kPhaseU;
 }
 
@@ -957,7 +950,7 @@ template <class TR, int OP>
 __global__ void __launch_bounds__(kPhaseBlock)
 reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uint64_t nvec, uint32_t tail,
                            PhaseSync* ps, int early_loads, int early_stores, long spin_ticks, uint32_t beyond,
-                           uint32_t wave_runs) {
+                           uint32_t wave_runs, uint32_t write_pace16) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     const uint64_t nload = nvec + beyond;               // vector nvec may be read when beyond = 1 (load_vectors)
@@ -1019,6 +1012,21 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
         phase_wait(ps, ++gen, give_up, spin_ticks);
         const bool more = p0 + per_phase < nvec;
         const int arrive_u = more ? kPhaseU - early_stores : -1;    // kPhaseU: after the last store
+        // With several destinations the write phase is hundreds of stores per lane long, the blocks drift apart, and the
+        // chip no longer writes one compact window of addresses at a time: HBM then takes the writes at 5.9 TB/s
+        // instead of the 6.8 of a write-only stream.  So the clock lets the stores out: group i of four stores (8 MiB
+        // over the chip) not before the phase's start + i * write_pace16 / 16 ticks, a little faster than HBM takes them.
+        // Every block reads the same clock, so the blocks stay within a fraction of a group of each other without
+        // exchanging a word; a block that is behind the schedule is never held.  8 -> 8 at 1 GiB: 6.95 against 6.40
+        // TB/s, 4 -> 4: 6.90 against 6.35, 2 -> 2: 6.63 against 6.30.  With one destination (44 stores per lane) there is
+        // nothing to gain: 7.04 against 7.10.
+        uint64_t pace_next16 = write_pace16 ? (uint64_t)wall_clock64() << 4 : 0;
+        auto paced = [&](int u) {       // u: slot within the phase; groups that lie behind the end of the data take no time
+            if (write_pace16 && (u & 3) == 0 && p0 + (uint64_t)u * gthreads < nvec) {
+                while (((uint64_t)wall_clock64() << 4) < pace_next16) __builtin_amdgcn_s_sleep(1);
+                pace_next16 += write_pace16;
+            }
+        };
         for (int k = 0; k < m; k++) {
             // The block's waves start every destination together: left alone they drift apart over the several hundred
             // stores per lane of a phase with many destinations, the chip then writes to several destinations at once,
@@ -1030,10 +1038,12 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
 #pragma unroll
             for (int u = 0; u < G * RG; u++) {
                 const uint64_t i = pos(p0, u);
+                paced(u);
                 if (i < nvec) st_loose(d + i, rs[u]);
             }
             for (int u = 0; u < kPhaseU; u++) {
                 const uint64_t i = pos(p0, G * RG + u);
+                paced(G * RG + u);
                 if (u == arrive_u && k == m - 1 && threadIdx.x == 0) phase_arrive(ps);
                 if (i < nvec) st_loose(d + i, stage[u * kPhaseBlock + threadIdx.x]);
             }
@@ -1181,10 +1191,16 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
         // (with several destinations the write phase, which wants the chip's stores in one compact window, loses more
         // to the runs than the reads gain: 8 -> 8 at 1 GiB 6.28 against 6.46 TB/s)
         const uint32_t wave_runs = a.tune.wave_runs == 2 || (a.tune.wave_runs == 1 && off_lines && a.m == 1);
+        // the write phase's pace (see the kernel): 1/16 clock ticks per group of four stores of the whole grid
+        uint32_t write_pace16 = 0;
+        if (a.m >= 2 && a.tune.write_pace > 0) {
+            const double bytes = (double)grid * kPhaseBlock * 16.0 * 4.0;
+            write_pace16 = (uint32_t)(bytes / ((double)a.tune.write_pace * 1e9) * (double)a.tune.wall_khz * 1e3 * 16.0 + 0.5);
+        }
         g_last_kernel = "reduce_multi_phased_kernel";
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
                            a.m, v.head, v.nvec, v.tail, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune, a.m),
-                           a.tune.spin_ticks, v.beyond, wave_runs);
+                           a.tune.spin_ticks, v.beyond, wave_runs, write_pace16);
         return hipGetLastError();
     }
     constexpr int UNROLL = 4;

@@ -167,6 +167,45 @@ def test_phased_form_over_several_phases(comp):
         comp.set_param("variant", 0)
 
 
+def test_write_phase_paced_by_the_clock(comp):
+    """With two or more destinations the device clock lets the write phase's stores out at a set rate
+    ("phase_write_pace", GB/s).  Timing only: unpaced, the default, a pace far below what HBM takes (every group of
+    stores waits for the clock), one far above (none does) and the largest value all give the oracle's bits, over
+    several phases, with the destinations at different alignments, one of them aliasing an input."""
+    import torch
+    rng = np.random.default_rng(29)
+    assert comp.get_param("phase_write_pace") == 7400 and comp.get_param("wall_clock_khz") > 0
+    comp.set_param("variant", 8)
+    try:
+        for dtype, n, m, count in [(O.BFLOAT16, 3, 3, 70_000_003), (O.FLOAT32, 2, 2, 40_000_001), (O.INT8, 4, 5, 1_000_003)]:
+            np_t, esz = O.NP_STORAGE[dtype], O.DTYPE_SIZE[dtype]
+            keep = 1 if dtype == O.BFLOAT16 else 0
+            srcs = make_inputs(rng, dtype, count, O.SUM, n)
+            want = O.reduce_n(srcs, dtype, O.SUM, keep=keep, threads=16)
+            for pace in (0, 7400, 1500, 60_000, 100_000):
+                comp.set_param("phase_write_pace", pace)
+                d = [to_dev(s) for s in srcs]
+                pad = 64
+                outs = [torch.zeros(count + 2 * pad, dtype=d[0].dtype, device="cuda") for _ in range(m - 1)]
+                shifts = [(k * 8) % pad for k in range(m - 1)]
+                ptrs = [d[n - 1].data_ptr()] + [o.data_ptr() + (pad + sh) * esz for o, sh in zip(outs, shifts)]
+                comp.comp_reduce_write_n(dtype, O.SUM, [t.data_ptr() for t in d], ptrs, count, lp_mode=keep)
+                torch.cuda.synchronize()
+                assert comp.last_kernel() == "reduce_multi_phased_kernel"
+                what = f"{O.DTYPE_NAMES[dtype]} n={n} m={m} count={count} pace={pace}"
+                assert_same(to_host(d[n - 1], np_t), want, dtype, what + " (destination that is an input)", srcs, O.SUM, keep=keep)
+                for o, sh in zip(outs, shifts):
+                    g = to_host(o, np_t)
+                    assert_same(g[pad + sh:pad + sh + count], want, dtype, what, srcs, O.SUM, keep=keep)
+                    assert not g[:pad + sh].view(np.uint8).any() and not g[pad + sh + count:].view(np.uint8).any(), "wrote outside: " + what
+        for bad in (-1, 1, 99, 100_001):
+            with pytest.raises(comp.CclError):
+                comp.set_param("phase_write_pace", bad)
+    finally:
+        comp.set_param("variant", 0)
+        comp.set_param("phase_write_pace", 7400)
+
+
 def test_equals_reduce_n_followed_by_copies_at_a_large_size(comp):
     """Size-independent property at 1 GiB per buffer: every destination equals mi_ccl_comp_reduce_n's output."""
     import torch
