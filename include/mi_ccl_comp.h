@@ -265,7 +265,7 @@ const char* mi_ccl_last_kernel(void);
  * handled element by element; buffers that share an offset from the lines then run like aligned ones, +6 %) and
  * "phase_write_pace" (phased reduce with two or more destinations: the rate in GB/s at which the device clock lets
  * the write phase's stores out, which keeps the blocks of the chip in step and the addresses written at any moment in
- * one compact window; default 7400, 0 = unpaced, otherwise 100 to 100000; 8 inputs stored to 8 buffers of 1 GiB run at 6.95 TB/s paced and 6.4
+ * one compact window; default 7300, 0 = unpaced, otherwise 100 to 100000; 8 inputs stored to 8 buffers of 1 GiB run at 6.95 TB/s paced and 6.4
  * unpaced; a block that is behind the schedule is never held, so a rate above what HBM takes only switches the
  * pacing off), "wall_clock_khz" (read only: the rate of that clock),
  * "wave_runs" (phased kernels: a wave's vectors of one step lie next to each other instead of a block apart, which

@@ -57,7 +57,7 @@ static std::atomic<int> g_fp16_impl{ MI_CCL_FP16_AVX512F };
 static std::atomic<int> g_realign{ 1 };
 static std::atomic<int> g_line_start{ 1 };
 static std::atomic<int> g_wave_runs{ 1 };
-static std::atomic<int> g_write_pace{ 7400 };
+static std::atomic<int> g_write_pace{ 7300 };
 static std::atomic<long> g_launch_block_limit{ 0 };     // 0: what HIP allows; smaller values are for tests of the splitting
 static_assert(kGeomBlock == kBlock, "the geometry header and the kernels agree on the block size");
 
@@ -258,7 +258,21 @@ static int reduce_n_impl(int dtype, int op, const void* const* srcs, int n, void
     if (n == 1 && !keep && tune.variant == 0) {
         if (m == 1)
             return dsts[0] == srcs[0] ? MI_CCL_SUCCESS : launch_copy(srcs[0], dsts[0], count * esz, true, (hipStream_t)stream);
-        return launch_broadcast(srcs[0], dsts, m, count * esz, (hipStream_t)stream);
+        if (!broadcast_wants_phased(tune, (uint64_t)count * esz))
+            return launch_broadcast(srcs[0], dsts, m, count * esz, (hipStream_t)stream);
+        // large: the phased reduce with one input, on bytes (a sum over one unsigned input hands every bit back)
+        LaunchArgs b;
+        b.srcs = srcs;
+        b.n = 1;
+        b.dst = dsts[0];
+        b.dsts = dsts;
+        b.m = m;
+        b.count = count * esz;
+        b.op = MI_CCL_SUM;
+        b.stream = (hipStream_t)stream;
+        b.tune = tune;
+        b.tune.variant = 8;
+        return status_of(dispatch(MI_CCL_UINT8, false, MI_CCL_BF16_AVX512BF, b));
     }
 
     LaunchArgs a;

@@ -1113,16 +1113,28 @@ inline hipError_t launch_fixed_unroll(const LaunchArgs& a, const VecSplit& v) {
     return launch_fixed<TR, OP, N, kDefault>(a, v);
 }
 
+// One buffer to m >= 2: the sectioned broadcast kernel re-reads every section from the L2s and keeps every destination an
+// ascending stream, 6.3-6.5 TB/s at any size; the phased form with the clock pacing its write phase reaches 6.7 (m = 2) to
+// 7.0 (m = 7) from 256 MiB per buffer, equals it at 128 MiB and loses below (one partly filled phase: 5.5-5.9 at 64 MiB).
+inline bool broadcast_wants_phased(const Tuning& t, uint64_t bytes) {
+    if (t.sync == nullptr || t.num_cus < kPhaseGroups || t.max_blocks > 0 || t.variant != 0 || t.write_pace <= 0) return false;
+    const uint64_t grid = (uint64_t)(t.num_cus / kPhaseGroups) * kPhaseGroups;
+    const uint64_t per_phase = grid * kPhaseBlock * (uint64_t)(4 * MultiPhaseRegs<U8Traits>::groups + kPhaseU) * 16u;
+    return bytes >= 2 * per_phase;
+}
+
 // When the phased form pays: from Tuning::phased_min_bytes of traffic per launch (default 160 MB), with two or more
 // inputs and one destination when its phases are full enough (phases_full_enough: long buffers always are: +8 % with
 // 2 inputs, +17 % with 8 at 4 GiB of traffic), with several destinations from twice that traffic.  One input stays with
-// the copy and broadcast kernels.  Tuning::variant 8 forces the phased form.
+// the copy and broadcast kernels, except that a buffer of two phases or more going to several destinations takes the
+// phased form with its paced write phase (broadcast_wants_phased).  Tuning::variant 8 forces the phased form.
 inline bool wants_phased(const LaunchArgs& a, uint64_t nvec, int reg_groups) {
     if (a.tune.sync == nullptr || a.tune.num_cus < kPhaseGroups) return false;
     if (a.tune.variant != 0) return a.tune.variant == 8;
     if (a.tune.max_blocks > 0) return false;        // a caller that caps the grid keeps CUs free: the phased form takes them all
     const uint64_t traffic = (uint64_t)(a.n + a.m) * nvec * 16u;
-    if (a.n < 2 || traffic < (uint64_t)a.tune.phased_min_bytes * (a.m > 1 ? 2u : 1u)) return false;
+    if (a.n < 2) return a.m > 1 && broadcast_wants_phased(a.tune, nvec * 16u);    // one input that is not a plain copy (bf16 keep-precision narrows it)
+    if (traffic < (uint64_t)a.tune.phased_min_bytes * (a.m > 1 ? 2u : 1u)) return false;
     if (a.m > 1) return true;
     const uint64_t grid = (uint64_t)(a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
     return phases_full_enough(nvec, grid * kPhaseBlock * (uint64_t)(4 * reg_groups + kPhaseU), a.n);

@@ -108,14 +108,22 @@ def test_copy_of_more_than_64_GiB(comp):
         assert torch.equal(f[lo:hi], h[lo:hi].to(torch.int32) << 16), f"widening differs in [{lo}, {hi})"
 
 
-def test_broadcast_of_more_than_10_GiB_to_seven(comp):
+@pytest.mark.parametrize("pace", [7300, 0])
+def test_broadcast_of_more_than_10_GiB_to_seven(comp, pace):
+    """By the phased kernel with its clock-paced write phase (the default from two phases' worth of bytes), and, with
+    the pace switched off, by the sectioned broadcast kernel, whose launches are cut at the block limit."""
     import torch
     n = (10 << 30) + 4099
     words = (n + 7) // 8 + 1
     src = torch.arange(words, dtype=torch.int64, device="cuda").mul_(0x9E3779B97F4A7C15 - (1 << 64)).view(torch.uint8)
     dsts = [torch.zeros(words * 8, dtype=torch.uint8, device="cuda") for _ in range(7)]
-    comp.comp_reduce_write_n(comp.UINT8, comp.SUM, [src], dsts, n)
-    torch.cuda.synchronize()
+    comp.set_param("phase_write_pace", pace)
+    try:
+        comp.comp_reduce_write_n(comp.UINT8, comp.SUM, [src], dsts, n)
+        torch.cuda.synchronize()
+        assert comp.last_kernel() == ("reduce_multi_phased_kernel" if pace else "broadcast_kernel")
+    finally:
+        comp.set_param("phase_write_pace", 7300)
     for d in dsts:
         assert torch.equal(d[:n], src[:n])
         assert int(d[n:].count_nonzero()) == 0

@@ -174,7 +174,7 @@ def test_write_phase_paced_by_the_clock(comp):
     several phases, with the destinations at different alignments, one of them aliasing an input."""
     import torch
     rng = np.random.default_rng(29)
-    assert comp.get_param("phase_write_pace") == 7400 and comp.get_param("wall_clock_khz") > 0
+    assert comp.get_param("phase_write_pace") == 7300 and comp.get_param("wall_clock_khz") > 0
     comp.set_param("variant", 8)
     try:
         for dtype, n, m, count in [(O.BFLOAT16, 3, 3, 70_000_003), (O.FLOAT32, 2, 2, 40_000_001), (O.INT8, 4, 5, 1_000_003)]:
@@ -182,7 +182,7 @@ def test_write_phase_paced_by_the_clock(comp):
             keep = 1 if dtype == O.BFLOAT16 else 0
             srcs = make_inputs(rng, dtype, count, O.SUM, n)
             want = O.reduce_n(srcs, dtype, O.SUM, keep=keep, threads=16)
-            for pace in (0, 7400, 1500, 60_000, 100_000):
+            for pace in (0, 7300, 1500, 60_000, 100_000):
                 comp.set_param("phase_write_pace", pace)
                 d = [to_dev(s) for s in srcs]
                 pad = 64
@@ -203,7 +203,7 @@ def test_write_phase_paced_by_the_clock(comp):
                 comp.set_param("phase_write_pace", bad)
     finally:
         comp.set_param("variant", 0)
-        comp.set_param("phase_write_pace", 7400)
+        comp.set_param("phase_write_pace", 7300)
 
 
 def test_equals_reduce_n_followed_by_copies_at_a_large_size(comp):
