@@ -1018,8 +1018,8 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
         // over the chip) not before the phase's start + i * write_pace16 / 16 ticks, a little faster than HBM takes them.
         // Every block reads the same clock, so the blocks stay within a fraction of a group of each other without
         // exchanging a word; a block that is behind the schedule is never held.  8 -> 8 at 1 GiB: 6.95 against 6.40
-        // TB/s, 4 -> 4: 6.90 against 6.35, 2 -> 2: 6.63 against 6.30.  With one destination (44 stores per lane) there is
-        // nothing to gain: 7.04 against 7.10.
+        // TB/s, 4 -> 4: 6.90 against 6.35, 2 -> 2: 6.63 against 6.30.  With one destination (44 stores per lane) and three
+        // or more inputs there is nothing to gain: 7.04 against 7.10.
         uint64_t pace_next16 = write_pace16 ? (uint64_t)wall_clock64() << 4 : 0;
         auto paced = [&](int u) {       // u: slot within the phase; groups that lie behind the end of the data take no time
             if (write_pace16 && (u & 3) == 0 && p0 + (uint64_t)u * gthreads < nvec) {
@@ -1205,9 +1205,14 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
         const uint32_t wave_runs = a.tune.wave_runs == 2 || (a.tune.wave_runs == 1 && off_lines && a.m == 1);
         // the write phase's pace (see the kernel): 1/16 clock ticks per group of four stores of the whole grid
         uint32_t write_pace16 = 0;
-        if (a.m >= 2 && a.tune.write_pace > 0) {
+        // Two inputs to one destination are paced too, a tenth faster (their write phase is a third of the traffic, but
+        // short: 2 GiB per buffer fp32 6.82-6.93 against 6.59-6.70 TB/s, bf16 6.63-6.70 against 6.56-6.59; best at
+        // 1.1 x the pace either way); from three inputs on one destination gains nothing (7.03-7.04 against 7.10 for
+        // eight) and stays unpaced.
+        const double rate = a.m >= 2 ? (double)a.tune.write_pace : a.n == 2 ? 1.1 * (double)a.tune.write_pace : 0.0;
+        if (rate > 0) {
             const double bytes = (double)grid * kPhaseBlock * 16.0 * 4.0;
-            write_pace16 = (uint32_t)(bytes / ((double)a.tune.write_pace * 1e9) * (double)a.tune.wall_khz * 1e3 * 16.0 + 0.5);
+            write_pace16 = (uint32_t)(bytes / (rate * 1e9) * (double)a.tune.wall_khz * 1e3 * 16.0 + 0.5);
         }
         g_last_kernel = "reduce_multi_phased_kernel";
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
