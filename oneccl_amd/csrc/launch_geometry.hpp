@@ -212,6 +212,16 @@ inline unsigned vector_start(const unsigned* in_addr, int n, const unsigned* out
     return best_start;
 }
 
+// ---- the pace of a phased reduce's write phase --------------------------------------------------------------------------
+// The kernel lets group i of four stores per lane out at the phase's start + i * pace: `bytes_per_group` is what the
+// whole grid stores in one group, `rate_gbps` the rate in GB/s the groups are let out at, `clock_khz` the rate of the
+// device's wall clock.  Returns the pace in 1/16 clock ticks (0: unpaced).
+inline uint32_t write_pace_ticks16(uint64_t bytes_per_group, double rate_gbps, int clock_khz) {
+    if (rate_gbps <= 0 || clock_khz <= 0) return 0;
+    const double ticks16 = (double)bytes_per_group / (rate_gbps * 1e9) * (double)clock_khz * 1e3 * 16.0 + 0.5;
+    return ticks16 >= 4294967295.0 ? 4294967295u : (uint32_t)ticks16;
+}
+
 // ---- when the phased form of a reduce pays -----------------------------------------------------------------------
 // A phase costs a fixed few microseconds on top of its traffic, so what counts is how full the phases are:
 // fill = result vectors / (phases x what one phase holds).  Measured against the streaming kernels (fp32 sum, one

@@ -1210,10 +1210,7 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
         // 1.1 x the pace either way); from three inputs on one destination gains nothing (7.03-7.04 against 7.10 for
         // eight) and stays unpaced.
         const double rate = a.m >= 2 ? (double)a.tune.write_pace : a.n == 2 ? 1.1 * (double)a.tune.write_pace : 0.0;
-        if (rate > 0) {
-            const double bytes = (double)grid * kPhaseBlock * 16.0 * 4.0;
-            write_pace16 = (uint32_t)(bytes / (rate * 1e9) * (double)a.tune.wall_khz * 1e3 * 16.0 + 0.5);
-        }
+        write_pace16 = write_pace_ticks16((uint64_t)grid * kPhaseBlock * 16u * 4u, rate, a.tune.wall_khz);
         g_last_kernel = "reduce_multi_phased_kernel";
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
                            a.m, v.head, v.nvec, v.tail, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune, a.m),

@@ -212,6 +212,16 @@ int main() {
             EXPECT(line_price(h0, in, n, out, m) > best || s == h0);        // among equals the head stays as short as it can be
         }
     }
+    // the write phase's pace: 8 MiB per group of stores at 7,300 GB/s on a 100 MHz clock is 1.149 us = 114.9 ticks
+    {
+        EXPECT(write_pace_ticks16(256ull * 512 * 16 * 4, 7300.0, 100000) == 1839);
+        EXPECT(write_pace_ticks16(256ull * 512 * 16 * 4, 8030.0, 100000) == 1671);
+        EXPECT(write_pace_ticks16(240ull * 512 * 16 * 4, 7300.0, 100000) == 1724);       // fewer CUs: less per group, a shorter pace
+        EXPECT(write_pace_ticks16(256ull * 512 * 16 * 4, 7300.0, 25000) == 460);         // a slower clock: fewer ticks
+        EXPECT(write_pace_ticks16(256ull * 512 * 16 * 4, 0.0, 100000) == 0 && write_pace_ticks16(1 << 23, 7300.0, 0) == 0);
+        EXPECT(write_pace_ticks16(256ull * 512 * 16 * 4, 100.0, 100000) == 134218);      // the slowest setting: 8.4 ms per group
+        EXPECT(write_pace_ticks16(~0ull, 1e-9, 100000) == 4294967295u);                  // saturates
+    }
     // whether the phased form pays: the measured crossovers (one phase holds 88 MiB of results on 256 CUs)
     {
         const uint64_t per = 256ull * 512 * 44;
