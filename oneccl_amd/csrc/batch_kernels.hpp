@@ -113,24 +113,57 @@ struct BatchSlot {                  // where one tile lives; the same for every 
     uint64_t nvec, nload;           // the job's vectors that are computed / that may be read
 };
 
+// What lane q of a wave knows about this block's q-th tile of the phase (batch_describe); the tile's owner-independent
+// facts are then handed to all lanes with v_readlane (batch_slot), so that the walk job table -> job -> first vector
+// happens once per phase and tile, beside the payload's loads instead of in front of them, and the write phase needs
+// no second walk.  (Walked per tile, by scalar code in front of the tile's first load, the same table cost the types
+// with more arithmetic per vector 5-8 % with four inputs per job and everything 6-17 % with two.)
+struct BatchDesc {
+    uint32_t job;       // index into the table; ~0u: the phase has no such tile
+    uint32_t headb;     // BatchTable::head of the job
+    uint64_t first;     // the tile's first vector, counted within the job
+    uint64_t nvec;      // the job's vectors that are computed
+};
+
+// `kt`: the job table where the kernel's arguments live in memory (a lane-indexed read of a by-value argument would
+// otherwise make the compiler copy the table to scratch memory).
 template <class TR>
-__device__ __forceinline__ BatchSlot batch_locate(const BatchTable& tb, int n, uint64_t tile, uint32_t total_tiles, int& j) {
-    if (tile >= total_tiles) return BatchSlot{ false, 0, 0, 0, 0, 0, 0 };
-    while (tb.tile_end[j] <= tile) j++;         // tile < total_tiles = tile_end[n_jobs - 1]: j stays below n_jobs
-    const uint32_t beg = j ? tb.tile_end[j - 1] : 0u;
-    const uint32_t beyond = tb.head[j] >> 7;
+__device__ __forceinline__ BatchDesc batch_describe(const BatchTable* kt, int n_jobs, uint64_t tile, uint32_t total_tiles) {
+    BatchDesc d = { ~0u, 0u, 0u, 0u };
+    if (tile < total_tiles) {
+        int lo = 0, hi = n_jobs - 1;                // first job whose tiles end beyond `tile`
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (kt->tile_end[mid] > tile) hi = mid;
+            else lo = mid + 1;
+        }
+        const uint32_t beg = lo ? kt->tile_end[lo - 1] : 0u;
+        d.job = (uint32_t)lo;
+        d.headb = kt->head[lo];
+        d.first = (tile - beg) * kBatchPhaseTile;
+        d.nvec = (kt->count[lo] - (d.headb & 0x7fu)) / TR::VEC - (d.headb >> 7);
+    }
+    return d;
+}
+__device__ __forceinline__ uint64_t readlane64(uint64_t v, int lane) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, lane);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), lane);
+    return ((uint64_t)hi << 32) | lo;
+}
+__device__ __forceinline__ BatchSlot batch_slot(const BatchDesc& d, int q, int n) {
     BatchSlot s;
-    s.valid = true;
-    s.job = (uint32_t)j;
-    s.p0 = (uint32_t)(j * (n + 1));
-    s.head = tb.head[j] & 0x7fu;
-    s.first = (tile - beg) * kBatchPhaseTile;
-    s.nvec = (tb.count[j] - s.head) / TR::VEC - beyond;
-    s.nload = s.nvec + beyond;
+    const uint32_t job = (uint32_t)__builtin_amdgcn_readlane((int)d.job, q);
+    const uint32_t headb = (uint32_t)__builtin_amdgcn_readlane((int)d.headb, q);
+    s.valid = job != ~0u;
+    s.job = s.valid ? job : 0u;
+    s.p0 = s.job * (uint32_t)(n + 1);
+    s.head = headb & 0x7fu;
+    s.first = readlane64(d.first, q);
+    s.nvec = readlane64(d.nvec, q);
+    s.nload = s.nvec + (headb >> 7);
     return s;
 }
 
-// One tile: four vectors per lane, the inputs one after the other (reduce_rt_tile for a job of the table).
 // Vector g of this lane within a tile: the four lie a quarter of the tile apart, or -- wave_runs, for buffers off the
 // 128-byte lines -- 64 vectors apart, so that a wave covers 4 KiB in one run (see reduce_multi_phased_kernel).
 __device__ __forceinline__ uint32_t batch_tile_vector(int g, uint32_t wave_runs) {
@@ -193,26 +226,21 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
     __shared__ u32x4 stage[kPhaseU * kPhaseBlock];
     const uint64_t grid = gridDim.x;
     const uint64_t per_phase = grid * (uint64_t)(RG + LG);  // tiles
+    static_assert(RG + LG <= 64, "one tile description per lane of a wave");
+    // the job table is the kernel's first argument: it starts the kernel-argument segment
+    const BatchTable* kt = (const BatchTable*)__builtin_amdgcn_kernarg_segment_ptr();
     bool give_up = false;
     unsigned gen = 0;
     if (threadIdx.x == 0) gen = phase_generation(ps);
     for (uint64_t t0 = 0; t0 < total_tiles; t0 += per_phase) {
-        const uint64_t tile0 = t0 + blockIdx.x;             // this block's tile of group q: tile0 + q * grid
-        int j0 = 0;                                         // the job of this block's first tile of the phase
-        if (tile0 < total_tiles) {
-            int lo = 0, hi = n_jobs - 1;
-            while (lo < hi) {
-                const int mid = (lo + hi) >> 1;
-                if (tb.tile_end[mid] > tile0) hi = mid;
-                else lo = mid + 1;
-            }
-            j0 = lo;
-        }
-        int jr = j0;
+        // lane q of every wave describes this block's tile of group q: tile t0 + q * grid + blockIdx.x
+        const uint32_t lane = threadIdx.x & 63u;
+        const BatchDesc desc = batch_describe<TR>(kt, n_jobs, lane < (uint32_t)(RG + LG) ? t0 + (uint64_t)lane * grid + blockIdx.x : (uint64_t)total_tiles,
+                                                  total_tiles);
         u32x4 rs[G * (RG > 0 ? RG : 1)];
 #pragma unroll
         for (int q = 0; q < RG; q++) {
-            const BatchSlot s = batch_locate<TR>(tb, n, tile0 + (uint64_t)q * grid, total_tiles, jr);
+            const BatchSlot s = batch_slot(desc, q, n);
             if (s.valid) {
                 u32x4 v[G];
                 reduce_batch_tile<TR, OP>(tb, n, s, wave_runs, v);
@@ -222,7 +250,7 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
         }
         bool arrived = false;
         for (int q = 0; q < LG; q++) {
-            const BatchSlot s = batch_locate<TR>(tb, n, tile0 + (uint64_t)(RG + q) * grid, total_tiles, jr);
+            const BatchSlot s = batch_slot(desc, RG + q, n);
             if (!s.valid) break;                            // tiles ascend with q: nothing further in this phase
             const int rem = (LG - q) * n * G;               // loads per lane still to issue in this phase
             int arrive_k = 0;
@@ -242,10 +270,9 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
         phase_wait(ps, ++gen, give_up, spin_ticks);
         const bool more = t0 + per_phase < total_tiles;
         const int arrive_u = more ? kPhaseU - early_stores : -1;    // kPhaseU: after the last store
-        int jw = j0;
 #pragma unroll
         for (int q = 0; q < RG; q++) {
-            const BatchSlot s = batch_locate<TR>(tb, n, tile0 + (uint64_t)q * grid, total_tiles, jw);
+            const BatchSlot s = batch_slot(desc, q, n);
             u32x4_u* d = (u32x4_u*)((unsigned char*)tb.p[s.p0 + n] + s.head * sizeof(E));
 #pragma unroll
             for (int g = 0; g < G; g++) {
@@ -254,7 +281,7 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
             }
         }
         for (int q = 0; q < LG; q++) {
-            const BatchSlot s = batch_locate<TR>(tb, n, tile0 + (uint64_t)(RG + q) * grid, total_tiles, jw);
+            const BatchSlot s = batch_slot(desc, RG + q, n);
             u32x4_u* d = (u32x4_u*)((unsigned char*)tb.p[s.p0 + n] + s.head * sizeof(E));
 #pragma unroll
             for (int g = 0; g < G; g++) {
