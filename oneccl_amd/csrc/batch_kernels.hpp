@@ -216,7 +216,7 @@ __device__ __forceinline__ void reduce_batch_edges(const BatchTable& tb, int n, 
 template <class TR, int OP>
 __global__ void __launch_bounds__(kPhaseBlock)
 reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tiles, PhaseSync* ps, int early_loads,
-                           int early_stores, long spin_ticks, uint32_t wave_runs) {
+                           int early_stores, long spin_ticks, uint32_t wave_runs, uint32_t write_pace16) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr int G = kBatchPhaseG;
@@ -232,11 +232,16 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
     bool give_up = false;
     unsigned gen = 0;
     if (threadIdx.x == 0) gen = phase_generation(ps);
+    // lane q of every wave describes this block's tile of group q of a phase: tile t0 + q * grid + blockIdx.x.  The
+    // first phase's tiles are described here, every later phase's while the block waits at the barrier in the middle of
+    // the phase before (the walk is a chain of dependent loads, about a microsecond).
+    const uint32_t lane = threadIdx.x & 63u;
+    auto describe = [&](uint64_t t0) {
+        return batch_describe<TR>(kt, n_jobs, lane < (uint32_t)(RG + LG) ? t0 + (uint64_t)lane * grid + blockIdx.x : (uint64_t)total_tiles,
+                                  total_tiles);
+    };
+    BatchDesc desc = describe(0);
     for (uint64_t t0 = 0; t0 < total_tiles; t0 += per_phase) {
-        // lane q of every wave describes this block's tile of group q: tile t0 + q * grid + blockIdx.x
-        const uint32_t lane = threadIdx.x & 63u;
-        const BatchDesc desc = batch_describe<TR>(kt, n_jobs, lane < (uint32_t)(RG + LG) ? t0 + (uint64_t)lane * grid + blockIdx.x : (uint64_t)total_tiles,
-                                                  total_tiles);
         u32x4 rs[G * (RG > 0 ? RG : 1)];
 #pragma unroll
         for (int q = 0; q < RG; q++) {
@@ -267,12 +272,21 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
         }
         if (early_loads == 0) __syncthreads();              // "when done" means the whole block, and its loads have landed
         if (!arrived && threadIdx.x == 0) phase_arrive(ps);
+        const BatchDesc next = describe(t0 + per_phase);
         phase_wait(ps, ++gen, give_up, spin_ticks);
         const bool more = t0 + per_phase < total_tiles;
         const int arrive_u = more ? kPhaseU - early_stores : -1;    // kPhaseU: after the last store
+        uint64_t pace_next16 = write_pace16 ? (uint64_t)wall_clock64() << 4 : 0;
+        auto paced = [&](bool valid) {
+            if (write_pace16 && valid) {
+                while (((uint64_t)wall_clock64() << 4) < pace_next16) __builtin_amdgcn_s_sleep(1);
+                pace_next16 += write_pace16;
+            }
+        };
 #pragma unroll
         for (int q = 0; q < RG; q++) {
             const BatchSlot s = batch_slot(desc, q, n);
+            paced(s.valid);
             u32x4_u* d = (u32x4_u*)((unsigned char*)tb.p[s.p0 + n] + s.head * sizeof(E));
 #pragma unroll
             for (int g = 0; g < G; g++) {
@@ -282,6 +296,7 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
         }
         for (int q = 0; q < LG; q++) {
             const BatchSlot s = batch_slot(desc, RG + q, n);
+            paced(s.valid);
             u32x4_u* d = (u32x4_u*)((unsigned char*)tb.p[s.p0 + n] + s.head * sizeof(E));
 #pragma unroll
             for (int g = 0; g < G; g++) {
@@ -297,6 +312,7 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
             }
             phase_wait(ps, ++gen, give_up, spin_ticks);
         }
+        desc = next;
     }
     // The jobs' edge elements, after the last phase and spread over the blocks: their loads depend on one another (the
     // inputs are taken in order), and inside a read phase that chain of round trips held up the one block of a job's
@@ -376,6 +392,7 @@ inline hipError_t launch_batch_op(const BatchLaunchArgs& a) {
                     off_lines |= (uint32_t)((uintptr_t)tb.p[q * (a.n + 1) + k] + split[q].head * sizeof(E)) & (kLineBytes - 1);
         }
         const uint32_t wave_runs = a.tune.wave_runs == 2 || (a.tune.wave_runs == 1 && off_lines);
+        const uint32_t write_pace16 = a.n == 2 ? write_pace_ticks16(phase_grid * kBatchPhaseTile * 16u, 1.1 * (double)a.tune.write_pace, a.tune.wall_khz) : 0u;
         j0 += nj;
         if (tiles == 0) continue;
         g_realigned_launches += realigned;
@@ -383,7 +400,7 @@ inline hipError_t launch_batch_op(const BatchLaunchArgs& a) {
             g_last_kernel = "reduce_batch_phased_kernel";
             hipLaunchKernelGGL((reduce_batch_phased_kernel<TR, OP>), dim3((unsigned)phase_grid), dim3(kPhaseBlock), 0, a.stream, tb, a.n,
                                nj, (uint32_t)tiles, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks,
-                               wave_runs);
+                               wave_runs, write_pace16);
         }
         else {
             g_last_kernel = "reduce_batch_kernel";

@@ -124,6 +124,15 @@ def test_chunk_sized_jobs_take_the_phased_form(comp):
     assert comp.last_kernel() == "reduce_batch_phased_kernel"
     _run(comp, rng, O.BFLOAT16, O.SUM, 2, [(48 << 20) // 2] * 7, in_place_every=0)
     assert comp.last_kernel() == "reduce_batch_phased_kernel"
+    # jobs of two inputs have their write phase paced by the device clock: unpaced, a pace no store keeps up with and
+    # one that every group of stores waits for give the same bits, with jobs that end inside a tile and in place
+    try:
+        for pace in (0, 100_000, 2000):
+            comp.set_param("phase_write_pace", pace)
+            _run(comp, rng, O.FLOAT32, O.SUM, 2, [(6 << 20) // 4 + 5 * j for j in range(40)], in_place_every=3)
+            assert comp.last_kernel() == "reduce_batch_phased_kernel"
+    finally:
+        comp.set_param("phase_write_pace", 7300)
 
 
 def test_sixteen_bit_modes_and_nan_patterns(comp):
