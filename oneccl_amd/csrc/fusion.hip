@@ -134,6 +134,7 @@ static hipError_t dispatch_fusion(int dtype, bool keep, int bf16_impl, const Fus
 struct StaticFusionTable {
     uint64_t off[MI_CCL_FUSION_STATIC_MAX_TENSORS];
     uint64_t bytes[MI_CCL_FUSION_STATIC_MAX_TENSORS];
+    uint32_t tile_end[MI_CCL_FUSION_STATIC_MAX_TENSORS];
     FusionItem items[MI_CCL_FUSION_STATIC_MAX_ITEMS];
 };
 // kStaticSlots tables per GPU, taken in turn by the calls on that GPU: a call's table is rewritten by the call that
@@ -171,21 +172,24 @@ struct FusionSizes {                // by-value kernel argument: the sizes of on
 
 // Block b writes the table rows of tensor t0 + b: its byte offset in the fusion buffer (running end rounded up to
 // `align`, from `end0`, the end of the tensor before the group), its size, and its work items from item index
-// `item0` + (items of the group's tensors before it).  Every lane walks the (at most kFusionGroup) sizes before its
+// `item0` + (items of the group's tensors before it), and the running count of kFusionTile-byte tiles through it.  Every lane walks the (at most kFusionGroup) sizes before its
 // tensor; they are kernel arguments, so the walk is scalar work.
 __global__ void __launch_bounds__(kBlock)
-fusion_table_kernel(FusionSizes sz, uint32_t t0, uint64_t end0, uint64_t align, uint64_t item0, StaticFusionTable* tab) {
+fusion_table_kernel(FusionSizes sz, uint32_t t0, uint64_t end0, uint64_t align, uint64_t item0, uint64_t tile0,
+                    StaticFusionTable* tab) {
     const uint32_t b = blockIdx.x;
-    uint64_t end = end0, item = item0;
+    uint64_t end = end0, item = item0, tile = tile0;
     for (uint32_t u = 0; u < b; u++) {
         end = ((end + align - 1) & ~(align - 1)) + sz.bytes[u];
         item += (sz.bytes[u] + kFusionChunk - 1) / kFusionChunk;
+        tile += (sz.bytes[u] + kFusionTile - 1) / kFusionTile;
     }
     const uint64_t off = (end + align - 1) & ~(align - 1);
     const uint64_t nb = sz.bytes[b];
     if (threadIdx.x == 0) {
         tab->off[t0 + b] = off;
         tab->bytes[t0 + b] = nb;
+        tab->tile_end[t0 + b] = (uint32_t)(tile + (nb + kFusionTile - 1) / kFusionTile);
     }
     const uint64_t chunks = (nb + kFusionChunk - 1) / kFusionChunk;
     for (uint64_t c = threadIdx.x; c < chunks; c += kBlock) tab->items[item + c] = FusionItem{ t0 + b, (uint32_t)c };
@@ -204,10 +208,12 @@ struct mi_ccl_fusion_plan {
     std::vector<size_t> counts;
     std::vector<size_t> offsets;           // bytes
     std::vector<uint64_t> item_begin;      // k + 1
-    void* d_table = nullptr;               // [off: k x u64][bytes: k x u64][items]
+    std::vector<uint64_t> tile_begin;      // k + 1: tiles of kFusionTile bytes
+    void* d_table = nullptr;               // [off: k x u64][bytes: k x u64][items][tile_end: k x u32]
     const uint64_t* d_off = nullptr;
     const uint64_t* d_bytes = nullptr;
     const FusionItem* d_items = nullptr;
+    const uint32_t* d_tile_end = nullptr;
 };
 
 extern "C" {
@@ -248,11 +254,17 @@ static int plan_build(mi_ccl_fusion_plan* p, const size_t* counts, size_t k, int
     }
     p->item_begin[k] = items.size();
     std::vector<uint64_t> host(2 * k);
+    std::vector<uint32_t> tile_end(k);
+    p->tile_begin.resize(k + 1);
+    p->tile_begin[0] = 0;
     for (size_t t = 0; t < k; t++) {
         host[t] = p->offsets[t];
         host[k + t] = (uint64_t)counts[t] * esz;
+        p->tile_begin[t + 1] = p->tile_begin[t] + (host[k + t] + kFusionTile - 1) / kFusionTile;
+        tile_end[t] = (uint32_t)p->tile_begin[t + 1];       // fits: there are no more tiles than items
     }
-    const size_t table_bytes = 2 * k * sizeof(uint64_t) + (items.size() ? items.size() : 1) * sizeof(FusionItem);
+    const size_t items_bytes = (items.size() ? items.size() : 1) * sizeof(FusionItem);
+    const size_t table_bytes = 2 * k * sizeof(uint64_t) + items_bytes + k * sizeof(uint32_t);
     hipError_t e = hipMalloc(&p->d_table, table_bytes);
     if (e != hipSuccess) {
         p->d_table = nullptr;
@@ -262,11 +274,15 @@ static int plan_build(mi_ccl_fusion_plan* p, const size_t* counts, size_t k, int
     if (e == hipSuccess && !items.empty())
         e = hipMemcpy((char*)p->d_table + 2 * k * sizeof(uint64_t), items.data(), items.size() * sizeof(FusionItem),
                       hipMemcpyHostToDevice);
+    if (e == hipSuccess)
+        e = hipMemcpy((char*)p->d_table + 2 * k * sizeof(uint64_t) + items_bytes, tile_end.data(), k * sizeof(uint32_t),
+                      hipMemcpyHostToDevice);
     if (e != hipSuccess)
         return fusion_status_of(e);
     p->d_off = (const uint64_t*)p->d_table;
     p->d_bytes = p->d_off + k;
     p->d_items = (const FusionItem*)(p->d_bytes + k);
+    p->d_tile_end = (const uint32_t*)((const char*)p->d_items + items_bytes);
     return MI_CCL_SUCCESS;
 }
 
@@ -382,7 +398,9 @@ int mi_ccl_fusion_reduce(mi_ccl_fusion_plan* plan, int op, const void* const* ow
     a.d_off = plan->d_off;
     a.d_bytes = plan->d_bytes;
     a.d_items = plan->d_items;
+    a.d_tile_end = plan->d_tile_end;
     a.item_begin = plan->item_begin.data();
+    a.tile_begin = plan->tile_begin.data();
     a.stream = (hipStream_t)stream;
     a.tune = current_tuning();
     if (fp16_impl != MI_CCL_FP16_DEFAULT)
@@ -408,12 +426,15 @@ int mi_ccl_fusion_reduce_static(const size_t* counts, size_t k, int dtype, size_
     if (k > MI_CCL_FUSION_STATIC_MAX_TENSORS)
         return MI_CCL_OUT_OF_RESOURCE;          // more tensors than the table holds
     uint64_t item_begin[MI_CCL_FUSION_STATIC_MAX_TENSORS + 1];      // on the stack: nothing is allocated here
-    uint64_t items = 0;
+    uint64_t tile_begin[MI_CCL_FUSION_STATIC_MAX_TENSORS + 1];
+    uint64_t items = 0, tiles = 0;
     for (size_t t = 0; t < k; t++) {
         item_begin[t] = items;
+        tile_begin[t] = tiles;
         if (counts[t] > ((uint64_t)1 << 40) / esz)
             return MI_CCL_OUT_OF_RESOURCE;
         items += ((uint64_t)counts[t] * esz + kFusionChunk - 1) / kFusionChunk;
+        tiles += ((uint64_t)counts[t] * esz + kFusionTile - 1) / kFusionTile;
         if (items > MI_CCL_FUSION_STATIC_MAX_ITEMS)
             return MI_CCL_OUT_OF_RESOURCE;      // more payload than the item list holds
         if (counts[t] == 0)
@@ -422,6 +443,7 @@ int mi_ccl_fusion_reduce_static(const size_t* counts, size_t k, int dtype, size_
             return MI_CCL_INVALID_ARGUMENTS;
     }
     item_begin[k] = items;
+    tile_begin[k] = tiles;
     for (int j = 0; j < n_peers; j++)
         if (!peers[j] || ((uintptr_t)peers[j] % esz))
             return MI_CCL_INVALID_ARGUMENTS;
@@ -439,7 +461,7 @@ int mi_ccl_fusion_reduce_static(const size_t* counts, size_t k, int dtype, size_
         FusionSizes sz;
         for (size_t t = t0; t < t1; t++) sz.bytes[t - t0] = (uint64_t)counts[t] * esz;
         hipLaunchKernelGGL(fusion_table_kernel, dim3((unsigned)(t1 - t0)), dim3(kBlock), 0, (hipStream_t)stream, sz,
-                           (uint32_t)t0, end, (uint64_t)align, item_begin[t0], tab);
+                           (uint32_t)t0, end, (uint64_t)align, item_begin[t0], tile_begin[t0], tab);
         e = hipGetLastError();
         if (e != hipSuccess)
             return fusion_status_of(e);
@@ -455,7 +477,9 @@ int mi_ccl_fusion_reduce_static(const size_t* counts, size_t k, int dtype, size_
     a.d_off = tab->off;             // address arithmetic on the looked-up device address, no host access
     a.d_bytes = tab->bytes;
     a.d_items = tab->items;
+    a.d_tile_end = tab->tile_end;
     a.item_begin = item_begin;
+    a.tile_begin = tile_begin;
     a.stream = (hipStream_t)stream;
     a.tune = current_tuning();
     if (fp16_impl != MI_CCL_FP16_DEFAULT)

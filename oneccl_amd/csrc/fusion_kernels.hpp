@@ -9,7 +9,7 @@
 // per launch of the fused reduce (two tables: inputs and outputs), more for pack and unpack (one table).
 #pragma once
 
-#include "reduce_kernels.hpp"
+#include "batch_kernels.hpp"
 
 namespace mi {
 
@@ -47,7 +47,9 @@ struct FusionLaunchArgs {
     const uint64_t* d_off;        // device tables of the plan
     const uint64_t* d_bytes;
     const FusionItem* d_items;
+    const uint32_t* d_tile_end;   // device: tiles of kFusionTile bytes of tensors 0..t together
     const uint64_t* item_begin;   // host: first item of tensor t, k + 1 entries
+    const uint64_t* tile_begin;   // host: first tile of tensor t, k + 1 entries
     hipStream_t stream;
     Tuning tune;
 };
@@ -310,6 +312,233 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// The phased fused reduce in tiles: the scheme of reduce_batch_phased_kernel with the tensors of a plan as its jobs.  A
+// tile is kFusionTile bytes of one tensor (four vectors per lane), the inputs -- the own tensor, then the peers' slices
+// in argument order -- are taken one after the other with four vectors of one input in flight per lane, the number of
+// peers is a run-time count, and what a tile needs to know (where it starts in the own tensor, in the output and in
+// the peers' buffers, its size, head and the realignment's needs) is worked out by lane q of every wave for the
+// block's q-th tile of a phase: the first phase's at the start, every later one's while the block waits at the
+// barrier in the middle of the phase before.  Elements before a tile's first and after its last vector are left to
+// a pass after the last phase.
+constexpr uint32_t kFusionTile = (uint32_t)kBatchPhaseTile * 16u;       // 32 KiB
+
+struct FusionDesc {
+    uint64_t a, o, poff;    // where the tile starts: own tensor, output tensor, offset into every peer's buffer
+    uint32_t nb;            // bytes of the tile; 0: the phase has no such tile
+    uint32_t headb;         // elements before the tile's first vector (bits 0-7); bits 8-9: fusion_beyond's answer;
+                            // bit 10: a buffer's first vector is off the 128-byte lines
+};
+
+template <class TR>
+__device__ __forceinline__ FusionDesc fusion_describe(const FusionPtrs& own, const FusionPtrs& out, const PeerPtrs& peers,
+                                                      int n_peers, const uint64_t* off, const uint64_t* bytes,
+                                                      const uint32_t* tile_end, uint32_t t0, uint32_t nt, uint32_t tile_base,
+                                                      uint64_t tile, uint32_t ntiles, uint32_t realign) {
+    typedef typename TR::elem_t E;
+    constexpr uint32_t ES = sizeof(E);
+    FusionDesc d = { 0, 0, 0, 0u, 0u };
+    if (tile < ntiles) {
+        const uint32_t key = tile_base + (uint32_t)tile;        // counted from the plan's first tensor, as tile_end is
+        uint32_t lo = t0, hi = t0 + nt - 1;                     // first tensor whose tiles end beyond `key`
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (tile_end[mid] > key) hi = mid;
+            else lo = mid + 1;
+        }
+        const uint32_t beg = lo > t0 ? tile_end[lo - 1] : tile_base;
+        const uint64_t at = (uint64_t)(key - beg) * kFusionTile;
+        const uint64_t left = bytes[lo] - at;
+        d.nb = left < kFusionTile ? (uint32_t)left : kFusionTile;
+        d.a = own.get(lo - t0) + at;
+        d.o = out.get(lo - t0) + at;
+        d.poff = off[lo] + at;
+        uint32_t head = fusion_head<ES>((const void*)(uintptr_t)d.o);
+        const uint32_t ne = d.nb / ES;
+        if (head > ne) head = ne;
+        d.headb = head | fusion_beyond<ES>((const void*)(uintptr_t)(d.a + head * ES), peers, n_peers, d.poff + head * ES,
+                                           (ne - head) / TR::VEC, left - d.nb, realign) << 8;
+        const uint32_t hbytes = head * ES;
+        uint32_t off_lines = (uint32_t)(d.a + hbytes) | (uint32_t)(d.o + hbytes);
+        for (int j = 0; j < n_peers; j++) off_lines |= (uint32_t)((uintptr_t)peers.p[j] + d.poff + hbytes);
+        if (off_lines & (kLineBytes - 1)) d.headb |= 1u << 10;
+    }
+    return d;
+}
+
+struct FusionSlot {             // a tile's description, the same in every lane
+    const unsigned char* a;
+    unsigned char* o;
+    uint64_t poff;
+    uint32_t nb, head, nvec, nload, tail;
+    bool runs;
+};
+template <class TR>
+__device__ __forceinline__ FusionSlot fusion_slot(const FusionDesc& d, int q, uint32_t wave_runs) {
+    constexpr uint32_t ES = sizeof(typename TR::elem_t);
+    FusionSlot s;
+    s.nb = (uint32_t)__builtin_amdgcn_readlane((int)d.nb, q);
+    const uint32_t hb = (uint32_t)__builtin_amdgcn_readlane((int)d.headb, q);
+    s.a = (const unsigned char*)(uintptr_t)readlane64(d.a, q);
+    s.o = (unsigned char*)(uintptr_t)readlane64(d.o, q);
+    s.poff = readlane64(d.poff, q);
+    const uint32_t ne = s.nb / ES;
+    s.head = hb & 0xffu;
+    s.nvec = (ne - s.head) / TR::VEC - ((hb >> 9) & 1u);
+    s.nload = s.nvec + ((hb >> 8) & 1u);
+    s.tail = ne - s.head - s.nvec * TR::VEC;
+    s.runs = wave_runs == 2 || (wave_runs == 1 && ((hb >> 10) & 1u));
+    return s;
+}
+
+template <class TR, int OP>
+__device__ __forceinline__ void fusion_tile(const PeerPtrs& peers, int n_peers, const FusionSlot& s, u32x4 (&out)[kBatchPhaseG],
+                                            PhaseSync* arrive_ps = nullptr, int arrive_k = 0) {
+    typedef typename TR::elem_t E;
+    constexpr int G = kBatchPhaseG;
+    constexpr uint32_t ES = sizeof(E);
+    Accs<TR> acc[G];
+    u32x4 x[G];
+    uint64_t idx[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) idx[g] = batch_tile_vector(g, s.runs ? 1u : 0u);
+    load_vectors<ES, G, false>(s.a + s.head * ES, idx, s.nvec, s.nload, x);
+#pragma unroll
+    for (int g = 0; g < G; g++) acc[g] = vec_init<TR>(x[g]);
+    for (int j = 0; j < n_peers; j++) {
+        if (j + 1 == arrive_k && threadIdx.x == 0) phase_arrive(arrive_ps);     // arrive_k == 0: never
+        load_vectors<ES, G, false>((const unsigned char*)peers.p[j] + s.poff + s.head * ES, idx, s.nvec, s.nload, x);
+#pragma unroll
+        for (int g = 0; g < G; g++) vec_step<TR, OP>(x[g], acc[g]);
+    }
+#pragma unroll
+    for (int g = 0; g < G; g++) out[g] = vec_finish<TR>(acc[g]);
+}
+
+template <class TR, int OP>
+__global__ void __launch_bounds__(kPhaseBlock)
+fusion_reduce_tiled_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers, const uint64_t* off,
+                           const uint64_t* bytes, const uint32_t* tile_end, uint32_t t0, uint32_t nt, uint32_t tile_base,
+                           uint32_t ntiles, PhaseSync* ps, int early_loads, int early_stores, long spin_ticks,
+                           uint32_t realign, uint32_t wave_runs) {
+    typedef typename TR::elem_t E;
+    kernel_prologue<TR, OP>();
+    constexpr uint32_t ES = sizeof(E);
+    constexpr int G = kBatchPhaseG;
+    constexpr int RG = MultiPhaseRegs<TR>::groups;
+    constexpr int LG = kPhaseU / G;
+    static_assert(RG + LG <= 64, "one tile description per lane of a wave");
+    __shared__ u32x4 stage[kPhaseU * kPhaseBlock];
+    const int n = n_peers + 1;
+    const uint64_t grid = gridDim.x;
+    const uint64_t per_phase = grid * (uint64_t)(RG + LG);      // tiles
+    const uint32_t lane = threadIdx.x & 63u;
+    auto describe = [&](uint64_t tile) {
+        return fusion_describe<TR>(own, out, peers, n_peers, off, bytes, tile_end, t0, nt, tile_base, tile, ntiles, realign);
+    };
+    bool give_up = false;
+    unsigned gen = 0;
+    if (threadIdx.x == 0) gen = phase_generation(ps);
+    FusionDesc desc = describe(lane < (uint32_t)(RG + LG) ? (uint64_t)lane * grid + blockIdx.x : (uint64_t)ntiles);
+    for (uint64_t p0 = 0; p0 < ntiles; p0 += per_phase) {
+        u32x4 rs[G * (RG > 0 ? RG : 1)];
+#pragma unroll
+        for (int q = 0; q < RG; q++) {
+            const FusionSlot s = fusion_slot<TR>(desc, q, wave_runs);
+            if (s.nb) {
+                u32x4 v[G];
+                fusion_tile<TR, OP>(peers, n_peers, s, v);
+#pragma unroll
+                for (int g = 0; g < G; g++) rs[q * G + g] = v[g];
+            }
+        }
+        bool arrived = false;
+        for (int q = 0; q < LG; q++) {
+            const FusionSlot s = fusion_slot<TR>(desc, RG + q, wave_runs);
+            if (!s.nb) break;                               // tiles ascend with q: nothing further in this phase
+            const int rem = (LG - q) * n * G;               // loads per lane still to issue in this phase
+            int arrive_k = 0;
+            if (!arrived) {
+                const int k = rem > early_loads ? (rem - early_loads + G - 1) / G : 0;
+                if (k == 0 && threadIdx.x == 0) phase_arrive(ps);
+                arrive_k = k < n ? k : 0;
+                arrived = k < n;
+            }
+            u32x4 v[G];
+            fusion_tile<TR, OP>(peers, n_peers, s, v, ps, arrive_k);
+#pragma unroll
+            for (int g = 0; g < G; g++) stage[(q * G + g) * kPhaseBlock + threadIdx.x] = v[g];
+        }
+        if (early_loads == 0) __syncthreads();              // "when done" means the whole block, and its loads have landed
+        if (!arrived && threadIdx.x == 0) phase_arrive(ps);
+        const uint64_t np = p0 + per_phase;
+        const FusionDesc next = describe(lane < (uint32_t)(RG + LG) ? np + (uint64_t)lane * grid + blockIdx.x : (uint64_t)ntiles);
+        phase_wait(ps, ++gen, give_up, spin_ticks);
+        const bool more = np < ntiles;
+        const int arrive_u = more ? kPhaseU - early_stores : -1;    // kPhaseU: after the last store
+#pragma unroll
+        for (int q = 0; q < RG; q++) {
+            const FusionSlot s = fusion_slot<TR>(desc, q, wave_runs);
+            u32x4_u* d = (u32x4_u*)(s.o + s.head * ES);
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const uint32_t i = batch_tile_vector(g, s.runs ? 1u : 0u);
+                if (i < s.nvec) st_loose(d + i, rs[q * G + g]);
+            }
+        }
+        for (int q = 0; q < LG; q++) {
+            const FusionSlot s = fusion_slot<TR>(desc, RG + q, wave_runs);
+            u32x4_u* d = (u32x4_u*)(s.o + s.head * ES);
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const uint32_t i = batch_tile_vector(g, s.runs ? 1u : 0u);
+                if (q * G + g == arrive_u && threadIdx.x == 0) phase_arrive(ps);
+                if (i < s.nvec) st_loose(d + i, stage[(q * G + g) * kPhaseBlock + threadIdx.x]);
+            }
+        }
+        if (more) {
+            if (arrive_u == kPhaseU) {
+                __syncthreads();                            // "when done": every wave's stores have been acknowledged
+                if (threadIdx.x == 0) phase_arrive(ps);
+            }
+            phase_wait(ps, ++gen, give_up, spin_ticks);
+        }
+        desc = next;
+    }
+    // The elements before a tile's first and after its last vector: this block's tiles once more, 64 at a time (lane
+    // L describes tile base + L * grid), and for those that have such elements one element per lane, the inputs in
+    // order.  After the last phase, because the loads of that chain depend on one another.
+    for (uint64_t base = blockIdx.x; base < ntiles; base += 64u * grid) {
+        const FusionDesc e = describe(base + (uint64_t)lane * grid);
+        uint32_t ne = e.nb / ES, eh = e.headb & 0xffu;
+        uint32_t ev = e.nb ? (ne - eh) / TR::VEC - ((e.headb >> 9) & 1u) : 0u;
+        unsigned long long todo = __ballot(e.nb != 0 && (eh + (ne - eh - ev * TR::VEC)) != 0);
+        while (todo) {
+            const int q = __builtin_ctzll(todo);
+            todo &= todo - 1;
+            const FusionSlot s = fusion_slot<TR>(e, q, 0);
+            if (threadIdx.x < s.head + s.tail) {
+                const uint32_t i = (threadIdx.x < s.head) ? threadIdx.x : s.head + s.nvec * TR::VEC + (threadIdx.x - s.head);
+                typename TR::acc_t r = TR::init(ld_elem<E>(s.a, i));
+                for (int j = 0; j < n_peers; j++) r = TR::template step<OP>(ld_elem<E>((const unsigned char*)peers.p[j] + s.poff, i), r);
+                st_elem<E>(s.o, i, TR::finish(r));
+            }
+        }
+    }
+}
+
+template <class TR, int OP>
+inline hipError_t launch_fusion_tiled(const FusionLaunchArgs& a, const FusionPtrs& own, const FusionPtrs& out,
+                                      const PeerPtrs& pp, size_t t0, size_t t1) {
+    const int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
+    g_last_kernel = "fusion_reduce_tiled_kernel";
+    hipLaunchKernelGGL((fusion_reduce_tiled_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, own, out, pp, a.n_peers,
+                       a.d_off, a.d_bytes, a.d_tile_end, (uint32_t)t0, (uint32_t)(t1 - t0), (uint32_t)a.tile_begin[t0],
+                       (uint32_t)(a.tile_begin[t1] - a.tile_begin[t0]), a.tune.sync, a.tune.early_loads,
+                       phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks, (uint32_t)a.tune.realign, (uint32_t)a.tune.wave_runs);
+    return hipGetLastError();
+}
+
 template <class TR, int OP, int NT>
 inline hipError_t launch_fusion_phased(const FusionLaunchArgs& a, const FusionPtrs& own, const FusionPtrs& out,
                                        const PeerPtrs& pp, uint64_t i0, uint64_t i1, size_t t0) {
@@ -335,23 +564,27 @@ inline hipError_t launch_fusion_op(const FusionLaunchArgs& a) {
         for (size_t t = t0; t < t1; t++)
             if (!own.set(t - t0, a.own[t]) || !out.set(t - t0, a.out[t])) return hipErrorInvalidValue;   // not a device address
         hipError_t e = hipSuccess;
-        // large groups with three or more peers (from 320 MB of traffic by default, 480 MB with three peers): separate
+        // Large groups with three or more peers (from 320 MB of traffic by default, 480 MB with three peers): separate
         // reads from writes in time (at most 16 KiB of padding per item is over-counted).  With one or two peers the
-        // phased form measures 5-25 % below the streaming one at every size (its two vectors of so few inputs are
-        // too few loads in flight per lane), so it is only taken when forced.
+        // phased forms measure 5-25 % below the streaming one at every size, so they are only taken when forced.
+        // From five peers on the tiled kernel (32 KiB tiles, the inputs one after the other, tile descriptions off the
+        // critical path) is the faster phased form -- 7 peers: 256 tensors in the 256-byte layout 6.52 against 6.35
+        // TB/s, 400 even-sized tensors packed tightly 6.73-6.75 against 6.18-6.28, 400 odd-sized ones 6.47 against 5.79 --
+        // and with three and four the item kernel, which has all inputs of an item in flight at once (256 tensors, 3
+        // peers: 6.33 against 6.08; 400 tensors: level).
         const uint64_t traffic = (uint64_t)(a.n_peers + 2) * (i1 - i0) * kFusionChunk;
         const uint64_t from = (uint64_t)a.tune.phased_min_bytes * (a.n_peers == 3 ? 3u : 2u);
-        const bool phased = a.tune.sync && a.tune.num_cus >= kPhaseGroups && a.n_peers >= 1 && a.n_peers <= 7 &&
+        const bool phased = a.tune.sync && a.tune.num_cus >= kPhaseGroups && a.n_peers >= 1 &&
                             (a.tune.variant == 8 || (a.tune.variant == 0 && a.tune.max_blocks == 0 && a.n_peers >= 3 && traffic >= from));
-        if (phased) {
+        if (phased && a.n_peers >= 5) {
+            e = launch_fusion_tiled<TR, OP>(a, own, out, pp, t0, t1);
+        }
+        else if (phased) {
             switch (a.n_peers) {
                 case 1: e = launch_fusion_phased<TR, OP, 2>(a, own, out, pp, i0, i1, t0); break;
                 case 2: e = launch_fusion_phased<TR, OP, 3>(a, own, out, pp, i0, i1, t0); break;
                 case 3: e = launch_fusion_phased<TR, OP, 4>(a, own, out, pp, i0, i1, t0); break;
-                case 4: e = launch_fusion_phased<TR, OP, 5>(a, own, out, pp, i0, i1, t0); break;
-                case 5: e = launch_fusion_phased<TR, OP, 6>(a, own, out, pp, i0, i1, t0); break;
-                case 6: e = launch_fusion_phased<TR, OP, 7>(a, own, out, pp, i0, i1, t0); break;
-                default: e = launch_fusion_phased<TR, OP, 8>(a, own, out, pp, i0, i1, t0); break;
+                default: e = launch_fusion_phased<TR, OP, 5>(a, own, out, pp, i0, i1, t0); break;
             }
         }
         else {

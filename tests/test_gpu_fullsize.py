@@ -190,7 +190,7 @@ def test_c4_fusion_256_tensors_full_counts(comp):
     for i in range(256):
         assert (outs[i].cpu().numpy().view(np.uint16) == want[i]).all(), f"pack/reduce/unpack: tensor {i} of {counts[i]} elements"
     # fused single pass: the default choice at this size (phased) and the streaming kernel
-    for variant, kernel in ((0, "fusion_reduce_phased_kernel"), (2, "fusion_reduce_kernel")):
+    for variant, kernel in ((0, "fusion_reduce_tiled_kernel"), (2, "fusion_reduce_kernel")):
         comp.set_param("variant", variant)
         try:
             outs = [torch.zeros_like(t) for t in d_t]

@@ -221,11 +221,13 @@ def test_fusion_config_bf16_256_tensors(comp):
 @pytest.mark.parametrize("dtype,op,n_peers,lp,impl,align", [
     (O.BFLOAT16, O.SUM, 7, 1, 2, 256), (O.FLOAT16, O.MAX, 1, 0, 2, 256), (O.INT8, O.MIN, 7, 0, 2, 256),
     (O.FLOAT64, O.PROD, 2, 0, 2, 256), (O.BFLOAT16, O.SUM, 5, 0, 2, 1), (O.INT32, O.SUM, 8, 0, 2, 256),
-    (O.FLOAT32, O.MIN, 4, 0, 2, 16), (O.BFLOAT16, O.PROD, 3, 0, 1, 256)])
+    (O.FLOAT32, O.MIN, 4, 0, 2, 16), (O.BFLOAT16, O.PROD, 3, 0, 1, 256), (O.UINT8, O.SUM, 6, 0, 2, 1),
+    (O.FLOAT16, O.SUM, 16, 0, 2, 2), (O.BFLOAT16, O.SUM, 7, 1, 2, 1)])
 def test_fused_reduce_over_several_phases(comp, dtype, op, n_peers, lp, impl, align):
-    """The phased fused kernel with enough work that every LDS and register slot of a phase is used and a second
-    phase follows (a phase holds 22 items of 16 KiB per block: 92 MB chip-wide), for several element types,
-    operations and peer counts (more than 7 peers take the streaming kernel), against the oracle tensor by tensor."""
+    """The phased fused kernels with enough work that every LDS and register slot of a phase is used and a second
+    phase follows (a phase holds 92 MB chip-wide), for several element types, operations and peer counts -- up to four
+    peers the item kernel (16 KiB items, all inputs of an item in flight), from five the tiled kernel (32 KiB tiles,
+    the inputs one after the other, any number of peers) -- against the oracle tensor by tensor."""
     import torch
     rng = np.random.default_rng(900 + dtype * 8 + n_peers)
     esz = O.DTYPE_SIZE[dtype]
@@ -242,7 +244,9 @@ def test_fused_reduce_over_several_phases(comp, dtype, op, n_peers, lp, impl, al
     peers = [make_inputs(rng, dtype, nelem, op, 1)[0] for _ in range(n_peers)]
     d_t = [to_dev(t) for t in tensors]
     d_p = [to_dev(p) for p in peers]
-    outs = [to_dev(np.zeros(c + 4, np_t)) for c in counts]
+    outs = [to_dev(np.zeros(c + 6, np_t)) for c in counts]
+    sh = [i % 3 for i in range(k)]                       # every third output on its holder's boundary, the others 1 and 2 elements off
+    views = [o[s_:s_ + c] for o, s_, c in zip(outs, sh, counts)]
     want = []
     for i, c in enumerate(counts):
         o = int(offs[i]) // esz
@@ -255,14 +259,15 @@ def test_fused_reduce_over_several_phases(comp, dtype, op, n_peers, lp, impl, al
         comp.set_param("phase_early_loads", loads)
         comp.set_param("phase_early_stores", stores)
         try:
-            plan.reduce(op, d_t, d_p, outs, lp_mode=lp, bf16_impl=impl)
+            plan.reduce(op, d_t, d_p, views, lp_mode=lp, bf16_impl=impl)
             torch.cuda.synchronize()
+            assert comp.last_kernel() == ("fusion_reduce_tiled_kernel" if n_peers >= 5 else "fusion_reduce_phased_kernel")
         finally:
             comp.set_param("variant", 0)
             comp.set_param("phase_early_loads", 12)
             comp.set_param("phase_early_stores", -1)
         for i, c in enumerate(counts):
             g = to_host(outs[i], np_t)
-            assert_same(g[:c], want[i], dtype, f"tensor {i} of {c} elements, early loads {loads} stores {stores}")
-            assert not g[c:].view(np.uint8).any(), "wrote past the tensor"
+            assert_same(g[sh[i]:sh[i] + c], want[i], dtype, f"tensor {i} of {c} elements, early loads {loads} stores {stores}")
+            assert not g[:sh[i]].view(np.uint8).any() and not g[sh[i] + c:].view(np.uint8).any(), "wrote outside the tensor"
     plan.close()
