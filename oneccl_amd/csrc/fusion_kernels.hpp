@@ -4,9 +4,10 @@
 // optionally rounded up to an alignment.
 //
 // Work is cut into items of kFusionChunk bytes of one tensor; a block of the fused reduce takes items grid-stride
-// (a block of pack / unpack takes a quarter of one item).  The item list and the per-tensor offset/size tables live in
-// device memory owned by the plan; the tensor pointers of a call travel as kernel arguments: kFusionGroup tensors
-// per launch of the fused reduce (two tables: inputs and outputs), more for pack and unpack (one table).
+// (a block of pack / unpack takes a quarter of one item; the tiled form of the fused reduce takes tiles of two items'
+// size).  The item list and the per-tensor offset, size and tile-count tables live in device memory owned by the
+// plan; the tensor pointers of a call travel as kernel arguments: kFusionGroup tensors per launch of the fused
+// reduce (two tables: inputs and outputs), more for pack and unpack (one table).
 #pragma once
 
 #include "batch_kernels.hpp"
