@@ -50,6 +50,60 @@ def test_graph_capture_and_replay(comp, variant):
         comp.set_param("variant", 0)
 
 
+def test_graph_of_the_paced_and_the_tiled_phased_kernels(comp):
+    """The phased reduce with several destinations (its write phase is let out by the device clock) and the fused
+    reduce against six peers (the tiled phased kernel, whose lanes describe the tiles of the next phase while the block
+    waits at a barrier), forced on at a few MB, captured together and replayed four times with eager work in between."""
+    import torch
+    rng = np.random.default_rng(77)
+    count, n, m = 2_000_003, 3, 3
+    srcs = [O.bf16_from_f32(rng.standard_normal(count).astype(np.float32)) for _ in range(n)]
+    want = O.reduce_n(srcs, O.BFLOAT16, O.SUM, keep=1, threads=8)
+    d = [to_dev(s) for s in srcs]
+    outs = [torch.zeros_like(d[0]) for _ in range(m)]
+    counts = [700_001, 5, 1_200_000, 99_997]
+    plan = comp.FusionPlan(counts, comp.BFLOAT16, 1)
+    tens_h = [O.bf16_from_f32(rng.standard_normal(c).astype(np.float32)) for c in counts]
+    peers_h = [O.bf16_from_f32(rng.standard_normal(plan.nbytes // 2).astype(np.float32)) for _ in range(6)]
+    tens, peers = [to_dev(t) for t in tens_h], [to_dev(p_) for p_ in peers_h]
+    res = [torch.zeros(c, dtype=tens[0].dtype, device="cuda") for c in counts]
+    offs, _ = O.fusion_offsets(counts, 2, 1)
+    want_res = [O.reduce_n([tens_h[t]] + [p_[offs[t] // 2:offs[t] // 2 + c] for p_ in peers_h], O.BFLOAT16, O.SUM, keep=1)
+                for t, c in enumerate(counts)]
+
+    def both():
+        comp.comp_reduce_write_n(comp.BFLOAT16, comp.SUM, d, outs, count, lp_mode=comp.LP_KEEP_PRECISION)
+        k1 = comp.last_kernel()
+        plan.reduce(comp.SUM, tens, peers, res, lp_mode=comp.LP_KEEP_PRECISION)
+        return k1, comp.last_kernel()
+
+    def check(tag):
+        torch.cuda.synchronize()
+        for o_ in outs:
+            assert (to_host(o_, np.uint16) == want).all(), tag
+        for r_, w_ in zip(res, want_res):
+            assert (to_host(r_, np.uint16) == w_).all(), tag
+
+    comp.set_param("variant", 8)
+    try:
+        assert both() == ("reduce_multi_phased_kernel", "fusion_reduce_tiled_kernel")
+        check("eager")
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            both()
+        for rep in range(4):
+            for t_ in outs + res:
+                t_.fill_(0)
+            torch.cuda.synchronize()
+            g.replay()
+            check(f"replay {rep}")
+            both()                          # an eager pair between the replays
+            check(f"eager after replay {rep}")
+    finally:
+        comp.set_param("variant", 0)
+        plan.close()
+
+
 def test_graph_of_copy_broadcast_converters_and_fused_reduce(comp):
     """A pipeline of the other kernels in one captured graph -- widen bf16 to fp32, copy, narrow back, broadcast to
     three buffers, fused reduce of two tensors against two peer fusion buffers -- replayed four times with eager work
