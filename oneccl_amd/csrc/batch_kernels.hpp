@@ -97,9 +97,9 @@ reduce_batch_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tiles) {
 // of kBatchPhaseTile vectors (32 KiB of every buffer of ONE job: four vectors per lane of a block, the group that
 // reduce_multi_phased_kernel keeps in flight per input; a job's last tile is padded), and the tiles are dealt out as
 // that kernel deals out its groups: group q of block b in a phase is tile (phase x 11 + q) x grid + b, so that at every
-// step the chip reads `grid` consecutive tiles.  A block's tiles of one phase ascend, so the job of a tile is found
-// by moving a cursor along the running tile counts (scalar work on kernel arguments) from a binary search for the
-// phase's first tile.  Staging (registers and LDS), barrier, early arrival and arithmetic are those of
+// step the chip reads `grid` consecutive tiles.  Which job a tile belongs to, and where in it the tile starts, is
+// worked out by lane q of every wave for the block's q-th tile of a phase (batch_describe), ahead of the phase.
+// Staging (registers and LDS), barrier, early arrival and arithmetic are those of
 // reduce_multi_phased_kernel; the jobs' edge elements are computed after the last phase, job j by block j mod grid.
 constexpr int kBatchPhaseG = 4;
 constexpr uint64_t kBatchPhaseTile = (uint64_t)kBatchPhaseG * kPhaseBlock;
