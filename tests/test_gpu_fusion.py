@@ -225,7 +225,7 @@ def test_fusion_config_bf16_256_tensors(comp):
     (O.FLOAT16, O.SUM, 16, 0, 2, 2), (O.BFLOAT16, O.SUM, 7, 1, 2, 1)])
 def test_fused_reduce_over_several_phases(comp, dtype, op, n_peers, lp, impl, align):
     """The phased fused kernels with enough work that every LDS and register slot of a phase is used and a second
-    phase follows (a phase holds 92 MB chip-wide), for several element types, operations and peer counts -- up to four
+    phase follows (a phase holds 92 MB chip-wide in the item kernel, 101 MB in the tiled one), for several element types, operations and peer counts -- up to four
     peers the item kernel (16 KiB items, all inputs of an item in flight), from five the tiled kernel (32 KiB tiles,
     the inputs one after the other, any number of peers) -- against the oracle tensor by tensor."""
     import torch
