@@ -392,7 +392,7 @@ inline hipError_t launch_batch_op(const BatchLaunchArgs& a) {
                     off_lines |= (uint32_t)((uintptr_t)tb.p[q * (a.n + 1) + k] + split[q].head * sizeof(E)) & (kLineBytes - 1);
         }
         const uint32_t wave_runs = a.tune.wave_runs == 2 || (a.tune.wave_runs == 1 && off_lines);
-        const uint32_t write_pace16 = a.n == 2 ? write_pace_ticks16(phase_grid * kBatchPhaseTile * 16u, 1.1 * (double)a.tune.write_pace, a.tune.wall_khz) : 0u;
+        const uint32_t write_pace16 = a.n >= 2 && a.n <= PhasePacedInputs<TR, OP>::value ? write_pace_ticks16(phase_grid * kBatchPhaseTile * 16u, 1.1 * (double)a.tune.write_pace, a.tune.wall_khz) : 0u;
         j0 += nj;
         if (tiles == 0) continue;
         g_realigned_launches += realigned;

@@ -149,7 +149,7 @@ template <class TR, int OP, int NT>
 __global__ void __launch_bounds__(kPhaseBlock)
 fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, const uint64_t* off, const uint64_t* bytes,
                             const FusionItem* items, uint32_t nitems, uint32_t t0, PhaseSync* ps, int early_loads,
-                            int early_stores, long spin_ticks, uint32_t realign, uint32_t wave_runs) {
+                            int early_stores, long spin_ticks, uint32_t realign, uint32_t wave_runs, uint32_t write_pace16) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr uint32_t ES = sizeof(E);
@@ -270,6 +270,9 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
         const int lead_w = early_stores / 2;
         const int arrive_w = nslots > lead_w ? nslots - lead_w : 0;
         arrived = false;
+        // the clock paces the items' stores as it does in reduce_multi_phased_kernel (write_pace16: 1/16 ticks per item
+        // of the whole grid; 0: unpaced)
+        uint64_t pace_next16 = write_pace16 ? (uint64_t)wall_clock64() << 4 : 0;
         for (int k = 0; k < SLOTS; k++) {
             if (more && lead_w > 0 && k == arrive_w) {
                 if (tid == 0) phase_arrive(ps);
@@ -277,6 +280,10 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
             }
             const uint32_t nb = __shfl(d_nb, k, 64);
             if (nb == 0) break;
+            if (write_pace16) {
+                while (((uint64_t)wall_clock64() << 4) < pace_next16) __builtin_amdgcn_s_sleep(1);
+                pace_next16 += write_pace16;
+            }
             unsigned char* o = (unsigned char*)(uintptr_t)__shfl(d_o, k, 64);
             {
                 const uint32_t nelem = nb / ES;
@@ -423,7 +430,7 @@ __global__ void __launch_bounds__(kPhaseBlock)
 fusion_reduce_tiled_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n_peers, const uint64_t* off,
                            const uint64_t* bytes, const uint32_t* tile_end, uint32_t t0, uint32_t nt, uint32_t tile_base,
                            uint32_t ntiles, PhaseSync* ps, int early_loads, int early_stores, long spin_ticks,
-                           uint32_t realign, uint32_t wave_runs) {
+                           uint32_t realign, uint32_t wave_runs, uint32_t write_pace16) {
     typedef typename TR::elem_t E;
     kernel_prologue<TR, OP>();
     constexpr uint32_t ES = sizeof(E);
@@ -479,9 +486,19 @@ fusion_reduce_tiled_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n
         phase_wait(ps, ++gen, give_up, spin_ticks);
         const bool more = np < ntiles;
         const int arrive_u = more ? kPhaseU - early_stores : -1;    // kPhaseU: after the last store
+        // the clock paces the tiles' stores as it does in reduce_multi_phased_kernel (write_pace16: 1/16 ticks per tile
+        // of the whole grid; 0: unpaced)
+        uint64_t pace_next16 = write_pace16 ? (uint64_t)wall_clock64() << 4 : 0;
+        auto paced = [&](bool valid) {
+            if (write_pace16 && valid) {
+                while (((uint64_t)wall_clock64() << 4) < pace_next16) __builtin_amdgcn_s_sleep(1);
+                pace_next16 += write_pace16;
+            }
+        };
 #pragma unroll
         for (int q = 0; q < RG; q++) {
             const FusionSlot s = fusion_slot<TR>(desc, q, wave_runs);
+            paced(s.nb != 0);
             u32x4_u* d = (u32x4_u*)(s.o + s.head * ES);
 #pragma unroll
             for (int g = 0; g < G; g++) {
@@ -491,6 +508,7 @@ fusion_reduce_tiled_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n
         }
         for (int q = 0; q < LG; q++) {
             const FusionSlot s = fusion_slot<TR>(desc, RG + q, wave_runs);
+            paced(s.nb != 0);
             u32x4_u* d = (u32x4_u*)(s.o + s.head * ES);
 #pragma unroll
             for (int g = 0; g < G; g++) {
@@ -530,6 +548,15 @@ fusion_reduce_tiled_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n
     }
 }
 
+// The write phase's pace for the phased fused kernels, in 1/16 clock ticks per `stores` stores of 16 bytes per lane of
+// the whole grid (a tile: 4, an item: 2): 1.1 x Tuning::write_pace while own buffer and peers together are few enough
+// inputs for the type (PhasePacedInputs), else unpaced.
+template <class TR, int OP>
+inline uint32_t fusion_write_pace16(const FusionLaunchArgs& a, int grid, int stores) {
+    if (a.n_peers < 1 || a.n_peers + 1 > PhasePacedInputs<TR, OP>::value) return 0;
+    return write_pace_ticks16((uint64_t)grid * kPhaseBlock * 16u * (uint32_t)stores, 1.1 * (double)a.tune.write_pace, a.tune.wall_khz);
+}
+
 template <class TR, int OP>
 inline hipError_t launch_fusion_tiled(const FusionLaunchArgs& a, const FusionPtrs& own, const FusionPtrs& out,
                                       const PeerPtrs& pp, size_t t0, size_t t1) {
@@ -538,7 +565,8 @@ inline hipError_t launch_fusion_tiled(const FusionLaunchArgs& a, const FusionPtr
     hipLaunchKernelGGL((fusion_reduce_tiled_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, own, out, pp, a.n_peers,
                        a.d_off, a.d_bytes, a.d_tile_end, (uint32_t)t0, (uint32_t)(t1 - t0), (uint32_t)a.tile_begin[t0],
                        (uint32_t)(a.tile_begin[t1] - a.tile_begin[t0]), a.tune.sync, a.tune.early_loads,
-                       phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks, (uint32_t)a.tune.realign, (uint32_t)a.tune.wave_runs);
+                       phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks, (uint32_t)a.tune.realign, (uint32_t)a.tune.wave_runs,
+                       fusion_write_pace16<TR, OP>(a, grid, 4));
     return hipGetLastError();
 }
 
@@ -550,7 +578,7 @@ inline hipError_t launch_fusion_phased(const FusionLaunchArgs& a, const FusionPt
     hipLaunchKernelGGL((fusion_reduce_phased_kernel<TR, OP, NT>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, own, out, pp,
                        a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0, a.tune.sync,
                        a.tune.early_loads, phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks, (uint32_t)a.tune.realign,
-                       (uint32_t)a.tune.wave_runs);
+                       (uint32_t)a.tune.wave_runs, fusion_write_pace16<TR, OP>(a, grid, 2));
     return hipGetLastError();
 }
 
@@ -567,18 +595,21 @@ inline hipError_t launch_fusion_op(const FusionLaunchArgs& a) {
         for (size_t t = t0; t < t1; t++)
             if (!own.set(t - t0, a.own[t]) || !out.set(t - t0, a.out[t])) return hipErrorInvalidValue;   // not a device address
         hipError_t e = hipSuccess;
-        // Large groups with three or more peers (from 320 MB of traffic by default, 480 MB with three peers): separate
-        // reads from writes in time (at most 16 KiB of padding per item is over-counted).  With one or two peers the
-        // phased forms measure 5-25 % below the streaming one at every size, so they are only taken when forced.
+        // Large groups with two or more peers (from 320 MB of traffic by default, 480 MB with three peers, 960 MB with
+        // two): separate reads from writes in time (at most 16 KiB of padding per item is over-counted).  With two
+        // peers and 1.07 GB of traffic the phased item kernel, its write phase paced, measures 6.61-6.66 against
+        // 5.96-6.16 TB/s for the 32- and 64-bit types, 6.47-6.57 against 5.92-6.04 for fp16, 6.38-6.40 against 5.99-6.12
+        // for the 8-bit ones and 6.24-6.27 against 6.04-6.17 for bfloat16; at half of that bfloat16 loses 4 %.  With one
+        // peer the phased forms measure 2-20 % below the streaming one at every size and are only taken when forced.
         // From five peers on the tiled kernel (32 KiB tiles, the inputs one after the other, tile descriptions off the
         // critical path) is the faster phased form -- 7 peers: 256 tensors in the 256-byte layout 6.52 against 6.35
         // TB/s, 400 even-sized tensors packed tightly 6.73-6.75 against 6.18-6.28, 400 odd-sized ones 6.47 against 5.79 --
         // and with three and four the item kernel, which has all inputs of an item in flight at once (256 tensors, 3
         // peers: 6.33 against 6.08; 400 tensors: level).
         const uint64_t traffic = (uint64_t)(a.n_peers + 2) * (i1 - i0) * kFusionChunk;
-        const uint64_t from = (uint64_t)a.tune.phased_min_bytes * (a.n_peers == 3 ? 3u : 2u);
+        const uint64_t from = (uint64_t)a.tune.phased_min_bytes * (a.n_peers == 2 ? 6u : a.n_peers == 3 ? 3u : 2u);
         const bool phased = a.tune.sync && a.tune.num_cus >= kPhaseGroups && a.n_peers >= 1 &&
-                            (a.tune.variant == 8 || (a.tune.variant == 0 && a.tune.max_blocks == 0 && a.n_peers >= 3 && traffic >= from));
+                            (a.tune.variant == 8 || (a.tune.variant == 0 && a.tune.max_blocks == 0 && a.n_peers >= 2 && traffic >= from));
         if (phased && a.n_peers >= 5) {
             e = launch_fusion_tiled<TR, OP>(a, own, out, pp, t0, t1);
         }

@@ -937,6 +937,30 @@ constexpr int kPhaseEarlyStores = 16;
 // at 1 GiB: 5.78 TB/s with 4 stores early against 6.25 with a strict report, 6.45 with the meeting and 16 early).  When
 // the clock paces the write phase (Tuning::write_pace) the last destination's 20 LDS-staged stores all come after the
 // report: 6.98 against 6.94 with 16.
+// Up to how many inputs a reduce to ONE destination has its write phase paced by the clock (see the kernel), at 1.1 x
+// Tuning::write_pace.  The shorter the read phase, the more it pays to start it with the chip's blocks in step;
+// measured at 512 MiB per buffer against the unpaced kernel, every operation: 3 inputs +2.0-2.9 %, 4 inputs +1.2-2.3 %,
+// 6 inputs +0.7-1.4 %, 8 inputs +0.1-1.1 %, 12 inputs -0.8..+0.7 % for the 16-bit integers, the 32- and 64-bit types
+// and fp16 sum / prod.  Where the read phase carries more arithmetic per byte it gains less and then loses: the 8-bit
+// types and fp16 min / max +1.3-2.8 % with 3 inputs, +0.2-0.7 % with 4, -0.2..-1.5 % from 6 on; both bfloat16 families
+// +-0.6 % with 3 and 4, -0.6..-2.0 % from 6 on (with 2 inputs every type gains: +1-4 %).
+template <class TR, int OP>
+struct PhasePacedInputs {
+    static constexpr int value = sizeof(typename TR::elem_t) == 1 ? 4 : 8;
+};
+template <bool RNE, bool VEC_SEM, int OP>
+struct PhasePacedInputs<Bf16PairwiseTraits<RNE, VEC_SEM>, OP> {
+    static constexpr int value = 3;
+};
+template <bool RNE, int OP>
+struct PhasePacedInputs<Bf16KeepTraits<RNE>, OP> {
+    static constexpr int value = 3;
+};
+template <bool NATIVE, int OP>
+struct PhasePacedInputs<Fp16Traits<NATIVE>, OP> {
+    static constexpr int value = (OP == OP_MIN || OP == OP_MAX) ? 4 : 8;
+};
+
 template <class TR>
 inline int phase_early_stores(const Tuning& t, int n_dsts) {
     const int v = t.early_stores >= 0 ? t.early_stores : n_dsts >= 2 ? (t.write_pace > 0 ? kPhaseU : 16) : kPhaseEarlyStores;
@@ -1205,11 +1229,11 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
         const uint32_t wave_runs = a.tune.wave_runs == 2 || (a.tune.wave_runs == 1 && off_lines && a.m == 1);
         // the write phase's pace (see the kernel): 1/16 clock ticks per group of four stores of the whole grid
         uint32_t write_pace16 = 0;
-        // Two inputs to one destination are paced too, a tenth faster (their write phase is a third of the traffic, but
-        // short: 2 GiB per buffer fp32 6.82-6.93 against 6.59-6.70 TB/s, bf16 6.63-6.70 against 6.56-6.59; best at
-        // 1.1 x the pace either way); from three inputs on one destination gains nothing (7.03-7.04 against 7.10 for
-        // eight) and stays unpaced.
-        const double rate = a.m >= 2 ? (double)a.tune.write_pace : a.n == 2 ? 1.1 * (double)a.tune.write_pace : 0.0;
+        // Several destinations at the pace itself; one destination a tenth faster (its write phase is short) while the
+        // inputs are few enough for the type (PhasePacedInputs).
+        const double rate = a.m >= 2                              ? (double)a.tune.write_pace
+                            : a.n <= PhasePacedInputs<TR, OP>::value ? 1.1 * (double)a.tune.write_pace
+                                                                      : 0.0;
         write_pace16 = write_pace_ticks16((uint64_t)grid * kPhaseBlock * 16u * 4u, rate, a.tune.wall_khz);
         g_last_kernel = "reduce_multi_phased_kernel";
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,

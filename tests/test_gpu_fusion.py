@@ -251,13 +251,15 @@ def test_fused_reduce_over_several_phases(comp, dtype, op, n_peers, lp, impl, al
     for i, c in enumerate(counts):
         o = int(offs[i]) // esz
         want.append(O.reduce_n([tensors[i]] + [p[o:o + c] for p in peers], dtype, op, keep=lp, bf16_impl=impl))
-    # the default, then other points at which a block reports its arrival at the barrier: timing only, same bits
-    for loads, stores in ((12, -1), (0, 0), (4096, 20), (40, 3)):
+    # the default, then other points at which a block reports its arrival at the barrier and other paces of the write
+    # phase (which only few enough inputs for the type take): timing only, same bits
+    for loads, stores, pace in ((12, -1, 7300), (0, 0, 0), (4096, 20, 30000), (40, 3, 400)):
         for o in outs:
             o.zero_()
         comp.set_param("variant", 8)
         comp.set_param("phase_early_loads", loads)
         comp.set_param("phase_early_stores", stores)
+        comp.set_param("phase_write_pace", pace)
         try:
             plan.reduce(op, d_t, d_p, views, lp_mode=lp, bf16_impl=impl)
             torch.cuda.synchronize()
@@ -266,8 +268,41 @@ def test_fused_reduce_over_several_phases(comp, dtype, op, n_peers, lp, impl, al
             comp.set_param("variant", 0)
             comp.set_param("phase_early_loads", 12)
             comp.set_param("phase_early_stores", -1)
+            comp.set_param("phase_write_pace", 7300)
         for i, c in enumerate(counts):
             g = to_host(outs[i], np_t)
-            assert_same(g[sh[i]:sh[i] + c], want[i], dtype, f"tensor {i} of {c} elements, early loads {loads} stores {stores}")
+            assert_same(g[sh[i]:sh[i] + c], want[i], dtype, f"tensor {i} of {c} elements, early loads {loads} stores {stores} pace {pace}")
             assert not g[:sh[i]].view(np.uint8).any() and not g[sh[i] + c:].view(np.uint8).any(), "wrote outside the tensor"
     plan.close()
+
+
+
+@pytest.mark.parametrize("dtype,op,lp,align", [(O.FLOAT32, O.SUM, 0, 256), (O.BFLOAT16, O.SUM, 1, 1)])
+def test_fused_reduce_with_two_peers_takes_the_phased_kernel_when_large(comp, dtype, op, lp, align):
+    """Two peers: the streaming kernel below 960 MB of traffic, the phased item kernel (write phase paced by the clock)
+    from there; the same bits either way, against the oracle tensor by tensor."""
+    import torch
+    rng = np.random.default_rng(77 + dtype)
+    esz = O.DTYPE_SIZE[dtype]
+    np_t = O.NP_STORAGE[dtype]
+    for target, kernel in ((300 << 20, "fusion_reduce_phased_kernel"), (100 << 20, "fusion_reduce_kernel")):
+        k = 23
+        w = rng.random(k) ** 2 + 0.01
+        counts = [max(1, int(target * x / w.sum()) // esz + int(rng.integers(0, 5))) for x in w]
+        plan = comp.FusionPlan(counts, dtype, align)
+        offs, total = O.fusion_offsets(counts, esz, align)
+        nelem = (total + esz - 1) // esz
+        tensors = [make_inputs(rng, dtype, c, op, 1)[0] for c in counts]
+        peers = [make_inputs(rng, dtype, nelem, op, 1)[0] for _ in range(2)]
+        d_t = [to_dev(t) for t in tensors]
+        d_p = [to_dev(p) for p in peers]
+        outs = [to_dev(np.zeros(c, np_t)) for c in counts]
+        plan.reduce(op, d_t, d_p, outs, lp_mode=lp)
+        torch.cuda.synchronize()
+        assert comp.last_kernel() == kernel
+        for i, c in enumerate(counts):
+            o = int(offs[i]) // esz
+            want = O.reduce_n([tensors[i]] + [p[o:o + c] for p in peers], dtype, op, keep=lp)
+            assert_same(to_host(outs[i], np_t), want, dtype, f"tensor {i} of {c} elements, {kernel}")
+        plan.close()
+        del d_t, d_p, outs

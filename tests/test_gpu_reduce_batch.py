@@ -124,12 +124,17 @@ def test_chunk_sized_jobs_take_the_phased_form(comp):
     assert comp.last_kernel() == "reduce_batch_phased_kernel"
     _run(comp, rng, O.BFLOAT16, O.SUM, 2, [(48 << 20) // 2] * 7, in_place_every=0)
     assert comp.last_kernel() == "reduce_batch_phased_kernel"
-    # jobs of two inputs have their write phase paced by the device clock: unpaced, a pace no store keeps up with and
-    # one that every group of stores waits for give the same bits, with jobs that end inside a tile and in place
+    # jobs of few enough inputs for their type (two for every type, up to eight for the 32-bit ones) have their write
+    # phase paced by the device clock: unpaced, a pace no store keeps up with and one that every group of stores waits
+    # for give the same bits, with jobs that end inside a tile and in place
     try:
         for pace in (0, 100_000, 2000):
             comp.set_param("phase_write_pace", pace)
             _run(comp, rng, O.FLOAT32, O.SUM, 2, [(6 << 20) // 4 + 5 * j for j in range(40)], in_place_every=3)
+            assert comp.last_kernel() == "reduce_batch_phased_kernel"
+            _run(comp, rng, O.UINT32, O.MAX, 5, [(3 << 20) // 4 + 3 * j for j in range(40)], in_place_every=4)
+            assert comp.last_kernel() == "reduce_batch_phased_kernel"
+            _run(comp, rng, O.BFLOAT16, O.SUM, 3, [(5 << 20) // 2 + j for j in range(40)], lp=comp.LP_KEEP_PRECISION, keep=1)
             assert comp.last_kernel() == "reduce_batch_phased_kernel"
     finally:
         comp.set_param("phase_write_pace", 7300)

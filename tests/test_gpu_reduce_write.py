@@ -168,8 +168,8 @@ def test_phased_form_over_several_phases(comp):
 
 
 def test_write_phase_paced_by_the_clock(comp):
-    """With two or more destinations (and with two inputs to one) the device clock lets the write phase's stores out at a set rate
-    ("phase_write_pace", GB/s).  Timing only: unpaced, the default, a pace far below what HBM takes (every group of
+    """With two or more destinations (and with few enough inputs for their type to one: two for every type, up to
+    eight for most) the device clock lets the write phase's stores out at a set rate ("phase_write_pace", GB/s).  Timing only: unpaced, the default, a pace far below what HBM takes (every group of
     stores waits for the clock), one far above (none does) and the largest value all give the oracle's bits, over
     several phases, with the destinations at different alignments, one of them aliasing an input."""
     import torch
@@ -178,7 +178,8 @@ def test_write_phase_paced_by_the_clock(comp):
     comp.set_param("variant", 8)
     try:
         for dtype, n, m, count in [(O.BFLOAT16, 3, 3, 70_000_003), (O.FLOAT32, 2, 2, 40_000_001), (O.INT8, 4, 5, 1_000_003),
-                                   (O.FLOAT32, 2, 1, 50_000_001), (O.BFLOAT16, 2, 1, 100_000_007)]:     # two inputs to one (in place) are paced too
+                                   (O.FLOAT32, 2, 1, 50_000_001), (O.BFLOAT16, 2, 1, 100_000_007),      # two inputs to one (in place) are paced too,
+                                   (O.INT64, 7, 1, 20_000_003), (O.UINT8, 4, 1, 150_000_001), (O.FLOAT16, 8, 1, 60_000_001)]:   # and up to eight
             np_t, esz = O.NP_STORAGE[dtype], O.DTYPE_SIZE[dtype]
             keep = 1 if dtype == O.BFLOAT16 else 0
             srcs = make_inputs(rng, dtype, count, O.SUM, n)
