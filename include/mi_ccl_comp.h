@@ -263,8 +263,9 @@ const char* mi_ccl_last_kernel(void);
  * (0/1, default 1: a reduce, copy or broadcast of 1 MiB or more per buffer starts its 16-byte vectors on a 128-byte
  * line of the buffers that matter most -- the outputs before the inputs -- so up to 127 bytes at the front are
  * handled element by element; buffers that share an offset from the lines then run like aligned ones, +6 %) and
- * "phase_write_pace" (phased reduce with two or more destinations, and, a tenth faster, with two inputs and one
- * destination, batched jobs of two inputs included: the rate in GB/s at which the device clock lets
+ * "phase_write_pace" (phased reduce with two or more destinations, and, a tenth faster, with one destination and few
+ * enough inputs for the element type -- 8; 4 for the 8-bit types and fp16 min / max; 3 for bfloat16 -- batched jobs
+ * and the phased fused reduces included, where it gains 1-4 %: the rate in GB/s at which the device clock lets
  * the write phase's stores out, which keeps the blocks of the chip in step and the addresses written at any moment in
  * one compact window; default 7300, 0 = unpaced, otherwise 100 to 100000; 8 inputs stored to 8 buffers of 1 GiB run at 6.95 TB/s paced and 6.4
  * unpaced; a block that is behind the schedule is never held, so a rate above what HBM takes only switches the
