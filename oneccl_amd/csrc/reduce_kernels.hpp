@@ -60,7 +60,7 @@ struct Tuning {
     int realign;             // 1: inputs off a 4-byte boundary are read on that boundary and realigned in registers
     int line_start;          // 1: large calls start their vectors on a 128-byte line of the buffers that matter most
     int wave_runs;           // phased kernels: a wave's vectors of a group lie next to each other; 0 never, 1 when a buffer is off the lines, 2 always
-    int write_pace;          // phased reduce with several destinations: the rate, in GB/s, at which the clock lets the write phase's stores out (0: unpaced)
+    int write_pace;          // phased kernels: the rate, in GB/s, at which the clock lets the write phase's stores out (0: unpaced)
     int wall_khz;            // what wall_clock64() counts, in kHz
 };
 
@@ -1042,8 +1042,9 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
         // over the chip) not before the phase's start + i * write_pace16 / 16 ticks, a little faster than HBM takes them.
         // Every block reads the same clock, so the blocks stay within a fraction of a group of each other without
         // exchanging a word; a block that is behind the schedule is never held.  8 -> 8 at 1 GiB: 6.95 against 6.40
-        // TB/s, 4 -> 4: 6.90 against 6.35, 2 -> 2: 6.63 against 6.30.  With one destination (44 stores per lane) and three
-        // or more inputs there is nothing to gain: 7.04 against 7.10.
+        // TB/s, 4 -> 4: 6.90 against 6.35, 2 -> 2: 6.63 against 6.30.  With one destination (44 stores per lane) a pace
+        // a tenth faster keeps the blocks in step for the read phase that follows, which pays while that is short
+        // (PhasePacedInputs).
         uint64_t pace_next16 = write_pace16 ? (uint64_t)wall_clock64() << 4 : 0;
         auto paced = [&](int u) {       // u: slot within the phase; groups that lie behind the end of the data take no time
             if (write_pace16 && (u & 3) == 0 && p0 + (uint64_t)u * gthreads < nvec) {
