@@ -248,7 +248,8 @@ const char* mi_ccl_last_kernel(void);
  * "phased_min_bytes" (scales the sizes from which the phased kernels are used; default 160 MB),
  * "phase_early_loads" / "phase_early_stores" (phased kernels: how many 16-byte loads / stores per lane a block still
  * has to issue when it reports the end of its read / write phase to the chip-wide barrier, which hides the barrier's
- * latency; defaults 12 and -1 = 16, or 20 with several destinations while the write phase is paced; 0 = report
+ * latency; defaults -1 = 12 loads, or 2 to 8 behind a paced write phase depending on the element type and the number
+ * of inputs, and -1 = 16 stores, or 20 with several destinations while the write phase is paced; 0 = report
  * when the whole block is done and its stores are acknowledged; timing only, results do not
  * depend on them), "phase_spin_ticks" (phased kernels: the longest a block waits at one barrier, in 100 MHz ticks,
  * before it goes on alone and stops waiting for the rest of the launch; default 20000 = 200 us; 0 = never wait, which
@@ -263,9 +264,9 @@ const char* mi_ccl_last_kernel(void);
  * (0/1, default 1: a reduce, copy or broadcast of 1 MiB or more per buffer starts its 16-byte vectors on a 128-byte
  * line of the buffers that matter most -- the outputs before the inputs -- so up to 127 bytes at the front are
  * handled element by element; buffers that share an offset from the lines then run like aligned ones, +6 %) and
- * "phase_write_pace" (phased reduce with two or more destinations, and, a tenth faster, with one destination and few
- * enough inputs for the element type -- 8; 4 for the 8-bit types and fp16 min / max; 3 for bfloat16 -- batched jobs
- * and the phased fused reduces included, where it gains 1-4 %: the rate in GB/s at which the device clock lets
+ * "phase_write_pace" (phased reduce with two or more destinations, and, a tenth faster, with one destination and up
+ * to 16 inputs -- 12 for the 8-bit types, bfloat16 and fp16 min / max -- batched jobs and the phased fused reduces
+ * included, where it gains 1-6 %: the rate in GB/s at which the device clock lets
  * the write phase's stores out, which keeps the blocks of the chip in step and the addresses written at any moment in
  * one compact window; default 7300, 0 = unpaced, otherwise 100 to 100000; 8 inputs stored to 8 buffers of 1 GiB run at 6.95 TB/s paced and 6.4
  * unpaced; a block that is behind the schedule is never held, so a rate above what HBM takes only switches the

@@ -399,7 +399,7 @@ inline hipError_t launch_batch_op(const BatchLaunchArgs& a) {
         if (phased) {
             g_last_kernel = "reduce_batch_phased_kernel";
             hipLaunchKernelGGL((reduce_batch_phased_kernel<TR, OP>), dim3((unsigned)phase_grid), dim3(kPhaseBlock), 0, a.stream, tb, a.n,
-                               nj, (uint32_t)tiles, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks,
+                               nj, (uint32_t)tiles, a.tune.sync, phase_early_loads<TR, OP>(a.tune, a.n, write_pace16 != 0), phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks,
                                wave_runs, write_pace16);
         }
         else {

@@ -50,7 +50,7 @@ static std::atomic<int> g_max_blocks{ 0 };
 static std::atomic<int> g_xcd_chunked{ 0 };
 static std::atomic<int> g_variant{ 0 };
 static std::atomic<long> g_phased_min_bytes{ 160L << 20 };
-static std::atomic<int> g_phase_early_loads{ 12 };
+static std::atomic<int> g_phase_early_loads{ -1 };
 static std::atomic<int> g_phase_early_stores{ -1 };
 static std::atomic<long> g_phase_spin_ticks{ kPhaseSpinTicks };
 static std::atomic<int> g_fp16_impl{ MI_CCL_FP16_AVX512F };
@@ -882,7 +882,7 @@ int mi_ccl_set_param(const char* name, long value) {
         g_phased_min_bytes.store(value);
         return MI_CCL_SUCCESS;
     }
-    if (!strcmp(name, "phase_early_loads") && value >= 0 && value <= 4096) {
+    if (!strcmp(name, "phase_early_loads") && value >= -1 && value <= 4096) {
         g_phase_early_loads.store((int)value);
         return MI_CCL_SUCCESS;
     }

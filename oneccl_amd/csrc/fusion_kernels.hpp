@@ -562,11 +562,12 @@ inline hipError_t launch_fusion_tiled(const FusionLaunchArgs& a, const FusionPtr
                                       const PeerPtrs& pp, size_t t0, size_t t1) {
     const int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
     g_last_kernel = "fusion_reduce_tiled_kernel";
+    const uint32_t pace16 = fusion_write_pace16<TR, OP>(a, grid, 4);
     hipLaunchKernelGGL((fusion_reduce_tiled_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, own, out, pp, a.n_peers,
                        a.d_off, a.d_bytes, a.d_tile_end, (uint32_t)t0, (uint32_t)(t1 - t0), (uint32_t)a.tile_begin[t0],
-                       (uint32_t)(a.tile_begin[t1] - a.tile_begin[t0]), a.tune.sync, a.tune.early_loads,
-                       phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks, (uint32_t)a.tune.realign, (uint32_t)a.tune.wave_runs,
-                       fusion_write_pace16<TR, OP>(a, grid, 4));
+                       (uint32_t)(a.tile_begin[t1] - a.tile_begin[t0]), a.tune.sync,
+                       phase_early_loads<TR, OP>(a.tune, a.n_peers + 1, pace16 != 0), phase_early_stores<TR>(a.tune, 1),
+                       a.tune.spin_ticks, (uint32_t)a.tune.realign, (uint32_t)a.tune.wave_runs, pace16);
     return hipGetLastError();
 }
 
@@ -575,10 +576,11 @@ inline hipError_t launch_fusion_phased(const FusionLaunchArgs& a, const FusionPt
                                        const PeerPtrs& pp, uint64_t i0, uint64_t i1, size_t t0) {
     int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
     g_last_kernel = "fusion_reduce_phased_kernel";
+    const uint32_t pace16 = fusion_write_pace16<TR, OP>(a, grid, 2);
     hipLaunchKernelGGL((fusion_reduce_phased_kernel<TR, OP, NT>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, own, out, pp,
                        a.d_off, a.d_bytes, a.d_items + i0, (uint32_t)(i1 - i0), (uint32_t)t0, a.tune.sync,
-                       a.tune.early_loads, phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks, (uint32_t)a.tune.realign,
-                       (uint32_t)a.tune.wave_runs, fusion_write_pace16<TR, OP>(a, grid, 2));
+                       phase_early_loads<TR, OP>(a.tune, NT, pace16 != 0), phase_early_stores<TR>(a.tune, 1), a.tune.spin_ticks,
+                       (uint32_t)a.tune.realign, (uint32_t)a.tune.wave_runs, pace16);
     return hipGetLastError();
 }
 

@@ -53,7 +53,7 @@ struct Tuning {
     int num_cus;
     long phased_min_bytes;   // automatic choice: no phased kernel below this much traffic per launch
     struct PhaseSync* sync;  // the set of device-resident barrier words this call uses (may be null)
-    int early_loads;         // phased kernels: loads per lane still to issue when a block reports the end of its reads
+    int early_loads;         // phased kernels: loads per lane still to issue when a block reports the end of its reads (< 0: phase_early_loads chooses)
     int early_stores;        // ... and stores per lane still to issue when it reports the end of its writes (< 0: per type)
     long spin_ticks;         // phased kernels: longest wait at one barrier, in 100 MHz ticks, before a block goes on alone
     int fp16_impl;           // which CPU implementation's float16 results to reproduce: 2, 3 (through fp32) or 4 (native)
@@ -937,29 +937,54 @@ constexpr int kPhaseEarlyStores = 16;
 // at 1 GiB: 5.78 TB/s with 4 stores early against 6.25 with a strict report, 6.45 with the meeting and 16 early).  When
 // the clock paces the write phase (Tuning::write_pace) the last destination's 20 LDS-staged stores all come after the
 // report: 6.98 against 6.94 with 16.
-// Up to how many inputs a reduce to ONE destination has its write phase paced by the clock (see the kernel), at 1.1 x
-// Tuning::write_pace.  The shorter the read phase, the more it pays to start it with the chip's blocks in step;
-// measured at 512 MiB per buffer against the unpaced kernel, every operation: 3 inputs +2.0-2.9 %, 4 inputs +1.2-2.3 %,
-// 6 inputs +0.7-1.4 %, 8 inputs +0.1-1.1 %, 12 inputs -0.8..+0.7 % for the 16-bit integers, the 32- and 64-bit types
-// and fp16 sum / prod.  Where the read phase carries more arithmetic per byte it gains less and then loses: the 8-bit
-// types and fp16 min / max +1.3-2.8 % with 3 inputs, +0.2-0.7 % with 4, -0.2..-1.5 % from 6 on; both bfloat16 families
-// +-0.6 % with 3 and 4, -0.6..-2.0 % from 6 on (with 2 inputs every type gains: +1-4 %).
+// Element types and operations whose read phase carries a lot of arithmetic per byte: the 8-bit types (byte lanes),
+// both bfloat16 families (widen, round) and fp16 min / max (NaN handling).
 template <class TR, int OP>
-struct PhasePacedInputs {
-    static constexpr int value = sizeof(typename TR::elem_t) == 1 ? 4 : 8;
+struct PhaseHeavy {
+    static constexpr bool value = sizeof(typename TR::elem_t) == 1;
 };
 template <bool RNE, bool VEC_SEM, int OP>
-struct PhasePacedInputs<Bf16PairwiseTraits<RNE, VEC_SEM>, OP> {
-    static constexpr int value = 3;
+struct PhaseHeavy<Bf16PairwiseTraits<RNE, VEC_SEM>, OP> {
+    static constexpr bool value = true;
 };
 template <bool RNE, int OP>
-struct PhasePacedInputs<Bf16KeepTraits<RNE>, OP> {
-    static constexpr int value = 3;
+struct PhaseHeavy<Bf16KeepTraits<RNE>, OP> {
+    static constexpr bool value = true;
 };
 template <bool NATIVE, int OP>
-struct PhasePacedInputs<Fp16Traits<NATIVE>, OP> {
-    static constexpr int value = (OP == OP_MIN || OP == OP_MAX) ? 4 : 8;
+struct PhaseHeavy<Fp16Traits<NATIVE>, OP> {
+    static constexpr bool value = OP == OP_MIN || OP == OP_MAX;
 };
+
+// Up to how many inputs a reduce to ONE destination has its write phase paced by the clock (see the kernel), at 1.1 x
+// Tuning::write_pace: the blocks of the chip then start the read phase that follows in step, which pays the more the
+// shorter that phase is.  Measured at 512 MiB per buffer against the unpaced kernel, each with its best early arrival
+// (phase_early_loads below): 2 inputs +1-4 %, 3 inputs +2.0-3.4 %, 4 inputs +1.2-3.0 %, 5 and 6 inputs +1.5-2.3 %,
+// 8 inputs +0.6-1.8 % (bfloat16, fp32 accumulation, 8 x 2 GB: 7.15-7.17 against 7.07-7.085 TB/s), 12 inputs
+// +0.4-1.1 % (the rounded-every-step bfloat16 family and bfloat16 min / max +-0), 16 inputs +0.5-0.8 % for the light
+// types and -0.7..+0.5 % for the heavy ones, which stay unpaced there.
+template <class TR, int OP>
+struct PhasePacedInputs {
+    static constexpr int value = PhaseHeavy<TR, OP>::value ? 12 : 16;
+};
+
+// Loads per lane still to issue when a block reports the end of its read phase (Tuning::early_loads < 0 asks for
+// this).  Unpaced, 12 hides the barrier's latency best for every type (8 to 16 are within 0.3 %).  Behind a paced write
+// phase the blocks reach the end of their reads almost together, and an arrival that early lets the first stores out
+// under the last reads: the light types then want 12 with up to four inputs and 8 from five on (+0.3-1 %), the heavy
+// ones 8 with two inputs, 5 with three and four, 2 from five on (512 MiB per buffer, 12 against the best: int8 with 4
+// inputs 6.92 against 7.09 TB/s, with 8 inputs 7.00 against 7.16; bfloat16 with 8 inputs 7.08 against 7.23, with 3
+// inputs 6.76 against 6.91; fp16 max with 4 inputs 6.83 against 7.01).  The same holds with several destinations
+// (1 GiB per buffer, bfloat16: 8 -> 8 6.92 against 7.12, 8 -> 2 6.93 against 7.08, 4 -> 4 6.91 against 7.02; one buffer
+// copied to 2: 6.80 against 6.88).
+constexpr int kPhaseEarlyLoads = 12;
+template <class TR, int OP>
+inline int phase_early_loads(const Tuning& t, int n, bool paced) {
+    if (t.early_loads >= 0) return t.early_loads;
+    if (!paced) return kPhaseEarlyLoads;
+    if (PhaseHeavy<TR, OP>::value) return n <= 2 ? 8 : n <= 4 ? 5 : 2;
+    return n <= 4 ? kPhaseEarlyLoads : 8;
+}
 
 template <class TR>
 inline int phase_early_stores(const Tuning& t, int n_dsts) {
@@ -1238,7 +1263,8 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
         write_pace16 = write_pace_ticks16((uint64_t)grid * kPhaseBlock * 16u * 4u, rate, a.tune.wall_khz);
         g_last_kernel = "reduce_multi_phased_kernel";
         hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
-                           a.m, v.head, v.nvec, v.tail, a.tune.sync, a.tune.early_loads, phase_early_stores<TR>(a.tune, a.m),
+                           a.m, v.head, v.nvec, v.tail, a.tune.sync, phase_early_loads<TR, OP>(a.tune, a.n, write_pace16 != 0),
+                           phase_early_stores<TR>(a.tune, a.m),
                            a.tune.spin_ticks, v.beyond, wave_runs, write_pace16);
         return hipGetLastError();
     }

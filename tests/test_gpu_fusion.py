@@ -253,7 +253,7 @@ def test_fused_reduce_over_several_phases(comp, dtype, op, n_peers, lp, impl, al
         want.append(O.reduce_n([tensors[i]] + [p[o:o + c] for p in peers], dtype, op, keep=lp, bf16_impl=impl))
     # the default, then other points at which a block reports its arrival at the barrier and other paces of the write
     # phase (which only few enough inputs for the type take): timing only, same bits
-    for loads, stores, pace in ((12, -1, 7300), (0, 0, 0), (4096, 20, 30000), (40, 3, 400)):
+    for loads, stores, pace in ((-1, -1, 7300), (0, 0, 0), (4096, 20, 30000), (40, 3, 400)):
         for o in outs:
             o.zero_()
         comp.set_param("variant", 8)
@@ -266,7 +266,7 @@ def test_fused_reduce_over_several_phases(comp, dtype, op, n_peers, lp, impl, al
             assert comp.last_kernel() == ("fusion_reduce_tiled_kernel" if n_peers >= 5 else "fusion_reduce_phased_kernel")
         finally:
             comp.set_param("variant", 0)
-            comp.set_param("phase_early_loads", 12)
+            comp.set_param("phase_early_loads", -1)
             comp.set_param("phase_early_stores", -1)
             comp.set_param("phase_write_pace", 7300)
         for i, c in enumerate(counts):

@@ -466,10 +466,10 @@ def test_phased_kernel_early_arrival_settings(comp, dtype, op, n, m):
     srcs = make_inputs(rng, dtype, count, op, n)
     want = O.reduce_n(srcs, dtype, op, keep=keep, threads=16)
     d = [to_dev(s) for s in srcs]
-    assert comp.get_param("phase_early_loads") == 12 and comp.get_param("phase_early_stores") == -1
+    assert comp.get_param("phase_early_loads") == -1 and comp.get_param("phase_early_stores") == -1
     comp.set_param("variant", 8)
     try:
-        for loads, stores in ((12, -1), (0, 0), (4, 20), (1000, 1), (4096, 7), (13, 19)):
+        for loads, stores in ((-1, -1), (12, -1), (0, 0), (4, 20), (1000, 1), (4096, 7), (13, 19)):
             comp.set_param("phase_early_loads", loads)
             comp.set_param("phase_early_stores", stores)
             outs = [torch.zeros_like(d[0]) for _ in range(m)]
@@ -479,12 +479,12 @@ def test_phased_kernel_early_arrival_settings(comp, dtype, op, n, m):
             for o in outs:
                 assert_same(to_host(o, O.NP_STORAGE[dtype]), want, dtype, f"early loads {loads} stores {stores}", srcs, op,
                             keep=keep)
-        for bad in (("phase_early_loads", -1), ("phase_early_loads", 4097), ("phase_early_stores", -2), ("phase_early_stores", 21)):
+        for bad in (("phase_early_loads", -2), ("phase_early_loads", 4097), ("phase_early_stores", -2), ("phase_early_stores", 21)):
             with pytest.raises(comp.CclError):
                 comp.set_param(*bad)
     finally:
         comp.set_param("variant", 0)
-        comp.set_param("phase_early_loads", 12)
+        comp.set_param("phase_early_loads", -1)
         comp.set_param("phase_early_stores", -1)
 
 
