@@ -100,7 +100,8 @@ reduce_batch_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tiles) {
 // step the chip reads `grid` consecutive tiles.  Which job a tile belongs to, and where in it the tile starts, is
 // worked out by lane q of every wave for the block's q-th tile of a phase (batch_describe), ahead of the phase.
 // Staging (registers and LDS), barrier, early arrival and arithmetic are those of
-// reduce_multi_phased_kernel; the jobs' edge elements are computed after the last phase, job j by block j mod grid.
+// reduce_multi_phased_kernel; the jobs' edge elements are computed between the report of the first write phase and
+// the wait that follows it, job j by block j mod grid.
 constexpr int kBatchPhaseG = 4;
 constexpr uint64_t kBatchPhaseTile = (uint64_t)kBatchPhaseG * kPhaseBlock;
 
@@ -207,8 +208,7 @@ __device__ __forceinline__ void reduce_batch_edges(const BatchTable& tb, int n, 
         const uint32_t p0 = (uint32_t)(j * (n + 1));
         const uint32_t e = threadIdx.x;
         const uint64_t i = (e < head) ? e : (uint64_t)head + nvec * TR::VEC + (e - head);
-        typename TR::acc_t r = TR::init(ld_elem<E>(tb.p[p0], i));
-        for (int k = 1; k < n; k++) r = TR::template step<OP>(ld_elem<E>(tb.p[p0 + k], i), r);
+        const typename TR::acc_t r = fold_element<TR, OP>(tb.p + p0, 1, n, i, TR::init(ld_elem<E>(tb.p[p0], i)));
         st_elem<E>((void*)tb.p[p0 + n], i, TR::finish(r));
     }
 }
@@ -305,19 +305,21 @@ reduce_batch_phased_kernel(BatchTable tb, int n, int n_jobs, uint32_t total_tile
                 if (i < s.nvec) st_loose(d + i, stage[(q * G + g) * kPhaseBlock + threadIdx.x]);
             }
         }
-        if (more) {
-            if (arrive_u == kPhaseU) {
-                __syncthreads();                            // "when done": every wave's stores have been acknowledged
-                if (threadIdx.x == 0) phase_arrive(ps);
-            }
-            phase_wait(ps, ++gen, give_up, spin_ticks);
+        if (more && arrive_u == kPhaseU) {
+            __syncthreads();                                // "when done": every wave's stores have been acknowledged
+            if (threadIdx.x == 0) phase_arrive(ps);
         }
+        // The jobs' edge elements, spread over the blocks, after the block's report of the first write phase and before
+        // its wait: there the round trip to memory costs nothing while other blocks still write.  Inside a read phase
+        // it held up the one block of a job's first tile, and with it the barrier (64 jobs of 4 x 4 MiB with 112-byte
+        // heads: 241 us against 222 us); after the last phase it is the last thing the chip does.
+        if (t0 == 0)
+            for (int j = blockIdx.x; j < n_jobs; j += gridDim.x) reduce_batch_edges<TR, OP>(tb, n, j);
+        if (more) phase_wait(ps, ++gen, give_up, spin_ticks);
         desc = next;
     }
-    // The jobs' edge elements, after the last phase and spread over the blocks: their loads depend on one another (the
-    // inputs are taken in order), and inside a read phase that chain of round trips held up the one block of a job's
-    // first tile, and with it the barrier (64 jobs of 4 x 4 MiB with 112-byte heads: 241 us against 222 us).
-    for (int j = blockIdx.x; j < n_jobs; j += gridDim.x) reduce_batch_edges<TR, OP>(tb, n, j);
+    if (total_tiles == 0)       // no phase at all
+        for (int j = blockIdx.x; j < n_jobs; j += gridDim.x) reduce_batch_edges<TR, OP>(tb, n, j);
 }
 
 // Host side: fills tables of at most kBatchMaxJobs jobs / kBatchMaxPtrs pointers and launches one kernel per table,

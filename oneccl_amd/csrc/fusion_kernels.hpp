@@ -327,8 +327,8 @@ fusion_reduce_phased_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, cons
 // peers is a run-time count, and what a tile needs to know (where it starts in the own tensor, in the output and in
 // the peers' buffers, its size, head and the realignment's needs) is worked out by lane q of every wave for the
 // block's q-th tile of a phase: the first phase's at the start, every later one's while the block waits at the
-// barrier in the middle of the phase before.  Elements before a tile's first and after its last vector are left to
-// a pass after the last phase.  A phase holds 12 tiles per block (28 vectors per lane in registers, 20 in LDS; no type
+// barrier in the middle of the phase before.  Elements before a tile's first and after its last vector are computed
+// phase by phase between the block's report of its write phase and its wait.  A phase holds 12 tiles per block (28 vectors per lane in registers, 20 in LDS; no type
 // spills with them): the 256-tensor configuration of 191 MB then takes two phases instead of two and a small third
 // (258 against 264 us), larger plans measure the same either way.
 constexpr uint32_t kFusionTile = (uint32_t)kBatchPhaseTile * 16u;       // 32 KiB
@@ -442,7 +442,8 @@ fusion_reduce_tiled_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n
     const int n = n_peers + 1;
     const uint64_t grid = gridDim.x;
     const uint64_t per_phase = grid * (uint64_t)(RG + LG);      // tiles
-    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    static_assert(3 * TR::VEC - 2 <= 64, "a wave holds a tile's edge elements");
     auto describe = [&](uint64_t tile) {
         return fusion_describe<TR>(own, out, peers, n_peers, off, bytes, tile_end, t0, nt, tile_base, tile, ntiles, realign);
     };
@@ -517,34 +518,42 @@ fusion_reduce_tiled_kernel(FusionPtrs own, FusionPtrs out, PeerPtrs peers, int n
                 if (i < s.nvec) st_loose(d + i, stage[(q * G + g) * kPhaseBlock + threadIdx.x]);
             }
         }
-        if (more) {
-            if (arrive_u == kPhaseU) {
-                __syncthreads();                            // "when done": every wave's stores have been acknowledged
-                if (threadIdx.x == 0) phase_arrive(ps);
-            }
-            phase_wait(ps, ++gen, give_up, spin_ticks);
+        if (more && arrive_u == kPhaseU) {
+            __syncthreads();                                // "when done": every wave's stores have been acknowledged
+            if (threadIdx.x == 0) phase_arrive(ps);
         }
+        // The elements before a tile's first and after its last vector, for this phase's tiles (lane q holds the q-th
+        // one's description): those that have such elements go round the block's waves, one element per lane (at most
+        // VEC - 1 in front and 2 VEC - 1 behind), the elements of eight inputs loaded before their steps so that the loads
+        // are in flight together.  Here, after the block's report and before its wait, the round trip costs nothing
+        // while other blocks still write; in front of the report it would hold the whole chip back.
+        {
+            const uint32_t ne = desc.nb / ES, eh = desc.headb & 0xffu;
+            const uint32_t ev = desc.nb ? (ne - eh) / TR::VEC - ((desc.headb >> 9) & 1u) : 0u;
+            unsigned long long todo = __ballot(desc.nb != 0 && (eh + (ne - eh - ev * TR::VEC)) != 0);
+            for (uint32_t turn = 0; todo; turn++) {
+                const int q = __builtin_ctzll(todo);
+                todo &= todo - 1;
+                if ((turn & (kPhaseBlock / 64 - 1)) != wave) continue;
+                const FusionSlot s = fusion_slot<TR>(desc, q, 0);
+                if (lane < s.head + s.tail) {
+                    const uint32_t i = (lane < s.head) ? lane : s.head + s.nvec * TR::VEC + (lane - s.head);
+                    typename TR::acc_t r = TR::init(ld_elem<E>(s.a, i));
+                    for (int j0 = 0; j0 < n_peers; j0 += 8) {
+                        E x[8];
+#pragma unroll
+                        for (int u = 0; u < 8; u++)
+                            if (j0 + u < n_peers) x[u] = ld_elem<E>((const unsigned char*)peers.p[j0 + u] + s.poff, i);
+#pragma unroll
+                        for (int u = 0; u < 8; u++)
+                            if (j0 + u < n_peers) r = TR::template step<OP>(x[u], r);
+                    }
+                    st_elem<E>(s.o, i, TR::finish(r));
+                }
+            }
+        }
+        if (more) phase_wait(ps, ++gen, give_up, spin_ticks);
         desc = next;
-    }
-    // The elements before a tile's first and after its last vector: this block's tiles once more, 64 at a time (lane
-    // L describes tile base + L * grid), and for those that have such elements one element per lane, the inputs in
-    // order.  After the last phase, because the loads of that chain depend on one another.
-    for (uint64_t base = blockIdx.x; base < ntiles; base += 64u * grid) {
-        const FusionDesc e = describe(base + (uint64_t)lane * grid);
-        uint32_t ne = e.nb / ES, eh = e.headb & 0xffu;
-        uint32_t ev = e.nb ? (ne - eh) / TR::VEC - ((e.headb >> 9) & 1u) : 0u;
-        unsigned long long todo = __ballot(e.nb != 0 && (eh + (ne - eh - ev * TR::VEC)) != 0);
-        while (todo) {
-            const int q = __builtin_ctzll(todo);
-            todo &= todo - 1;
-            const FusionSlot s = fusion_slot<TR>(e, q, 0);
-            if (threadIdx.x < s.head + s.tail) {
-                const uint32_t i = (threadIdx.x < s.head) ? threadIdx.x : s.head + s.nvec * TR::VEC + (threadIdx.x - s.head);
-                typename TR::acc_t r = TR::init(ld_elem<E>(s.a, i));
-                for (int j = 0; j < n_peers; j++) r = TR::template step<OP>(ld_elem<E>((const unsigned char*)peers.p[j] + s.poff, i), r);
-                st_elem<E>(s.o, i, TR::finish(r));
-            }
-        }
     }
 }
 

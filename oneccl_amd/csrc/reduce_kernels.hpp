@@ -651,6 +651,24 @@ __device__ __forceinline__ void load_vectors(const unsigned char* base, const ui
     for (int g = 0; g < G; g++) x[g] = (FULL || idx[g] < nvec) ? ld_loose(sp + idx[g]) : u32x4{ 0, 0, 0, 0 };
 }
 
+// Element i of inputs p[first] .. p[last - 1] folded into r in that order, eight loads in flight together (a plain
+// loop waits for every load before the next is issued: one trip to memory per input at the end of a launch).
+template <class TR, int OP, class PTR>
+__device__ __forceinline__ typename TR::acc_t fold_element(const PTR* p, int first, int last, uint64_t i,
+                                                           typename TR::acc_t r) {
+    typedef typename TR::elem_t E;
+    for (int j0 = first; j0 < last; j0 += 8) {
+        E x[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (j0 + u < last) x[u] = ld_elem<E>(p[j0 + u], i);
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (j0 + u < last) r = TR::template step<OP>(x[u], r);
+    }
+    return r;
+}
+
 // The count % VEC elements after the last full vector and the elements before the first aligned one:
 // at most 127 + 2 * VEC - 1 <= 158 elements (the head may reach to a 128-byte line), one per lane of block 0.
 template <class TR, int OP, class SRC>
@@ -660,8 +678,7 @@ __device__ __forceinline__ void reduce_edges(const SRC& src, int n, void* dst, u
     uint32_t t = threadIdx.x;
     if (t < head + tail) {
         uint64_t i = (t < head) ? t : (uint64_t)head + nvec * TR::VEC + (t - head);
-        typename TR::acc_t a = TR::init(ld_elem<E>(src.p[0], i));
-        for (int j = 1; j < n; j++) a = TR::template step<OP>(ld_elem<E>(src.p[j], i), a);
+        const typename TR::acc_t a = fold_element<TR, OP>(src.p, 1, n, i, TR::init(ld_elem<E>(src.p[0], i)));
         st_elem<E>(dst, i, TR::finish(a));
     }
 }
@@ -887,8 +904,7 @@ __device__ __forceinline__ void reduce_multi_edges(const SrcTable& src, int n, c
     uint32_t t = threadIdx.x;
     if (t < head + tail) {
         uint64_t i = (t < head) ? t : (uint64_t)head + nvec * TR::VEC + (t - head);
-        typename TR::acc_t a = TR::init(ld_elem<E>(src.p[0], i));
-        for (int j = 1; j < n; j++) a = TR::template step<OP>(ld_elem<E>(src.p[j], i), a);
+        const typename TR::acc_t a = fold_element<TR, OP>(src.p, 1, n, i, TR::init(ld_elem<E>(src.p[0], i)));
         const E r = TR::finish(a);
         for (int k = 0; k < m; k++) st_elem<E>(dst.p[k], i, r);
     }
@@ -1098,15 +1114,18 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
                 if (i < nvec) st_loose(d + i, stage[u * kPhaseBlock + threadIdx.x]);
             }
         }
-        if (more) {
-            if (arrive_u == kPhaseU) {
-                __syncthreads();                    // "when done": every wave's stores have been acknowledged
-                if (threadIdx.x == 0) phase_arrive(ps);
-            }
-            phase_wait(ps, ++gen, give_up, spin_ticks);
+        if (more && arrive_u == kPhaseU) {
+            __syncthreads();                        // "when done": every wave's stores have been acknowledged
+            if (threadIdx.x == 0) phase_arrive(ps);
         }
+        // The elements in front of the first and behind the last vector, once, by block 0: after its report of the
+        // first write phase and before its wait, where the round trip to memory costs nothing while other blocks still
+        // write (at the end of the launch it would be the last thing the chip does, in front of a report it would hold
+        // every block back).
+        if (p0 == 0 && blockIdx.x == 0 && (head | tail)) reduce_multi_edges<TR, OP>(src, n, dst, m, head, nvec, tail);
+        if (more) phase_wait(ps, ++gen, give_up, spin_ticks);
     }
-    if (blockIdx.x == 0 && (head | tail)) reduce_multi_edges<TR, OP>(src, n, dst, m, head, nvec, tail);
+    if (nvec == 0 && blockIdx.x == 0 && (head | tail)) reduce_multi_edges<TR, OP>(src, n, dst, m, head, nvec, tail);   // no phase at all
 }
 
 // ---------------------------------------------------------------------------------------------------
