@@ -54,6 +54,35 @@ def test_reduce_n_all_dtypes_ops(comp, dtype, op):
                                 f"kind={kind} lp={lp} impl={impl}", srcs, op, keep=keep, bf16_impl=impl)
 
 
+@pytest.mark.parametrize("dtype,op", [(O.BFLOAT16, O.SUM), (O.INT8, O.MIN), (O.FLOAT64, O.PROD), (O.UINT16, O.MAX)])
+def test_reduce_n_many_inputs(comp, dtype, op):
+    """17 to 64 inputs (the most one call takes): the elements in front of the first and behind the last vector are
+    folded eight inputs at a time, so these counts leave one, two and no input over, in the streaming and in the phased
+    kernel, with the buffers two elements off their holders' boundary."""
+    import torch
+    rng = np.random.default_rng(5200 + dtype * 4 + op)
+    np_t = O.NP_STORAGE[dtype]
+    keep = 1 if dtype == O.BFLOAT16 else 0
+    for n in (17, 18, 25, 33, 64):
+        for count in (5, 4099, 70001):
+            srcs = make_inputs(rng, dtype, count, op, n)
+            holders = [to_dev(np.concatenate([np.zeros(2, np_t), s_])) for s_ in srcs]
+            want = O.reduce_n(srcs, dtype, op, keep=keep)
+            for variant in (0, 8):
+                out = to_dev(np.zeros(count + 4, np_t))
+                comp.set_param("variant", variant)
+                try:
+                    comp.comp_reduce_n(dtype, op, [h[2:] for h in holders], out[2:], count, lp_mode=keep)
+                    torch.cuda.synchronize()
+                finally:
+                    comp.set_param("variant", 0)
+                g = to_host(out, np_t)
+                assert_same(g[2:2 + count], want, dtype, f"n={n} count={count} variant={variant}", srcs, op, keep=keep)
+                assert not g[:2].view(np.uint8).any() and not g[2 + count:].view(np.uint8).any(), "wrote outside"
+    with pytest.raises(comp.CclError):
+        comp.comp_reduce_n(dtype, op, [holders[0]] * 65, out, 5, lp_mode=keep)
+
+
 @pytest.mark.parametrize("fam,dtype", [("bf16", O.BFLOAT16), ("fp16", O.FLOAT16)])
 def test_pairwise_against_reference_made_golden_vectors(comp, golden, fam, dtype):
     """GPU result vs what the reference's ccl_bf16_reduce_impl_* / ccl_fp16_reduce_impl_* produced."""
