@@ -260,7 +260,10 @@ const char* mi_ccl_last_kernel(void);
  * default 1: an input of a 16- or 8-bit type whose vectors start off a 4-byte boundary -- a peer's block behind an odd
  * number of elements, a tensor behind an odd-sized one in a tight fusion buffer -- is read on that boundary and shifted
  * into place in registers instead of with misaligned vector loads; same results, about a fifth faster for such
- * layouts), "realigned_launches" (read only: how many launches of the calling thread took that path), "line_start"
+ * layouts), "realigned_launches" (read only: how many launches of the calling thread took that path),
+ * "wide_phase_launches" (read only: how many phased reduces of the calling thread kept four more result vectors per
+ * lane in registers, 96 instead of 88 MiB of results per phase on 256 CUs, because that took a whole phase off a launch
+ * of at most six phases), "line_start"
  * (0/1, default 1: a reduce, copy or broadcast of 1 MiB or more per buffer starts its 16-byte vectors on a 128-byte
  * line of the buffers that matter most -- the outputs before the inputs -- so up to 127 bytes at the front are
  * handled element by element; buffers that share an offset from the lines then run like aligned ones, +6 %) and

@@ -44,6 +44,7 @@ MI_DECLARE(Bf16KeepTraits<true>);
 
 thread_local const char* g_last_kernel = "";
 thread_local unsigned long g_realigned_launches = 0;
+thread_local unsigned long g_wide_phase_launches = 0;
 
 static std::atomic<int> g_waves_per_cu{ 256 };
 static std::atomic<int> g_max_blocks{ 0 };
@@ -950,6 +951,8 @@ long mi_ccl_get_param(const char* name) {
         return g_realign.load();
     if (!strcmp(name, "realigned_launches"))
         return (long)g_realigned_launches;
+    if (!strcmp(name, "wide_phase_launches"))
+        return (long)g_wide_phase_launches;
     if (!strcmp(name, "line_start"))
         return g_line_start.load();
     if (!strcmp(name, "wave_runs"))

@@ -69,6 +69,7 @@ struct Tuning {
 extern thread_local const char* g_last_kernel;
 // Launches by the calling thread whose inputs off a 4-byte boundary were realigned in registers (tests ask for it).
 extern thread_local unsigned long g_realigned_launches;
+extern thread_local unsigned long g_wide_phase_launches;    // launches of the phased reduce with one more register group (phase_reg_groups)
 
 struct LaunchArgs {
     const void* const* srcs;    // host array of n device pointers
@@ -1008,10 +1009,11 @@ inline int phase_early_stores(const Tuning& t, int n_dsts) {
     return v < kPhaseU ? v : kPhaseU;
 }
 
-// The phased form of the same: kPhaseU vectors per lane in LDS and 4 x MultiPhaseRegs::groups in registers are
+// The phased form of the same: kPhaseU vectors per lane in LDS and 4 x RG in registers (RG = MultiPhaseRegs::groups, or
+// one more where that saves a phase: phase_reg_groups) are
 // reduced while HBM sees only reads, then stored to every destination while it sees only writes.  The register
 // groups are unrolled (a register file has no run-time index); the loop over the inputs inside each stays a loop.
-template <class TR, int OP>
+template <class TR, int OP, int RG>
 __global__ void __launch_bounds__(kPhaseBlock)
 reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t head, uint64_t nvec, uint32_t tail,
                            PhaseSync* ps, int early_loads, int early_stores, long spin_ticks, uint32_t beyond,
@@ -1020,7 +1022,6 @@ reduce_multi_phased_kernel(SrcTable src, int n, DstTable dst, int m, uint32_t he
     kernel_prologue<TR, OP>();
     const uint64_t nload = nvec + beyond;               // vector nvec may be read when beyond = 1 (load_vectors)
     constexpr int G = 4;                                // vectors per lane and input in flight
-    constexpr int RG = MultiPhaseRegs<TR>::groups;
     constexpr int LG = kPhaseU / G;                     // groups staged in LDS
     static_assert(kPhaseU % G == 0, "LDS steps must be a multiple of the group size");
     __shared__ u32x4 stage[kPhaseU * kPhaseBlock];
@@ -1197,6 +1198,9 @@ inline bool broadcast_wants_phased(const Tuning& t, uint64_t bytes) {
 // 2 inputs, +17 % with 8 at 4 GiB of traffic), with several destinations from twice that traffic.  One input stays with
 // the copy and broadcast kernels, except that a buffer of two phases or more going to several destinations takes the
 // phased form with its paced write phase (broadcast_wants_phased).  Tuning::variant 8 forces the phased form.
+inline uint64_t phase_lanes(const Tuning& t) {       // lanes of a phased launch: one block of kPhaseBlock on every CU
+    return (uint64_t)(t.num_cus / kPhaseGroups) * kPhaseGroups * kPhaseBlock;
+}
 inline bool wants_phased(const LaunchArgs& a, uint64_t nvec, int reg_groups) {
     if (a.tune.sync == nullptr || a.tune.num_cus < kPhaseGroups) return false;
     if (a.tune.variant != 0) return a.tune.variant == 8;
@@ -1263,7 +1267,8 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
     for (int k = 0; k < a.m; k++) d.p[k] = a.dsts ? a.dsts[k] : a.dst;
     const VecSplit v = vector_split<E, TR::VEC>(a);
     g_realigned_launches += v.beyond;
-    if (wants_phased(a, v.nvec, MultiPhaseRegs<TR>::groups)) {
+    const int reg_groups = phase_reg_groups(v.nvec, phase_lanes(a.tune), MultiPhaseRegs<TR>::groups, kPhaseU);
+    if (wants_phased(a, v.nvec, reg_groups)) {
         int grid = (a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
         // does any buffer's first vector start off a 128-byte line?
         uint32_t off_lines = 0;
@@ -1281,7 +1286,10 @@ inline hipError_t launch_multi_op(const LaunchArgs& a) {
                                                                       : 0.0;
         write_pace16 = write_pace_ticks16((uint64_t)grid * kPhaseBlock * 16u * 4u, rate, a.tune.wall_khz);
         g_last_kernel = "reduce_multi_phased_kernel";
-        hipLaunchKernelGGL((reduce_multi_phased_kernel<TR, OP>), dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
+        constexpr int kUsual = MultiPhaseRegs<TR>::groups;
+        g_wide_phase_launches += reg_groups > kUsual;
+        const auto kernel = reg_groups > kUsual ? reduce_multi_phased_kernel<TR, OP, kUsual + 1> : reduce_multi_phased_kernel<TR, OP, kUsual>;
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kPhaseBlock), 0, a.stream, s, a.n, d,
                            a.m, v.head, v.nvec, v.tail, a.tune.sync, phase_early_loads<TR, OP>(a.tune, a.n, write_pace16 != 0),
                            phase_early_stores<TR>(a.tune, a.m),
                            a.tune.spin_ticks, v.beyond, wave_runs, write_pace16);
@@ -1301,7 +1309,8 @@ inline hipError_t launch_op(const LaunchArgs& a) {
     typedef typename TR::elem_t E;
     if (a.m > 1 || a.n > kMaxFixedN) return launch_multi_op<TR, OP>(a);     // run-time counts of inputs and outputs
     const VecSplit v = vector_split<E, TR::VEC>(a);
-    if (wants_phased(a, v.nvec, MultiPhaseRegs<TR>::groups)) return launch_multi_op<TR, OP>(a);     // the phased kernel takes any number of inputs
+    if (wants_phased(a, v.nvec, phase_reg_groups(v.nvec, phase_lanes(a.tune), MultiPhaseRegs<TR>::groups, kPhaseU)))
+        return launch_multi_op<TR, OP>(a);          // the phased kernel takes any number of inputs
     // five or more inputs in the range between latency-bound and phased (64 to 240 MB of traffic): taking the inputs
     // one after the other, as the run-time-count streaming kernel does, measures 5-12 % above loading them together
     if (a.n >= 5 && a.tune.variant == 0 && (uint64_t)(a.n + 1) * v.nvec * 16u >= (uint64_t)a.tune.phased_min_bytes / 5 * 2)

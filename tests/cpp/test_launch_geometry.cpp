@@ -233,6 +233,21 @@ int main() {
         for (int n = 2; n <= 64; n++) EXPECT(phases_full_enough(mib(2000), per, n));    // long buffers always
         EXPECT(!phases_full_enough(0, per, 8) && !phases_full_enough(100, 0, 8));
     }
+    // one more register group where it takes a phase off a launch of few phases (88 MiB per phase as usual, 96 MiB wider)
+    {
+        const uint64_t lanes = 256ull * 512;
+        auto mib = [](uint64_t m) { return (m << 20) / 16; };
+        EXPECT(phase_reg_groups(mib(64), lanes, 6, 20) == 6 && phase_reg_groups(mib(88), lanes, 6, 20) == 6);     // one phase either way
+        EXPECT(phase_reg_groups(mib(88) + 1, lanes, 6, 20) == 7 && phase_reg_groups(mib(96), lanes, 6, 20) == 7);   // two phases -> one
+        EXPECT(phase_reg_groups(mib(96) + 1, lanes, 6, 20) == 6 && phase_reg_groups(mib(176), lanes, 6, 20) == 6);  // two either way
+        EXPECT(phase_reg_groups(mib(192), lanes, 6, 20) == 7 && phase_reg_groups(mib(256), lanes, 6, 20) == 6);
+        EXPECT(phase_reg_groups(mib(384), lanes, 6, 20) == 7);                                                      // five -> four
+        EXPECT(phase_reg_groups(mib(528), lanes, 6, 20) == 6 && phase_reg_groups(mib(570), lanes, 6, 20) == 6);     // six either way; seven -> six: too many to matter
+        EXPECT(phase_reg_groups(mib(1024), lanes, 6, 20) == 6 && phase_reg_groups(1003782144ull / 8, lanes, 6, 20) == 6);
+        EXPECT(phase_reg_groups(0, lanes, 6, 20) == 6 && phase_reg_groups(mib(96), 0, 6, 20) == 6);
+        // with the wider phase 92 MiB from two inputs is one phase at fill 0.96: phased
+        EXPECT(phases_full_enough(mib(92), lanes * 48, 2) && !phases_full_enough(mib(92), lanes * 44, 2));
+    }
     printf("%d checks, %d failed\n", checks, failed);
     return failed ? 1 : 0;
 }

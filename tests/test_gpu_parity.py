@@ -83,6 +83,46 @@ def test_reduce_n_many_inputs(comp, dtype, op):
         comp.comp_reduce_n(dtype, op, [holders[0]] * 65, out, 5, lp_mode=keep)
 
 
+@pytest.mark.parametrize("dtype", range(12))
+def test_phased_reduce_with_the_wider_phase(comp, dtype):
+    """Results of 88 to 96 MiB take one phase when a lane keeps four more vectors in registers (two phases otherwise),
+    and the library then launches that form of the phased kernel: every element type and 16-bit mode, two inputs (and
+    eight for bfloat16), against the oracle over every element."""
+    import torch
+    rng = np.random.default_rng(8800 + dtype)
+    esz = O.DTYPE_SIZE[dtype]
+    assert comp.get_param("num_cus") == 256, "sizes below are for 256 CUs"
+    count = (92 << 20) // esz + 3
+    op = (O.SUM, O.MAX, O.PROD, O.MIN)[dtype % 4]
+    for n in ((2, 8) if dtype == O.BFLOAT16 else (2,)):
+        srcs = make_inputs(rng, dtype, count, op, n)
+        d = [to_dev(s) for s in srcs]
+        for lp, impl, keep, quirk in lp_variants(dtype):
+            if quirk:
+                continue
+            out = torch.empty_like(d[0])
+            wide = comp.get_param("wide_phase_launches")
+            comp.comp_reduce_n(dtype, op, d, out, count, lp_mode=lp, bf16_impl=impl)
+            torch.cuda.synchronize()
+            assert comp.last_kernel() == "reduce_multi_phased_kernel" and comp.get_param("wide_phase_launches") == wide + 1
+            want = O.reduce_n(srcs, dtype, op, keep=keep, bf16_impl=impl, threads=16)
+            assert_same(to_host(out, O.NP_STORAGE[dtype]), want, dtype, f"n={n} lp={lp} impl={impl}", srcs, op, keep=keep, bf16_impl=impl)
+        if dtype == O.FLOAT16:      # the avx512fp16 implementation is a kernel family of its own
+            out = torch.empty_like(d[0])
+            comp.comp_reduce_n(dtype, op, d, out, count, fp16_impl=comp.FP16_AVX512FP16)
+            torch.cuda.synchronize()
+            want = O.reduce_n(srcs, dtype, op, fp16_impl=O.FP16_AVX512FP16, threads=16)
+            assert_same(to_host(out, O.NP_STORAGE[dtype]), want, dtype, f"n={n} native fp16", srcs, op, fp16_impl=O.FP16_AVX512FP16)
+        del d
+    # 80 MiB is one phase either way, 1 GiB twelve against eleven: the usual form
+    wide = comp.get_param("wide_phase_launches")
+    small = (80 << 20) // esz
+    a, b = to_dev(np.zeros(small, O.NP_STORAGE[dtype])), to_dev(np.zeros(small, O.NP_STORAGE[dtype]))
+    comp.comp_reduce_n(dtype, O.MAX, [a, b], a, small)
+    torch.cuda.synchronize()
+    assert comp.get_param("wide_phase_launches") == wide
+
+
 @pytest.mark.parametrize("fam,dtype", [("bf16", O.BFLOAT16), ("fp16", O.FLOAT16)])
 def test_pairwise_against_reference_made_golden_vectors(comp, golden, fam, dtype):
     """GPU result vs what the reference's ccl_bf16_reduce_impl_* / ccl_fp16_reduce_impl_* produced."""
