@@ -1209,6 +1209,11 @@ inline bool wants_phased(const LaunchArgs& a, uint64_t nvec, int reg_groups) {
     if (a.n < 2) return a.m > 1 && broadcast_wants_phased(a.tune, nvec * 16u);    // one input that is not a plain copy (bf16 keep-precision narrows it)
     if (traffic < (uint64_t)a.tune.phased_min_bytes * (a.m > 1 ? 2u : 1u)) return false;
     if (a.m > 1) return true;
+    // Five or more inputs meet a stronger streaming kernel (reduce_multi_kernel, which takes the inputs one after the
+    // other: 6.15-6.4 TB/s from 64 MB of traffic on): the phased form passes it at about 300 MB of traffic -- 8 inputs of
+    // 24 / 28 / 32 / 40 MiB: 5.83 / 5.82 / 6.17 / 6.38 against 6.2; 12 inputs of 16 / 20 / 24 / 32 MiB: 5.79 / 5.76 / 6.25 / 6.47
+    // against 6.41 / 6.35 / 6.27 / 6.18; 6 inputs of 32 / 40 / 48 MiB: 5.89 / 6.13 / 6.30 against 6.2.
+    if (a.n >= 5 && traffic < (uint64_t)a.tune.phased_min_bytes / 8 * 15) return false;
     const uint64_t grid = (uint64_t)(a.tune.num_cus / kPhaseGroups) * kPhaseGroups;
     return phases_full_enough(nvec, grid * kPhaseBlock * (uint64_t)(4 * reg_groups + kPhaseU), a.n);
 }
@@ -1311,7 +1316,7 @@ inline hipError_t launch_op(const LaunchArgs& a) {
     const VecSplit v = vector_split<E, TR::VEC>(a);
     if (wants_phased(a, v.nvec, phase_reg_groups(v.nvec, phase_lanes(a.tune), MultiPhaseRegs<TR>::groups, kPhaseU)))
         return launch_multi_op<TR, OP>(a);          // the phased kernel takes any number of inputs
-    // five or more inputs in the range between latency-bound and phased (64 to 240 MB of traffic): taking the inputs
+    // five or more inputs in the range between latency-bound and phased (64 to 315 MB of traffic): taking the inputs
     // one after the other, as the run-time-count streaming kernel does, measures 5-12 % above loading them together
     if (a.n >= 5 && a.tune.variant == 0 && (uint64_t)(a.n + 1) * v.nvec * 16u >= (uint64_t)a.tune.phased_min_bytes / 5 * 2)
         return launch_multi_op<TR, OP>(a);
